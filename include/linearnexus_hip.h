@@ -1,0 +1,126 @@
+/*
+ * C-ABI of the MI355X (gfx950) delta-rule scan library, liblinearnexus_hip.so.
+ *
+ * The reference (saran-gangster/linearnexus) is pure Python/JAX and has no native
+ * interface of its own; these entry points are what an XLA-FFI / ctypes binding for
+ * its layer ops would bind.  Every function returns 0 on success and a negative
+ * lnx_status otherwise; lnx_last_error() gives the thread-local message.  Nothing
+ * here allocates or frees device memory, synchronises the device, or keeps mutable
+ * global state: the caller owns all buffers (workspace included) and the stream.
+ *
+ * Tensor conventions (the reference's, linearnexus/modules/linear_attn/delta_net.py:126-134):
+ *   q, k  [B, H, T, dk]   v, o  [B, H, T, dv]   beta [B, H, T]   state [B, H, dk, dv] fp32
+ *   gate  g: none | [B, H, T] (Gated DeltaNet) | [B, H, T, dk] (KDA), fp32 log-decay <= 0
+ * All tensors are dense, last dimension contiguous.  q/k/v (and dO, dq, dk, dv) share
+ * one element type `dtype` (fp32 or bf16); beta, g, states and their gradients are fp32.
+ * With cu_seqlens != NULL the batch is packed: B must be 1, sequences are
+ * [cu[s], cu[s+1]) along T, states are [nseq, H, dk, dv] and reset at every boundary.
+ */
+#ifndef LINEARNEXUS_HIP_H
+#define LINEARNEXUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { LNX_F32 = 0, LNX_BF16 = 1 } lnx_dtype;
+typedef enum { LNX_GATE_NONE = 0, LNX_GATE_SCALAR = 1, LNX_GATE_VECTOR = 2 } lnx_gate;
+
+typedef enum {
+  LNX_OK = 0,
+  LNX_ERR_NULL = -1,        /* a required pointer is NULL */
+  LNX_ERR_SHAPE = -2,       /* unsupported or inconsistent dimensions */
+  LNX_ERR_DTYPE = -3,       /* unsupported element type */
+  LNX_ERR_WORKSPACE = -4,   /* workspace missing or too small */
+  LNX_ERR_LAUNCH = -5,      /* HIP reported a launch error */
+  LNX_ERR_DEVICE = -6       /* not a gfx950 device / no device */
+} lnx_status;
+
+/* One argument block for every entry point; fields an entry point does not use are ignored. */
+typedef struct lnx_scan_args {
+  int32_t B, H, T, dk, dv;
+  int32_t chunk;            /* chunk length; 64 is the only supported value (must be % 16 == 0) */
+  int32_t dtype;            /* lnx_dtype of q, k, v, dO, dq, dk, dv */
+  int32_t o_dtype;          /* lnx_dtype of o */
+  int32_t gate;             /* lnx_gate */
+  int32_t use_qk_l2norm;    /* normalise q, k rows as x / (|x|_2 + 1e-6) inside the op */
+  int32_t nseq;             /* number of packed sequences; 0 for a dense batch */
+  float scale;              /* multiplies q (after normalisation) */
+
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* beta;
+  const float* g;               /* NULL when gate == LNX_GATE_NONE */
+  const float* initial_state;   /* NULL = zeros */
+  const int32_t* cu_seqlens;    /* NULL for a dense batch; device pointer, nseq + 1 entries */
+  void* o;
+  float* final_state;           /* may alias initial_state for the decode step (in place) */
+
+  /* backward only */
+  const void* d_o;              /* [B,H,T,dv] in dtype */
+  const float* d_final_state;   /* NULL = zeros */
+  void* d_q;                    /* gradient outputs, same shapes/dtypes as q, k, v */
+  void* d_k;
+  void* d_v;
+  float* d_beta;
+  float* d_g;                   /* NULL when gate == LNX_GATE_NONE */
+  float* d_initial_state;       /* NULL = not wanted */
+
+  void* workspace;
+  uint64_t workspace_bytes;
+} lnx_scan_args;
+
+/* Library identification; also the symbol a loader probes first. */
+int lnx_abi_version(void);
+const char* lnx_last_error(void);
+
+/*
+ * Single-token decode step, state updated in place when final_state == initial_state.
+ * q,k [B,H,dk], v,o [B,H,dv], beta [B,H], g [B,H] or [B,H,dk]; T is ignored.
+ * Replaces delta_rule_step (delta_net.py:357-397), gated_delta_rule_step
+ * (gated_deltanet.py:539-597) and kda_step (kda.py:286-347).
+ */
+int lnx_decode_step(const lnx_scan_args* a, void* hip_stream);
+
+/*
+ * Token-by-token scan in fp32 with the state held in registers.
+ * Replaces delta_rule_recurrent (delta_net.py:126-213; also the Pallas kernel
+ * kernels/pallas/delta_rule.py:47-281), gated_delta_rule_recurrent
+ * (gated_deltanet.py:136-229) and kda_recurrent (kda.py:179-283).
+ */
+int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
+
+/*
+ * Chunked (WY) forward on MFMA.  Replaces delta_rule_chunkwise (delta_net.py:216-354),
+ * gated_delta_rule_chunkwise (gated_deltanet.py:232-534), kda_chunkwise (kda.py:350-655).
+ * The workspace keeps the per-chunk tensors the backward pass re-uses; pass the same
+ * workspace, unchanged, to lnx_chunk_bwd.
+ */
+uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
+int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);
+
+/*
+ * Chunked backward: gradients of <o, dO> + <final_state, d_final_state>.  The reference
+ * has no backward code (gradients come from JAX autodiff through lax.scan,
+ * linearnexus/train/sft.py:126-127); this entry point is what its jax.custom_vjp
+ * rule would call.  Needs the workspace filled by lnx_chunk_fwd on the same inputs.
+ */
+int lnx_chunk_bwd(const lnx_scan_args* a, void* hip_stream);
+
+/*
+ * Row-wise x / (|x|_2 + 1e-6) over the last dimension and its vector-Jacobian product,
+ * the normalisation the reference applies inside its ops when use_qk_l2norm is set
+ * (gated_deltanet.py:193-195, :273-275).  x, y, dy, dx: [rows, d] in `dtype`.
+ */
+int lnx_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t d, int32_t dtype, void* hip_stream);
+int lnx_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t d, int32_t dtype,
+                   void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LINEARNEXUS_HIP_H */

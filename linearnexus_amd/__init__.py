@@ -1,0 +1,25 @@
+"""MI355X-native delta-rule scan (DeltaNet / Gated DeltaNet / KDA) behind the reference's op names."""
+from .backend import KernelBackend, select_kernel_backend
+from .linear_attn import (
+    DeltaNetState,
+    GatedDeltaNetState,
+    KDAState,
+    delta_rule_chunkwise,
+    delta_rule_recurrent,
+    delta_rule_step,
+    gated_delta_rule_chunkwise,
+    gated_delta_rule_recurrent,
+    gated_delta_rule_step,
+    kda_chunkwise,
+    kda_recurrent,
+    kda_step,
+    l2norm_rows,
+)
+
+__all__ = [
+    "KernelBackend", "select_kernel_backend",
+    "DeltaNetState", "GatedDeltaNetState", "KDAState",
+    "delta_rule_recurrent", "delta_rule_chunkwise", "delta_rule_step",
+    "gated_delta_rule_recurrent", "gated_delta_rule_chunkwise", "gated_delta_rule_step",
+    "kda_recurrent", "kda_chunkwise", "kda_step", "l2norm_rows",
+]

@@ -1,0 +1,75 @@
+"""ctypes binding of liblinearnexus_hip.so (the C-ABI declared in include/linearnexus_hip.h).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liblinearnexus_hip.so")
+
+LNX_F32, LNX_BF16 = 0, 1
+GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
+
+EXPORTS = (
+    "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
+    "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
+)
+
+
+class ScanArgs(C.Structure):
+    """Mirror of ``struct lnx_scan_args``."""
+
+    _fields_ = [
+        ("B", C.c_int32), ("H", C.c_int32), ("T", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32),
+        ("chunk", C.c_int32), ("dtype", C.c_int32), ("o_dtype", C.c_int32), ("gate", C.c_int32),
+        ("use_qk_l2norm", C.c_int32), ("nseq", C.c_int32), ("scale", C.c_float),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("beta", C.c_void_p), ("g", C.c_void_p),
+        ("initial_state", C.c_void_p), ("cu_seqlens", C.c_void_p), ("o", C.c_void_p),
+        ("final_state", C.c_void_p),
+        ("d_o", C.c_void_p), ("d_final_state", C.c_void_p), ("d_q", C.c_void_p), ("d_k", C.c_void_p),
+        ("d_v", C.c_void_p), ("d_beta", C.c_void_p), ("d_g", C.c_void_p), ("d_initial_state", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
+    ]
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads the library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m linearnexus_amd.build` "
+            "(there is no CPU or PyTorch fallback for these ops)"
+        )
+    lib = C.CDLL(LIB_PATH)
+    lib.lnx_abi_version.restype = C.c_int
+    lib.lnx_last_error.restype = C.c_char_p
+    for name in ("lnx_decode_step", "lnx_recurrent_fwd", "lnx_chunk_fwd", "lnx_chunk_bwd"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.POINTER(ScanArgs), C.c_void_p]
+    lib.lnx_chunk_workspace_bytes.restype = C.c_uint64
+    lib.lnx_chunk_workspace_bytes.argtypes = [C.POINTER(ScanArgs)]
+    lib.lnx_l2norm_fwd.restype = C.c_int
+    lib.lnx_l2norm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lnx_l2norm_bwd.restype = C.c_int
+    lib.lnx_l2norm_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    _lib = lib
+    return lib
+
+
+class HipKernelError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().lnx_last_error().decode("utf-8", "replace")
+        raise HipKernelError(f"{what} failed (status {status}): {msg}")

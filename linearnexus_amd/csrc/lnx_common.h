@@ -1,0 +1,49 @@
+// Shared device helpers for the gfx950 delta-rule kernels: element types, conversions,
+// wavefront reductions and the error channel of the C-ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/linearnexus_hip.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define LNX_WAVE 64
+#define LNX_L2_EPS 1e-6f
+
+// Host side: records a message for lnx_last_error() and returns `code`.
+int lnx_set_error(int code, const char* fmt, ...);
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return (float)x; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
+
+// Loads 4 consecutive elements as fp32.
+__device__ __forceinline__ floatx4 load4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+__device__ __forceinline__ floatx4 load4(const bf16_t* p) {
+  bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+  floatx4 r = {(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+  return r;
+}
+__device__ __forceinline__ void store4(float* p, floatx4 x) { *reinterpret_cast<floatx4*>(p) = x; }
+__device__ __forceinline__ void store4(bf16_t* p, floatx4 x) {
+  bf16x4 t = {(bf16_t)x[0], (bf16_t)x[1], (bf16_t)x[2], (bf16_t)x[3]};
+  *reinterpret_cast<bf16x4*>(p) = t;
+}
+
+// Sum over all 64 lanes; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, LNX_WAVE);
+  return x;
+}

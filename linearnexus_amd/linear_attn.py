@@ -1,0 +1,341 @@
+"""Delta-rule layer ops on MI355X with the reference's signatures.
+
+The nine ops mirror ``linearnexus.modules.linear_attn`` (names, positional order, defaults,
+return conventions; linearnexus/modules/linear_attn/__init__.py:15-58): head-first
+``[B, H, T, d]`` tensors in, ``(output, final_state)`` out, fp32 state.  Tensors are
+``torch`` CUDA tensors (PyTorch only supplies device memory and the stream); every op
+launches hand-written gfx950 kernels through the C-ABI and raises if the library is
+missing -- there is no other code path.
+
+Differences from the reference, all additive: ``*_step`` take ``inplace=True`` to update
+the state buffer in place; the chunk ops take ``cu_seqlens`` for packed variable-length
+batches and are differentiable (``torch.autograd``) through the HIP backward kernels.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import GATE_NONE, GATE_SCALAR, GATE_VECTOR, LNX_BF16, LNX_F32, ScanArgs
+
+Tensor = torch.Tensor
+_DT = {torch.float32: LNX_F32, torch.bfloat16: LNX_BF16}
+CHUNK = 64  # the kernels' chunk length; results do not depend on it
+
+
+# --------------------------------------------------------------------------------------
+# helpers
+# --------------------------------------------------------------------------------------
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_inputs(q: Tensor, k: Tensor, v: Tensor) -> int:
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name} must be a torch.Tensor on an AMD GPU, got {type(t).__name__}")
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}; the delta-rule ops run on the GPU only")
+    if q.dtype not in _DT:
+        raise RuntimeError(f"unsupported dtype {q.dtype}: use float32 or bfloat16")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError(f"q, k, v must share one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+    if q.shape != k.shape or q.shape[:-1] != v.shape[:-1]:
+        raise RuntimeError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    return _DT[q.dtype]
+
+
+def _f32(t: Tensor) -> Tensor:
+    return t.to(torch.float32).contiguous()
+
+
+def _squeeze_beta(beta: Tensor, ndim: int) -> Tensor:
+    # delta_net.py:166-167, :257-258, :378-379 -- a trailing singleton is accepted
+    return beta.squeeze(-1) if beta.dim() == ndim else beta
+
+
+def _gate_kind(g: Optional[Tensor], lead_shape, dk: int) -> int:
+    if g is None:
+        return GATE_NONE
+    if tuple(g.shape) == tuple(lead_shape):
+        return GATE_SCALAR
+    if tuple(g.shape) == tuple(lead_shape) + (dk,):
+        return GATE_VECTOR
+    raise RuntimeError(f"gate shape {tuple(g.shape)} matches neither {tuple(lead_shape)} nor {tuple(lead_shape) + (dk,)}")
+
+
+def _base_args(B, H, T, dk, dv, dtype, o_dtype, gate, l2norm, scale) -> ScanArgs:
+    a = ScanArgs()
+    a.B, a.H, a.T, a.dk, a.dv = B, H, T, dk, dv
+    a.chunk = CHUNK
+    a.dtype, a.o_dtype, a.gate = dtype, o_dtype, gate
+    a.use_qk_l2norm = int(bool(l2norm))
+    a.nseq = 0
+    a.scale = float(scale)
+    return a
+
+
+# --------------------------------------------------------------------------------------
+# state caches (delta_net.py:81-118, gated_deltanet.py:72-128, kda.py:57-113)
+# --------------------------------------------------------------------------------------
+
+@dataclass
+class _ScanState:
+    S: Tensor
+    conv_state: Optional[Tensor] = None
+
+    @classmethod
+    def zeros(cls, batch_size, num_heads, key_dim, value_dim, conv_channels=None, conv_size=4, device="cuda"):
+        S = torch.zeros(batch_size, num_heads, key_dim, value_dim, dtype=torch.float32, device=device)
+        conv = None
+        if conv_channels is not None:
+            conv = torch.zeros(batch_size, conv_size - 1, conv_channels, dtype=torch.float32, device=device)
+        return cls(S=S, conv_state=conv)
+
+
+class DeltaNetState(_ScanState):
+    pass
+
+
+class GatedDeltaNetState(_ScanState):
+    pass
+
+
+class KDAState(_ScanState):
+    pass
+
+
+# --------------------------------------------------------------------------------------
+# single-token decode step
+# --------------------------------------------------------------------------------------
+
+def _step(q, k, v, g, beta, state, scale, l2norm, o_dtype_from_state, inplace):
+    dt = _check_inputs(q, k, v)
+    if q.dim() != 3:
+        raise RuntimeError(f"step ops take [B, H, d] vectors, got q {tuple(q.shape)}")
+    B, H, dk = q.shape
+    dv = v.shape[-1]
+    beta = _squeeze_beta(beta, 3)
+    gate = _gate_kind(g, (B, H), dk)
+    if tuple(state.shape) != (B, H, dk, dv):
+        raise RuntimeError(f"state shape {tuple(state.shape)} != {(B, H, dk, dv)}")
+    if scale is None:
+        scale = dk ** -0.5
+    if inplace:
+        if state.dtype != torch.float32 or not state.is_contiguous():
+            raise RuntimeError("inplace=True needs a contiguous float32 state")
+        s_in = s_out = state
+    else:
+        s_in = _f32(state)
+        s_out = torch.empty_like(s_in)
+    o_t = torch.float32 if o_dtype_from_state else q.dtype
+    o = torch.empty(B, H, dv, dtype=o_t, device=q.device)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    beta = _f32(beta)
+    g = None if g is None else _f32(g)
+    a = _base_args(B, H, 1, dk, dv, dt, _DT[o_t], gate, l2norm, scale)
+    a.q, a.k, a.v, a.beta, a.g = _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(g)
+    a.initial_state, a.final_state, a.o = _ptr(s_in), _ptr(s_out), _ptr(o)
+    lib = _lib.load()
+    _lib.check(lib.lnx_decode_step(a, _stream(q)), "lnx_decode_step")
+    return o, s_out
+
+
+def delta_rule_step(q, k, v, beta, state, scale=None, *, inplace=False) -> Tuple[Tensor, Tensor]:
+    """One decode token of plain DeltaNet (delta_net.py:357-397)."""
+    return _step(q, k, v, None, beta, state, scale, False, False, inplace)
+
+
+def gated_delta_rule_step(q, k, v, g, beta, state, scale=None, use_qk_l2norm=True, *, inplace=False):
+    """One decode token of Gated DeltaNet, ``g [B,H]`` (gated_deltanet.py:539-597)."""
+    return _step(q, k, v, g, beta, state, scale, use_qk_l2norm, False, inplace)
+
+
+def kda_step(q, k, v, g, beta, state, scale=None, use_qk_l2norm=True, *, inplace=False):
+    """One decode token of KDA, ``g [B,H,dk]``; output in the state's dtype (kda.py:286-347)."""
+    return _step(q, k, v, g, beta, state, scale, use_qk_l2norm, True, inplace)
+
+
+# --------------------------------------------------------------------------------------
+# token-by-token scan
+# --------------------------------------------------------------------------------------
+
+def _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens):
+    dt = _check_inputs(q, k, v)
+    if q.dim() != 4:
+        raise RuntimeError(f"scan ops take [B, H, T, d] tensors, got q {tuple(q.shape)}")
+    B, H, T, dk = q.shape
+    dv = v.shape[-1]
+    beta = _squeeze_beta(beta, 4)
+    if tuple(beta.shape) != (B, H, T):
+        raise RuntimeError(f"beta shape {tuple(beta.shape)} != {(B, H, T)}")
+    gate = _gate_kind(g, (B, H, T), dk)
+    nseq = 0
+    if cu_seqlens is not None:
+        if B != 1:
+            raise RuntimeError("cu_seqlens needs a packed batch with B == 1")
+        cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()
+        nseq = cu_seqlens.numel() - 1
+    nstate = nseq if nseq else B
+    if initial_state is not None and tuple(initial_state.shape) != (nstate, H, dk, dv):
+        raise RuntimeError(f"initial_state shape {tuple(initial_state.shape)} != {(nstate, H, dk, dv)}")
+    return dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu_seqlens
+
+
+def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):
+    dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
+    if scale is None:
+        scale = dk ** -0.5
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    beta = _f32(beta)
+    g = None if g is None else _f32(g)
+    s0 = None if initial_state is None else _f32(initial_state)
+    o = torch.empty(B, H, T, dv, dtype=q.dtype, device=q.device)
+    sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
+    a = _base_args(B, H, T, dk, dv, dt, dt, gate, l2norm, scale)
+    a.nseq = nseq
+    a.q, a.k, a.v, a.beta, a.g = _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(g)
+    a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
+    lib = _lib.load()
+    _lib.check(lib.lnx_recurrent_fwd(a, _stream(q)), "lnx_recurrent_fwd")
+    return o, sT
+
+
+def delta_rule_recurrent(q, k, v, beta, initial_state=None, scale=None, backend=None, *, cu_seqlens=None):
+    """Token-by-token DeltaNet scan in fp32 (delta_net.py:126-213)."""
+    return _recurrent(q, k, v, None, beta, scale, initial_state, False, cu_seqlens)
+
+
+def gated_delta_rule_recurrent(q, k, v, g, beta, scale=None, initial_state=None, use_qk_l2norm=True, *,
+                               cu_seqlens=None):
+    """Token-by-token Gated DeltaNet scan, ``g [B,H,T]`` (gated_deltanet.py:136-229)."""
+    return _recurrent(q, k, v, g, beta, scale, initial_state, use_qk_l2norm, cu_seqlens)
+
+
+def kda_recurrent(q, k, v, g, beta, scale=None, initial_state=None, use_qk_l2norm=True, *, cu_seqlens=None):
+    """Token-by-token KDA scan, ``g [B,H,T,dk]`` (kda.py:179-283)."""
+    return _recurrent(q, k, v, g, beta, scale, initial_state, use_qk_l2norm, cu_seqlens)
+
+
+# --------------------------------------------------------------------------------------
+# chunked scan (forward + backward)
+# --------------------------------------------------------------------------------------
+
+def l2norm_rows(x: Tensor) -> Tensor:
+    """``x / (|x|_2 + 1e-6)`` over the last dimension, in x's dtype (gated_deltanet.py:273-275)."""
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    d = x.shape[-1]
+    _lib.check(_lib.load().lnx_l2norm_fwd(_ptr(x), _ptr(y), x.numel() // d, d, _DT[x.dtype], _stream(x)), "lnx_l2norm_fwd")
+    return y
+
+
+def _l2norm_rows_bwd(x: Tensor, dy: Tensor) -> Tensor:
+    x, dy = x.contiguous(), dy.contiguous()
+    dx = torch.empty_like(x)
+    d = x.shape[-1]
+    _lib.check(_lib.load().lnx_l2norm_bwd(_ptr(x), _ptr(dy), _ptr(dx), x.numel() // d, d, _DT[x.dtype], _stream(x)),
+               "lnx_l2norm_bwd")
+    return dx
+
+
+class _ChunkScan(torch.autograd.Function):
+    """Pairs lnx_chunk_fwd with lnx_chunk_bwd (the role ``jax.custom_vjp`` plays for a JAX caller)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens):
+        dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
+        q_in, k_in = q.contiguous(), k.contiguous()
+        # the reference's chunk path normalises in the input dtype before anything else
+        # (gated_deltanet.py:273-275, kda.py:379-381)
+        qn = l2norm_rows(q_in) if l2norm else q_in
+        kn = l2norm_rows(k_in) if l2norm else k_in
+        v = v.contiguous()
+        beta_f = _f32(beta)
+        g_f = None if g is None else _f32(g)
+        s0 = None if initial_state is None else _f32(initial_state)
+        o = torch.empty(B, H, T, dv, dtype=o_dtype, device=q.device)
+        sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
+        a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
+        a.nseq = nseq
+        a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
+        a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
+        lib = _lib.load()
+        nbytes = int(lib.lnx_chunk_workspace_bytes(a))
+        if nbytes == 0 and T > 0 and B > 0:
+            _lib.check(-2, "lnx_chunk_workspace_bytes")
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = _ptr(ws), nbytes
+        _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
+        ctx.save_for_backward(q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
+        ctx.meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
+                    None if g is None else g.dtype, initial_state is not None)
+        return o, sT
+
+    @staticmethod
+    def backward(ctx, d_o, d_sT):
+        q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws = ctx.saved_tensors
+        dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0 = ctx.meta
+        dev = qn.device
+        d_o = torch.zeros(B, H, T, dv, dtype=qn.dtype, device=dev) if d_o is None else d_o.to(qn.dtype).contiguous()
+        d_sT = None if d_sT is None else _f32(d_sT)
+        dq, dk_, dv_ = torch.empty_like(qn), torch.empty_like(kn), torch.empty_like(v)
+        dbeta = torch.empty_like(beta_f)
+        dg = None if g_f is None else torch.empty_like(g_f)
+        nstate = nseq if nseq else B
+        ds0 = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=dev) if has_s0 else None
+        a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
+        a.nseq = nseq
+        a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
+        a.initial_state, a.cu_seqlens = _ptr(s0), _ptr(cu)
+        a.d_o, a.d_final_state = _ptr(d_o), _ptr(d_sT)
+        a.d_q, a.d_k, a.d_v, a.d_beta, a.d_g, a.d_initial_state = (_ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(dbeta),
+                                                                   _ptr(dg), _ptr(ds0))
+        a.workspace, a.workspace_bytes = _ptr(ws), ws.numel()
+        _lib.check(_lib.load().lnx_chunk_bwd(a, _stream(qn)), "lnx_chunk_bwd")
+        if l2norm:
+            dq = _l2norm_rows_bwd(q_in, dq)
+            dk_ = _l2norm_rows_bwd(k_in, dk_)
+        dbeta = dbeta.to(beta_dt)
+        if dg is not None:
+            dg = dg.to(g_dt)
+        return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None
+
+
+def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, need_mult16, cu_seqlens):
+    if need_mult16 and chunk_size % 16 != 0:
+        # gated_deltanet.py:318-320, kda.py:438-440
+        raise ValueError(f"chunk_size (BT={chunk_size}) must be divisible by BC=16.")
+    if chunk_size <= 0:
+        raise ValueError(f"chunk_size must be positive, got {chunk_size}")
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    return _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+
+
+def delta_rule_chunkwise(q, k, v, beta, initial_state=None, chunk_size=64, scale=None, backend=None, *,
+                         cu_seqlens=None):
+    """Chunked (WY) DeltaNet scan (delta_net.py:216-354).  ``chunk_size`` is validated and then
+    ignored: the kernels always use 64-token chunks, which the result does not depend on."""
+    return _chunk(q, k, v, None, beta, scale, initial_state, chunk_size, False, q.dtype, False, cu_seqlens)
+
+
+def gated_delta_rule_chunkwise(q, k, v, g, beta, scale=None, initial_state=None, chunk_size=64,
+                               use_qk_l2norm=True, *, cu_seqlens=None):
+    """Chunked Gated DeltaNet scan, ``g [B,H,T]`` (gated_deltanet.py:232-534)."""
+    return _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, use_qk_l2norm, q.dtype, True, cu_seqlens)
+
+
+def kda_chunkwise(q, k, v, g, beta, scale=None, initial_state=None, chunk_size=64, use_qk_l2norm=True, *,
+                  cu_seqlens=None, output_dtype=torch.float32):
+    """Chunked KDA scan, ``g [B,H,T,dk]`` (kda.py:350-655).  Like the reference, the output is
+    float32 whatever the input dtype (kda.py:416, :655); pass ``output_dtype`` to change that."""
+    return _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, use_qk_l2norm, output_dtype, True, cu_seqlens)

@@ -1,0 +1,91 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, validates arguments without touching a GPU, and the Python ops keep the reference's
+signatures and error types."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+
+import linearnexus_amd as la
+from linearnexus_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "linearnexus_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lnx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert set(names) >= set(_lib.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.lnx_abi_version() >= 1
+
+
+def test_struct_layout_matches_header():
+    # 12 four-byte scalars, then 17 pointers, then the workspace size
+    assert ctypes.sizeof(_lib.ScanArgs) == 48 + 18 * 8 + 8
+    assert _lib.ScanArgs.q.offset == 48
+
+
+def test_argument_validation_without_gpu():
+    lib = _lib.load()
+    a = _lib.ScanArgs()
+    assert lib.lnx_decode_step(a, None) == -1 and b"required" in lib.lnx_last_error()
+    assert lib.lnx_chunk_fwd(a, None) < 0
+    assert lib.lnx_chunk_bwd(a, None) < 0
+    assert lib.lnx_l2norm_fwd(None, None, 4, 8, 0, None) == -1
+
+
+SIGNATURES = {
+    # linearnexus/modules/linear_attn/delta_net.py:126-134, :216-225, :357-364
+    "delta_rule_recurrent": ["q", "k", "v", "beta", "initial_state", "scale", "backend"],
+    "delta_rule_chunkwise": ["q", "k", "v", "beta", "initial_state", "chunk_size", "scale", "backend"],
+    "delta_rule_step": ["q", "k", "v", "beta", "state", "scale"],
+    # gated_deltanet.py:136-145, :232-242, :539-548
+    "gated_delta_rule_recurrent": ["q", "k", "v", "g", "beta", "scale", "initial_state", "use_qk_l2norm"],
+    "gated_delta_rule_chunkwise": ["q", "k", "v", "g", "beta", "scale", "initial_state", "chunk_size", "use_qk_l2norm"],
+    "gated_delta_rule_step": ["q", "k", "v", "g", "beta", "state", "scale", "use_qk_l2norm"],
+    # kda.py:179-188, :350-360, :286-295
+    "kda_recurrent": ["q", "k", "v", "g", "beta", "scale", "initial_state", "use_qk_l2norm"],
+    "kda_chunkwise": ["q", "k", "v", "g", "beta", "scale", "initial_state", "chunk_size", "use_qk_l2norm"],
+    "kda_step": ["q", "k", "v", "g", "beta", "state", "scale", "use_qk_l2norm"],
+}
+
+
+@pytest.mark.parametrize("name", sorted(SIGNATURES))
+def test_op_signatures_match_reference(name):
+    sig = inspect.signature(getattr(la, name))
+    positional = [p.name for p in sig.parameters.values() if p.kind == p.POSITIONAL_OR_KEYWORD]
+    assert positional == SIGNATURES[name]
+    d = {p.name: p.default for p in sig.parameters.values()}
+    if "chunk_size" in d:
+        assert d["chunk_size"] == 64
+    if "use_qk_l2norm" in d:
+        assert d["use_qk_l2norm"] is True
+    assert d["scale"] is None
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    import torch
+    q = torch.randn(1, 1, 4, 8)
+    with pytest.raises(RuntimeError):
+        la.delta_rule_recurrent(q, q, q, torch.ones(1, 1, 4))
+
+
+def test_chunk_size_error_type():
+    import torch
+    q = torch.randn(1, 1, 4, 8)
+    with pytest.raises(ValueError):  # gated_deltanet.py:318-320
+        la.gated_delta_rule_chunkwise(q, q, q, torch.zeros(1, 1, 4), torch.ones(1, 1, 4), chunk_size=24)
+
+
+def test_backend_seam():
+    assert la.select_kernel_backend("pallas") is la.KernelBackend.HIP
