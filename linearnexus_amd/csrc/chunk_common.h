@@ -1,0 +1,92 @@
+// Geometry and workspace layout shared by the chunk forward and backward kernels.
+//
+// A "row" is one (batch, head) pair -- or one head of the packed batch; a row owns N chunk
+// slots of 64 tokens.  Dense batch: N = ceil(T / 64), slot n covers tokens [64 n, 64 n + 64).
+// Packed batch: chunks restart at every sequence boundary, so N = T / 64 + nseq slots are
+// reserved and a table built on the device maps slot -> (first token, length, sequence);
+// unused slots have length 0.
+//
+// Per-slot tensors kept in the workspace (element type T = bf16 or fp32 unless noted):
+//   G    fp32 [64] or [64][dk]   cumulative gate inside the chunk
+//   P    [64][64]   scale * <q_i, k_j> * exp(G_i - G_j), i >= j
+//   W    [64][dk]   (I + A)^-1 diag(beta) (K * exp(G))
+//   U    [64][dv]   (I + A)^-1 diag(beta) V
+//   KT   [dk][64]   K^T (scalar / no gate) or (K * exp(G_last - G))^T (vector gate)
+//   TmT  [64][64]   ((I + A)^-1)^T, used by the backward pass
+//   D    [64][dv]   U - W S            DT [dv][64] its transpose
+//   SnT  [dv][dk]   transpose of the state entering the chunk
+// Backward adds dOT [dv][64], dD [64][dv], dDT [dv][64], dSn [dk][dv] (gradient of the state
+// leaving the chunk) and dW [64][dk].
+#pragma once
+
+#include "mma_tiles.h"
+
+struct ChunkGeom {
+  int H, T, N, nseq, rows;       // rows = B * H (dense) or H (packed); N = chunk slots per row
+  const int32_t* cu;             // device cu_seqlens or nullptr
+  const int32_t* tab;            // packed only: [N][2] (token0, len) then seq_chunk0[nseq + 1]
+};
+
+__device__ __forceinline__ void chunk_span(const ChunkGeom& g, int n, int& tok0, int& len) {
+  if (g.tab) {
+    tok0 = g.tab[2 * n];
+    len = g.tab[2 * n + 1];
+  } else {
+    tok0 = n * LNX_C;
+    len = min(LNX_C, g.T - tok0);
+  }
+}
+
+// Chunk-slot range [c0, c1) of state index `s` (batch element or sequence).
+__device__ __forceinline__ void seq_chunks(const ChunkGeom& g, int s, int& c0, int& c1) {
+  if (g.tab) {
+    c0 = g.tab[2 * g.N + s];
+    c1 = g.tab[2 * g.N + s + 1];
+  } else {
+    c0 = 0;
+    c1 = g.N;
+  }
+}
+
+struct ChunkWs {
+  uint64_t tab, G, P, W, U, KT, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, total;
+};
+
+inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
+
+inline int lnx_chunk_slots(const lnx_scan_args* a) {
+  return a->cu_seqlens ? a->T / LNX_C + a->nseq : (a->T + LNX_C - 1) / LNX_C;
+}
+
+inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
+  ChunkWs w;
+  const uint64_t es = (a->dtype == LNX_BF16) ? 2 : 4;
+  const uint64_t rows = a->cu_seqlens ? (uint64_t)a->H : (uint64_t)a->B * a->H;
+  const uint64_t N = (uint64_t)lnx_chunk_slots(a);
+  const uint64_t slots = rows * N, dk = a->dk, dv = a->dv, C = LNX_C;
+  uint64_t off = 0;
+  auto take = [&](uint64_t bytes) { uint64_t o = off; off = lnx_align256(off + bytes); return o; };
+  w.tab = take(a->cu_seqlens ? (2 * N + a->nseq + 1) * 4 : 0);
+  w.G = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
+  w.P = take(slots * C * C * es);
+  w.W = take(slots * C * dk * es);
+  w.U = take(slots * C * dv * es);
+  w.KT = take(slots * dk * C * es);
+  w.TmT = take(slots * C * C * es);
+  w.D = take(slots * C * dv * es);
+  w.DT = take(slots * dv * C * es);
+  w.SnT = take(slots * dv * dk * es);
+  w.dOT = take(slots * dv * C * es);
+  w.dD = take(slots * C * dv * es);
+  w.dDT = take(slots * dv * C * es);
+  w.dSn = take(slots * dk * dv * es);
+  w.dW = take(slots * C * dk * es);
+  w.total = off;
+  return w;
+}
+
+// Shared argument validation of the chunk entry points; returns LNX_OK or an error status.
+int lnx_chunk_check(const lnx_scan_args* a, bool backward);
+
+// Builds the packed-batch chunk table (no-op for dense batches).
+void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st);

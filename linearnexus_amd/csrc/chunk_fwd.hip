@@ -1,5 +1,497 @@
-// placeholder until the MFMA chunk kernels land
-#include "lnx_common.h"
-extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) { (void)a; return 0; }
-extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* s) { (void)a; (void)s; return lnx_set_error(LNX_ERR_SHAPE, "chunk forward not built"); }
-extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* s) { (void)a; (void)s; return lnx_set_error(LNX_ERR_SHAPE, "chunk backward not built"); }
+// Chunked (WY) delta-rule forward on gfx950 MFMA, three kernels per call:
+//
+//   chunk_prepare  (one workgroup per 64-token chunk, all chunks in parallel)
+//       A = tril(diag(beta) K K^T * E, -1);  Tm = (I + A)^-1 (fp32, block forward substitution +
+//       MFMA block merges);  W = Tm diag(beta e^G) K;  U = Tm diag(beta) V;
+//       P = scale * tril(Q K^T * E);  also K^T and Tm^T for later kernels.
+//   chunk_scan     (one workgroup per (state, 64-column slab of dv), sequential over chunks)
+//       D = U - W S;  S <- e^{G_last} S + (K e^{G_last - G})^T D, with the fp32 state held in
+//       MFMA accumulators across the whole sequence; stores D, D^T and the entering state.
+//   chunk_output   (one workgroup per (chunk, 64-column slab), all in parallel)
+//       O = scale (Q e^G) S_n + P D.
+//
+// This is the algorithm of linearnexus/modules/linear_attn/gated_deltanet.py:444-523
+// (delta_net.py:296-330 without a gate, kda.py:569-648 with a vector gate); E_ij =
+// exp(G_i - G_j) with G the cumulative log-decay inside the chunk.
+
+#include "chunk_common.h"
+
+namespace {
+
+struct FwdParams {
+  ChunkGeom geom;
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* beta;
+  const float* g;
+  const float* s0;
+  float* sT_out;
+  void* o;
+  int dv, o_dtype;
+  float scale;
+  char* ws;
+  ChunkWs off;
+};
+
+template <typename T> __device__ __forceinline__ T* ws_ptr(const FwdParams& p, uint64_t off) {
+  return reinterpret_cast<T*>(p.ws + off);
+}
+
+// Inclusive prefix sum over the 64 lanes of a wavefront.
+__device__ __forceinline__ float wave_cumsum(float x, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const float y = __shfl_up(x, d, LNX_WAVE);
+    if (lane >= d) x += y;
+  }
+  return x;
+}
+
+// ---------------------------------------------------------------------------------------
+// chunk_prepare
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct PrepSmem {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD;      // row-major [64][DK] tiles
+  static constexpr int LDC = LNX_C + PAD;   // transposed [d][64] tiles and [64][64] tiles
+  static constexpr int kK = 64 * LDK;                       // sK, later sTw
+  static constexpr int kKT = DK * LDC;                      // sKT
+  static constexpr int kQ = (64 * LDK > 64 * LDC) ? 64 * LDK : 64 * LDC;  // sQ, later a V^T slab
+  static constexpr size_t bytes = sizeof(T) * (kK + kKT + kQ) + sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36 + 128);
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
+  typedef PrepSmem<T, DK> L;
+  constexpr int LDK = L::LDK, LDC = L::LDC;
+  extern __shared__ __align__(16) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);
+  T* sKT = sK + L::kK;
+  T* sQ = sKT + L::kKT;
+  float* sA = reinterpret_cast<float*>(sQ + L::kQ);
+  float* sT = sA + 64 * LNX_LDA;
+  float* sX = sT + 64 * LNX_LDA;
+  float* sBeta = sX + 32 * 36;
+  float* sG = sBeta + 64;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+
+  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
+  stage_rows_t<T>(sKT, LDC, kg, DK, 64, len, DK, tid, UnitScale());
+  stage_rows<T>(sQ, LDK, qg, DK, 64, len, DK, tid);
+  if (wave == 0) {
+    const bool ok = lane < len;
+    sBeta[lane] = ok ? p.beta[tbase + lane] : 0.f;
+    float gv = 0.f;
+    if (GATE == LNX_GATE_SCALAR && ok) gv = p.g[tbase + lane];
+    gv = wave_cumsum(gv, lane);
+    sG[lane] = gv;
+    ws_ptr<float>(p, p.off.G)[slot * 64 + lane] = gv;
+  }
+  __syncthreads();
+
+  // X = K K^T and Q K^T, one 32x32 tile per wave (the upper-right tile is all zero)
+  {
+    const int wi = wave >> 1, wj = wave & 1;
+    floatx16 ax[1][1], ap[1][1];
+    frag_zero(ax);
+    frag_zero(ap);
+    if (!(wi == 0 && wj == 1)) {
+      mma_nt<T, 1, 1>(ax, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+      mma_nt<T, 1, 1>(ap, sQ + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+    }
+    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * ax[0][0][e] : 0.f;
+      Pg[i * 64 + j] = from_f32<T>((i >= j) ? p.scale * dec * ap[0][0][e] : 0.f);
+    }
+  }
+  __syncthreads();
+  tri_inverse_64(sA, sT, sX, tid);
+
+  // Tw = Tm * diag(beta e^G) (into the sK region), Tu = Tm * diag(beta) (into the sA region),
+  // Tm^T to the workspace.
+  T* sTw = sK;
+  T* sTu = reinterpret_cast<T*>(sA);
+  {
+    T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
+    for (int idx = tid; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
+      TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
+    }
+    __syncthreads();  // everyone is done reading sA (inverse) and sK (products)
+    for (int idx = tid; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
+      const float t = sT[r * LNX_LDA + c];
+      const float bu = sBeta[c];
+      const float bw = (GATE == LNX_GATE_NONE) ? bu : bu * __expf(sG[c]);
+      sTu[r * LDC + c] = from_f32<T>(t * bu);
+      sTw[r * LDC + c] = from_f32<T>(t * bw);
+    }
+  }
+  __syncthreads();
+
+  const int wi = wave >> 1, wj = wave & 1;
+  // W = Tw K, 64 columns at a time
+  {
+    T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
+    for (int c0 = 0; c0 < DK; c0 += 64) {
+      floatx16 acc[1][1];
+      frag_zero(acc);
+      mma_nt<T, 1, 1>(acc, sTw + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
+      frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
+    }
+    // K^T for the scan kernel
+    unstage_rows<T>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, 64, tid);
+  }
+  // U = Tu V, one transposed 64-column slab of V at a time (slab overlays sQ)
+  {
+    T* sVT = sQ;
+    T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
+    for (int c0 = 0; c0 < p.dv; c0 += 64) {
+      __syncthreads();
+      stage_rows_t<T>(sVT, LDC, vg + c0, p.dv, 64, len, 64, tid, UnitScale());
+      __syncthreads();
+      floatx16 acc[1][1];
+      frag_zero(acc);
+      mma_nt<T, 1, 1>(acc, sTu + 32 * wi * LDC, LDC, sVT + 32 * wj * LDC, LDC, 64, lane);
+      frag_store<T, 1, 1>(acc, Ug + 32 * wi * p.dv + c0 + 32 * wj, p.dv, lane);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// chunk_scan
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct ScanSmem {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD;
+  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int BV = 64;
+  static constexpr int kW = 64 * LDK, kKT = DK * LDC, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
+  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 64;
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
+  typedef ScanSmem<T, DK> L;
+  typedef typename Vec16<T>::V V16;
+  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD;
+  constexpr int VN = Vec16<T>::N;
+  // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and both column tiles,
+  // DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
+  constexpr int NT = (DK == 128) ? 2 : 1;
+  extern __shared__ __align__(16) char smem[];
+  T* sW = reinterpret_cast<T*>(smem);
+  T* sKT = sW + L::kW;
+  T* sU = sKT + L::kKT;
+  T* sST = sU + L::kU;
+  T* sDT = sST + L::kST;
+  float* sG = reinterpret_cast<float*>(sDT + L::kDT);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int H = p.geom.H, N = p.geom.N;
+  const int sidx = blockIdx.x;  // state index
+  const int row = p.geom.tab ? sidx % H : sidx;
+  const int v0 = blockIdx.y * BV;
+  int c0, c1;
+  seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+  const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
+  const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
+
+  floatx16 S[1][NT];
+  frag_zero(S);
+  if (p.s0) {
+    const float* s0 = p.s0 + (int64_t)sidx * DK * p.dv + v0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        S[0][j][e] = s0[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
+  }
+
+  // register prefetch of the next chunk's tiles
+  constexpr int NW = 64 * DK / VN / 256, NK = DK * 64 / VN / 256, NU = 64 * BV / VN / 256;
+  V16 rW[NW], rK[NK], rU[NU];
+  float rG = 0.f;
+  auto fetch = [&](int n) {
+    const int64_t slot = (int64_t)row * N + n;
+    const T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
+    const T* Kg = ws_ptr<T>(p, p.off.KT) + slot * DK * 64;
+    const T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)(tid + 256 * i) * VN);
+#pragma unroll
+    for (int i = 0; i < NK; ++i) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)(tid + 256 * i) * VN);
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
+      rU[i] = *reinterpret_cast<const V16*>(Ug + (int64_t)r * p.dv + c);
+    }
+    if (GATE != LNX_GATE_NONE && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
+      *reinterpret_cast<V16*>(sW + r * LDK + c) = rW[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int idx = tid + 256 * i, r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
+      *reinterpret_cast<V16*>(sKT + r * LDC + c) = rK[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
+      *reinterpret_cast<V16*>(sU + r * LDU + c) = rU[i];
+    }
+    if (tid < 64) sG[tid] = rG;
+  };
+
+  if (c0 < c1) fetch(c0);
+  for (int n = c0; n < c1; ++n) {
+    const int64_t slot = (int64_t)row * N + n;
+    commit();
+    // entering state -> LDS (B operand of W S) and -> workspace, both transposed [dv][dk]
+    frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
+    frag_store_t<T, 1, NT>(S, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)(v0 + scol) * DK + srow, DK, lane);
+    __syncthreads();
+    if (n + 1 < c1) fetch(n + 1);
+
+    // D = U - W S  (one 32x32 tile per wave)
+    const int wi = wave >> 1, wj = wave & 1;
+    floatx16 d[1][1];
+    frag_zero(d);
+    mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+    const float gl = (GATE == LNX_GATE_NONE) ? 0.f : sG[63];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+      d[0][0][e] = to_f32(sU[r * LDU + c]) - d[0][0][e];
+    }
+    frag_store<T, 1, 1>(d, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj,
+                        p.dv, lane);
+    frag_store_t<T, 1, 1>(d, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)(v0 + 32 * wj) * 64 + 32 * wi, 64,
+                          lane);
+    if (GATE != LNX_GATE_NONE) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
+    }
+    frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
+    __syncthreads();
+
+    // S <- e^{G_last} S + K^T (D e^{G_last - G})
+    if (GATE != LNX_GATE_NONE) {
+      const float dec = __expf(gl);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[0][j][e] *= dec;
+    }
+    mma_nt<T, 1, NT>(S, sKT + srow * LDC, LDC, sDT + scol * LDC, LDC, 64, lane);
+    __syncthreads();
+  }
+
+  float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0;
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      out[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = S[0][j][e];
+}
+
+// ---------------------------------------------------------------------------------------
+// chunk_output
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct OutSmem {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD;
+  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int BV = 64;
+  static constexpr size_t bytes = sizeof(T) * (64 * LDK + BV * LDK + 64 * LDC + BV * LDC) + sizeof(float) * 64;
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
+  typedef OutSmem<T, DK> L;
+  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV;
+  extern __shared__ __align__(16) char smem[];
+  T* sQ = reinterpret_cast<T*>(smem);
+  T* sST = sQ + 64 * LDK;
+  T* sP = sST + BV * LDK;
+  T* sDT = sP + 64 * LDC;
+  float* sG = reinterpret_cast<float*>(sDT + BV * LDC);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  const int v0 = blockIdx.y * BV;
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+
+  stage_rows<T>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, 64, len, DK, tid);
+  stage_rows<T>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, BV, DK, tid);
+  stage_rows<T>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, 64, 64, tid);
+  stage_rows<T>(sDT, LDC, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, BV, BV, 64, tid);
+  if (tid < 64) sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
+  __syncthreads();
+
+  const int wi = wave >> 1, wj = wave & 1;
+  floatx16 acc[1][1];
+  frag_zero(acc);
+  mma_nt<T, 1, 1>(acc, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const float gm = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+    acc[0][0][e] *= gm;
+  }
+  mma_nt<T, 1, 1>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj * LDC, LDC, 64, lane);
+  const int64_t obase = (tbase + 32 * wi) * p.dv + v0 + 32 * wj;
+  if (p.o_dtype == LNX_BF16)
+    frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, p.dv, lane, len - 32 * wi);
+  else
+    frag_store<float, 1, 1>(acc, reinterpret_cast<float*>(p.o) + obase, p.dv, lane, len - 32 * wi);
+}
+
+// state-only path for T == 0: final = initial (or zeros)
+__global__ void copy_state_kernel(const float* src, float* dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src ? src[i] : 0.f;
+}
+
+// packed batches: slot table [N][2] = (token0, len) followed by seq_chunk0[nseq + 1]
+__global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* tab) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int c = 0;
+  for (int s = 0; s < nseq; ++s) {
+    tab[2 * N + s] = c;
+    for (int t = cu[s]; t < cu[s + 1] && c < N; t += LNX_C) {
+      tab[2 * c] = t;
+      tab[2 * c + 1] = min(LNX_C, cu[s + 1] - t);
+      ++c;
+    }
+  }
+  tab[2 * N + nseq] = c;
+  for (; c < N; ++c) {
+    tab[2 * c] = 0;
+    tab[2 * c + 1] = 0;
+  }
+}
+
+template <typename T, int DK, int GATE>
+int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
+  const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
+  auto k1 = chunk_prepare_kernel<T, DK, GATE>;
+  auto k2 = chunk_scan_kernel<T, DK, GATE>;
+  auto k3 = chunk_output_kernel<T, DK, GATE>;
+  const size_t b1 = PrepSmem<T, DK>::bytes, b2 = ScanSmem<T, DK>::bytes, b3 = OutSmem<T, DK>::bytes;
+  hipError_t e;
+  if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
+      (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
+      (e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b3)) != hipSuccess)
+    return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / 64)), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k3, dim3((unsigned)slots, (unsigned)(p.dv / 64)), dim3(256), b3, st, p);
+  return LNX_OK;
+}
+
+template <typename T, int DK>
+int launch_fwd_gate(int gate, const FwdParams& p, int nstate, hipStream_t st) {
+  switch (gate) {
+    case LNX_GATE_NONE: return launch_fwd<T, DK, LNX_GATE_NONE>(p, nstate, st);
+    case LNX_GATE_SCALAR: return launch_fwd<T, DK, LNX_GATE_SCALAR>(p, nstate, st);
+    default: return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels: gate kind %d is not supported yet", gate);
+  }
+}
+
+}  // namespace
+
+int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
+  if (!a) return lnx_set_error(LNX_ERR_NULL, "args is NULL");
+  if (!a->q || !a->k || !a->v || !a->beta) return lnx_set_error(LNX_ERR_NULL, "q, k, v and beta are required");
+  if (!backward && (!a->o || !a->final_state)) return lnx_set_error(LNX_ERR_NULL, "o and final_state are required");
+  if (backward && (!a->d_o || !a->d_q || !a->d_k || !a->d_v || !a->d_beta))
+    return lnx_set_error(LNX_ERR_NULL, "d_o, d_q, d_k, d_v and d_beta are required");
+  if (a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
+  if (backward && a->gate != LNX_GATE_NONE && !a->d_g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs d_g", a->gate);
+  if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
+  if (a->B < 0 || a->H <= 0 || a->T < 0) return lnx_set_error(LNX_ERR_SHAPE, "bad dimensions B=%d H=%d T=%d", a->B, a->H, a->T);
+  if (a->dk != 64 && a->dk != 128) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128}, got %d", a->dk);
+  if (a->dv <= 0 || a->dv % 64 != 0) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dv %% 64 == 0, got %d", a->dv);
+  if (a->chunk != LNX_C) return lnx_set_error(LNX_ERR_SHAPE, "chunk length must be %d, got %d", LNX_C, a->chunk);
+  if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
+  if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);
+  if (a->use_qk_l2norm) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take pre-normalised q, k (use lnx_l2norm_fwd)");
+  if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
+    return lnx_set_error(LNX_ERR_SHAPE, "packed batches need B == 1 and nseq > 0 (B=%d nseq=%d)", a->B, a->nseq);
+  return LNX_OK;
+}
+
+void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st) {
+  if (!a->cu_seqlens) return;
+  hipLaunchKernelGGL(build_table_kernel, dim3(1), dim3(64), 0, st, a->cu_seqlens, a->nseq, lnx_chunk_slots(a),
+                     reinterpret_cast<int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab));
+}
+
+extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
+  // only the geometry matters here; tensor pointers may still be unset
+  if (!a || a->H <= 0 || a->T < 0 || a->B < 0 || (a->dk != 64 && a->dk != 128) || a->dv <= 0 || a->dv % 64 != 0 ||
+      (a->cu_seqlens && a->nseq <= 0))
+    return 0;
+  return lnx_chunk_ws_layout(a).total;
+}
+
+extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
+  int rc = lnx_chunk_check(a, false);
+  if (rc != LNX_OK) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  const bool packed = a->cu_seqlens != nullptr;
+  const int nstate = packed ? a->nseq : a->B;
+  if (nstate == 0) return LNX_OK;
+  if (a->T == 0) {
+    const int64_t n = (int64_t)nstate * a->H * a->dk * a->dv;
+    hipLaunchKernelGGL(copy_state_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a->initial_state,
+                       a->final_state, n);
+    return LNX_OK;
+  }
+  const ChunkWs w = lnx_chunk_ws_layout(a);
+  if (!a->workspace || a->workspace_bytes < w.total)
+    return lnx_set_error(LNX_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)w.total,
+                         (unsigned long long)a->workspace_bytes);
+  lnx_chunk_build_table(a, w, st);
+  FwdParams p;
+  p.geom.H = a->H; p.geom.T = a->T; p.geom.N = lnx_chunk_slots(a); p.geom.nseq = a->nseq;
+  p.geom.rows = packed ? a->H : a->B * a->H;
+  p.geom.cu = a->cu_seqlens;
+  p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
+  p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.g = a->g; p.s0 = a->initial_state;
+  p.sT_out = a->final_state; p.o = a->o; p.dv = a->dv; p.o_dtype = a->o_dtype; p.scale = a->scale;
+  p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
+  if (a->dtype == LNX_BF16)
+    rc = (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+  else
+    rc = (a->dk == 128) ? launch_fwd_gate<float, 128>(a->gate, p, nstate, st) : launch_fwd_gate<float, 64>(a->gate, p, nstate, st);
+  if (rc != LNX_OK) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk forward launch: %s", hipGetErrorString(e));
+  return LNX_OK;
+}

@@ -1,0 +1,266 @@
+// MFMA tile primitives for gfx950 shared by the chunk kernels.
+//
+// All block-level products have the "NT" form C[M x N] += A[M x K] * B[N x K]^T with both
+// operands K-contiguous in LDS, which is the native operand layout of the 32x32 MFMA
+// instructions: lane = (row r = lane & 31, k-group kg = lane >> 5) holds VEC consecutive
+// k-elements of row r.  bf16 uses v_mfma_f32_32x32x16_bf16 (8 elements per lane), fp32 uses
+// four v_mfma_f32_32x32x2_f32 per 8-wide k-step (4 elements per lane).
+//
+// Accumulator fragment (floatx16) of one 32x32 tile: element e of lane l is
+//   row = 8 * (e / 4) + 4 * (l >> 5) + (e % 4),  col = l & 31.
+// Four consecutive e share a column and cover four consecutive rows, so a fragment can be
+// written transposed ([col][row]) with 4-element vector stores.
+#pragma once
+
+#include "lnx_common.h"
+
+#define LNX_C 64  // chunk length (tokens)
+
+template <typename T> struct Mma;
+
+template <> struct Mma<bf16_t> {
+  static constexpr int KS = 16;   // k per step
+  static constexpr int VEC = 8;   // elements per lane per step == elements per 16-byte vector
+  static constexpr int PAD = 8;   // LDS row padding (elements) = 16 bytes
+  typedef bf16x8 Frag;
+  typedef bf16x4 Quad;
+  static __device__ __forceinline__ Frag load(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+  static __device__ __forceinline__ void mma(floatx16& c, const Frag& a, const Frag& b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <> struct Mma<float> {
+  static constexpr int KS = 8;
+  static constexpr int VEC = 4;
+  static constexpr int PAD = 4;
+  typedef floatx4 Frag;
+  typedef floatx4 Quad;
+  static __device__ __forceinline__ Frag load(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+  static __device__ __forceinline__ void mma(floatx16& c, const Frag& a, const Frag& b) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+  }
+};
+
+template <int MT, int NT>
+__device__ __forceinline__ void frag_zero(floatx16 (&acc)[MT][NT]) {
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+}
+
+// acc[i][j] += A[32 i .. , :K] * B[32 j .. , :K]^T ; A, B point at this wave's first rows.
+template <typename T, int MT, int NT>
+__device__ __forceinline__ void mma_nt(floatx16 (&acc)[MT][NT], const T* A, int lda, const T* B, int ldb, int K,
+                                       int lane) {
+  typedef Mma<T> M;
+  const int r = lane & 31, ko = (lane >> 5) * M::VEC;
+  const T* ap = A + r * lda + ko;
+  const T* bp = B + r * ldb + ko;
+  for (int k0 = 0; k0 < K; k0 += M::KS) {
+    typename M::Frag a[MT], b[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) a[i] = M::load(ap + i * 32 * lda + k0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) b[j] = M::load(bp + j * 32 * ldb + k0);
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) M::mma(acc[i][j], a[i], b[j]);
+  }
+}
+
+__device__ __forceinline__ int frag_row(int e, int lane) { return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3); }
+__device__ __forceinline__ int frag_col(int lane) { return lane & 31; }
+
+// Calls f(row, col, value&) for every element of the fragments (rows/cols relative to the
+// wave's tile origin).
+template <int MT, int NT, typename F>
+__device__ __forceinline__ void frag_foreach(floatx16 (&acc)[MT][NT], int lane, F f) {
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) f(32 * i + frag_row(e, lane), 32 * j + frag_col(lane), acc[i][j][e]);
+}
+
+// dst[row][col] = acc (row-major tile with leading dimension ld); dst points at the tile origin.
+template <typename T, int MT, int NT>
+__device__ __forceinline__ void frag_store(const floatx16 (&acc)[MT][NT], T* dst, int64_t ld, int lane,
+                                           int row_limit = 1 << 30) {
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = 32 * i + frag_row(e, lane);
+        if (row < row_limit) dst[row * ld + 32 * j + frag_col(lane)] = from_f32<T>(acc[i][j][e]);
+      }
+}
+
+// dst[col][row] = acc: transposed store, four consecutive rows per vector.
+template <typename T, int MT, int NT>
+__device__ __forceinline__ void frag_store_t(const floatx16 (&acc)[MT][NT], T* dst, int64_t ld, int lane) {
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = 32 * i + 8 * q + 4 * (lane >> 5);
+        const int col = 32 * j + frag_col(lane);
+        floatx4 x = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        store4(dst + col * ld + row, x);
+      }
+}
+
+// ---------------------------------------------------------------------------------------
+// global <-> LDS staging of [rows x cols] tiles by a 256-thread block
+// ---------------------------------------------------------------------------------------
+
+template <typename T> struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  typedef typename Mma<T>::Frag V;
+};
+
+template <typename T>
+__device__ __forceinline__ typename Vec16<T>::V vec_zero() {
+  typename Vec16<T>::V z;
+#pragma unroll
+  for (int e = 0; e < Vec16<T>::N; ++e) z[e] = (T)0.f;
+  return z;
+}
+
+// dst[r][c] = src[r * stride + c] for r < rows (rows >= valid are zero-filled); cols % VEC == 0.
+template <typename T>
+__device__ __forceinline__ void stage_rows(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
+                                           int cols, int tid) {
+  constexpr int N = Vec16<T>::N;
+  const int vpr = cols / N;
+  for (int idx = tid; idx < rows * vpr; idx += 256) {
+    const int r = idx / vpr, c = (idx - r * vpr) * N;
+    typename Vec16<T>::V x = vec_zero<T>();
+    if (r < valid) x = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
+    *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = x;
+  }
+}
+
+// dst[c][r] = f(r) * src[r * stride + c]: transposed staging through 4-row x N-column register
+// micro-tiles (coalesced 16-byte global loads, 4-element LDS stores).  rows % 4 == 0.
+template <typename T, typename F>
+__device__ __forceinline__ void stage_rows_t(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
+                                             int cols, int tid, F row_scale) {
+  constexpr int N = Vec16<T>::N;
+  const int vpr = cols / N;
+  for (int idx = tid; idx < (rows / 4) * vpr; idx += 256) {
+    const int rg = idx / vpr, c = (idx - rg * vpr) * N;
+    typename Vec16<T>::V x[4];
+    float s[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * rg + i;
+      x[i] = vec_zero<T>();
+      if (r < valid) x[i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
+      s[i] = row_scale(r);
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      floatx4 y = {to_f32(x[0][e]) * s[0], to_f32(x[1][e]) * s[1], to_f32(x[2][e]) * s[2], to_f32(x[3][e]) * s[3]};
+      store4(dst + (c + e) * ld + 4 * rg, y);
+    }
+  }
+}
+
+struct UnitScale {
+  __device__ __forceinline__ float operator()(int) const { return 1.f; }
+};
+
+// Copies an LDS tile [rows][cols] (leading dimension ld) to global memory with 16-byte vectors.
+template <typename T>
+__device__ __forceinline__ void unstage_rows(T* dst, int64_t stride, const T* src, int ld, int rows, int cols, int tid) {
+  constexpr int N = Vec16<T>::N;
+  const int vpr = cols / N;
+  for (int idx = tid; idx < rows * vpr; idx += 256) {
+    const int r = idx / vpr, c = (idx - r * vpr) * N;
+    *reinterpret_cast<typename Vec16<T>::V*>(dst + r * stride + c) =
+        *reinterpret_cast<const typename Vec16<T>::V*>(src + r * ld + c);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// 16x16 fp32 products on v_mfma_f32_16x16x4_f32, operands row-major in LDS
+//   returns C[i][j] = sum_k A[i][k] * B[k][j];  fragment: c[e] is row 4*(lane>>4)+e, col lane&15
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ floatx4 mm16_f32(const float* A, int lda, const float* B, int ldb, int K, int lane) {
+  floatx4 c = {0.f, 0.f, 0.f, 0.f};
+  const int i = lane & 15, kq = lane >> 4;
+  for (int k0 = 0; k0 < K; k0 += 4) {
+    const float a = A[i * lda + k0 + kq];
+    const float b = B[(k0 + kq) * ldb + i];
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  return c;
+}
+
+__device__ __forceinline__ void mm16_store(float* dst, int ld, floatx4 c, int lane, float sign) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) dst[(4 * (lane >> 4) + e) * ld + (lane & 15)] = sign * c[e];
+}
+
+#define LNX_LDA 68  // leading dimension of the fp32 64x64 matrices in LDS
+
+// In-LDS inverse of the unit lower-triangular matrix I + A (A strictly lower, 64x64, fp32,
+// leading dimension LNX_LDA):  Tm = (I + A)^-1.  `sA` is read only; `sT` receives the full
+// matrix (upper triangle zero); `sX` is a [32][36] fp32 scratch.  Must be called by all 256
+// threads.  Diagonal 16x16 blocks by forward substitution, then two levels of block merges
+//   [[L0, 0], [B, L1]]^-1 = [[L0^-1, 0], [-L1^-1 B L0^-1, L1^-1]].
+__device__ __forceinline__ void tri_inverse_64(const float* sA, float* sT, float* sX, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) sT[idx] = 0.f;
+  __syncthreads();
+  if (lane < 16) {
+    const int r0 = 16 * wave, c = lane;
+    float d[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float s = (i == c) ? 1.f : 0.f;
+#pragma unroll
+      for (int m = 0; m < i; ++m) s -= sA[(r0 + i) * LNX_LDA + r0 + m] * d[m];
+      d[i] = s;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sT[(r0 + i) * LNX_LDA + r0 + c] = d[i];
+  }
+  __syncthreads();
+  // level 1: blocks (1,0) and (3,2) of the 16x16 grid, one per wave 0/1
+  float* sXw = sX + (wave & 1) * 16 * 36;
+  const int b = 32 * (wave & 1);  // super-block origin
+  if (wave < 2) {
+    floatx4 x = mm16_f32(sA + (b + 16) * LNX_LDA + b, LNX_LDA, sT + b * LNX_LDA + b, LNX_LDA, 16, lane);
+    mm16_store(sXw, 36, x, lane, 1.f);
+  }
+  __syncthreads();
+  if (wave < 2) {
+    floatx4 y = mm16_f32(sT + (b + 16) * LNX_LDA + b + 16, LNX_LDA, sXw, 36, 16, lane);
+    mm16_store(sT + (b + 16) * LNX_LDA + b, LNX_LDA, y, lane, -1.f);
+  }
+  __syncthreads();
+  // level 2: the 32x32 lower-left block, one 16x16 output per wave
+  const int bi = 16 * (wave >> 1), bj = 16 * (wave & 1);
+  {
+    floatx4 x = mm16_f32(sA + (32 + bi) * LNX_LDA, LNX_LDA, sT + bj, LNX_LDA, 32, lane);
+    mm16_store(sX + bi * 36 + bj, 36, x, lane, 1.f);
+  }
+  __syncthreads();
+  {
+    floatx4 y = mm16_f32(sT + (32 + bi) * LNX_LDA + 32, LNX_LDA, sX + bj, 36, 32, lane);
+    mm16_store(sT + (32 + bi) * LNX_LDA + bj, LNX_LDA, y, lane, -1.f);
+  }
+  __syncthreads();
+}
