@@ -1,8 +1,645 @@
-// placeholder until the backward kernels land
+// Chunked delta-rule backward on gfx950 MFMA.  Gradients of <o, dO> + <S_T, dS_T> with respect
+// to q, k, v, beta, g and S_0, from the tensors lnx_chunk_fwd left in the workspace.  The
+// reference has no backward code (its gradients come from JAX autodiff of the recurrent scan,
+// linearnexus/train/sft.py:126-127); this is the hand-derived adjoint of the chunk algorithm of
+// gated_deltanet.py:444-523.  Four kernels:
+//
+//   bwd_local  (chunk x dv-slab parallel)   dD_loc = P^T dO;  also stores dO^T
+//   bwd_scan   (sequential, reverse)        dD = dD_loc + (K r) dS;  dS <- e^{G_last} dS + (Q~ e^G)^T dO - W^T dD
+//   bwd_dqk    (chunk parallel)             dP, dq, the P/K^r parts of dk, dW = -dD S^T, gate terms
+//   bwd_wy     (chunk parallel)             through W = Tm B_w, U = Tm B_u and Tm = (I + A)^-1:
+//                                           dv, dbeta, the remaining parts of dk, dg (reverse cumsum)
+// with r_j = exp(G_last - G_j), G the cumulative log-decay inside the chunk.
+
 #include "chunk_common.h"
-extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* s) {
-  (void)s;
+
+namespace {
+
+struct BwdParams {
+  ChunkGeom geom;
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* beta;
+  const void* d_o;
+  const float* d_sT;
+  void* dq;
+  void* dk;
+  void* dv_out;
+  float* dbeta;
+  float* dg;
+  float* ds0;
+  int dv;
+  float scale;
+  char* ws;
+  ChunkWs off;
+};
+
+template <typename T> __device__ __forceinline__ T* wsp(const BwdParams& p, uint64_t off) {
+  return reinterpret_cast<T*>(p.ws + off);
+}
+
+// Tiling of a [64 x DK] product over four waves: DK=128 -> both row tiles, column tile = wave;
+// DK=64 -> one 32x32 tile per wave.
+template <int DK> struct RowTiles {
+  static constexpr int MT = (DK == 128) ? 2 : 1;
+  static __device__ __forceinline__ int row0(int wave) { return (DK == 128) ? 0 : 32 * (wave >> 1); }
+  static __device__ __forceinline__ int col0(int wave) { return (DK == 128) ? 32 * wave : 32 * (wave & 1); }
+};
+
+// acc_rows[row0 + r] += sum over this wave's columns of acc[r][c] * partner(r, c); the caller
+// zeroes `rows` and synchronises.  partner(row, col) gives the element to multiply with.
+template <int MT, typename F>
+__device__ __forceinline__ void frag_rowdot(const floatx16 (&acc)[MT][1], int row0, int col0, int lane, float* rows,
+                                            F partner) {
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = row0 + 32 * i + frag_row(e, lane), c = col0 + frag_col(lane);
+      float s = acc[i][0][e] * partner(r, c);
+#pragma unroll
+      for (int m = 1; m < 32; m <<= 1) s += __shfl_xor(s, m, LNX_WAVE);
+      if ((lane & 31) == 0) atomicAdd(&rows[r], s);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// bwd_local: dD_loc[j][v] = sum_i P[i][j] dO[i][v]; dO^T slab to the workspace
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
+  constexpr int LDC = LNX_C + Mma<T>::PAD;
+  __shared__ __align__(16) T sPT[64 * LDC];
+  __shared__ __align__(16) T sdOT[64 * LDC];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  const int v0 = blockIdx.y * 64;
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  stage_rows_t<T>(sPT, LDC, wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, 64, 64, tid, UnitScale());
+  stage_rows_t<T>(sdOT, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, 64, len, 64, tid, UnitScale());
+  __syncthreads();
+  unstage_rows<T>(wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdOT, LDC, 64, 64, tid);
+  const int wi = wave >> 1, wj = wave & 1;
+  floatx16 acc[1][1];
+  frag_zero(acc);
+  mma_nt<T, 1, 1>(acc, sPT + 32 * wi * LDC, LDC, sdOT + 32 * wj * LDC, LDC, 64, lane);
+  frag_store<T, 1, 1>(acc, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// bwd_scan
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct BScanCfg {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int BV = (sizeof(T) == 4 && DK == 128) ? 32 : 64;  // dv slab per workgroup
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDU = BV + PAD;
+  static constexpr int kK = 64 * LDK, kQT = DK * LDC, kWT = DK * LDC, kdOT = BV * LDC, kdDl = 64 * LDU,
+                       kdST = BV * LDK, kdDT = BV * LDC;
+  static constexpr size_t bytes = sizeof(T) * (kK + kQT + kWT + kdOT + kdDl + kdST + kdDT) + sizeof(float) * 64;
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
+  typedef BScanCfg<T, DK> L;
+  typedef typename Vec16<T>::V V16;
+  constexpr int LDK = L::LDK, LDC = L::LDC, LDU = L::LDU, BV = L::BV, VN = Vec16<T>::N;
+  constexpr int CT = BV / 32;                      // column tiles of the slab
+  constexpr int NT = (DK == 128) ? CT : 1;         // state tiles per wave (row tile = wave or wave & 1)
+  static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
+  extern __shared__ __align__(16) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);
+  T* sQT = sK + L::kK;
+  T* sWT = sQT + L::kQT;
+  T* sdOT = sWT + L::kWT;
+  T* sdDl = sdOT + L::kdOT;
+  T* sdST = sdDl + L::kdDl;
+  T* sdDT = sdST + L::kdST;
+  float* sG = reinterpret_cast<float*>(sdDT + L::kdDT);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int H = p.geom.H, N = p.geom.N;
+  const int sidx = blockIdx.x;
+  const int row = p.geom.tab ? sidx % H : sidx;
+  const int v0 = blockIdx.y * BV;
+  int c0, c1;
+  seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+  const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
+  const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
+  // tile of the [64 x BV] token-by-value products owned by this wave (none for CT == 1, wave >= 2)
+  const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
+  const bool has_tile = (CT == 2) || wave < 2;
+
+  floatx16 dS[1][NT];
+  frag_zero(dS);
+  if (p.d_sT) {
+    const float* src = p.d_sT + (int64_t)sidx * DK * p.dv + v0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        dS[0][j][e] = src[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
+  }
+
+  constexpr int NK = 64 * DK / VN / 256, NO = (BV * 64 / VN + 255) / 256;
+  V16 rK[NK], rQ[NK], rW[NK], rO[NO], rD[NO];  // K rows; (scale Q e^G)^T and W^T rows
+  float rG = 0.f;
+  auto fetch = [&](int n) {
+    const int64_t slot = (int64_t)row * N + n;
+    int tok0, len;
+    chunk_span(p.geom, n, tok0, len);
+    const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+    const T* Wg = wsp<T>(p, p.off.WT) + slot * DK * 64;
+    const T* Qg = wsp<T>(p, p.off.QgT) + slot * DK * 64;
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int idx = tid + 256 * i, r = idx / (DK / VN);
+      rK[i] = vec_zero<T>();
+      if (r < len) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
+      rQ[i] = *reinterpret_cast<const V16*>(Qg + (int64_t)idx * VN);
+      rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)idx * VN);
+    }
+    const T* Og = wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64;
+    const T* Dg = wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0;
+#pragma unroll
+    for (int i = 0; i < NO; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < BV * 64 / VN) {
+        rO[i] = *reinterpret_cast<const V16*>(Og + (int64_t)idx * VN);
+        const int r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
+        rD[i] = *reinterpret_cast<const V16*>(Dg + (int64_t)r * p.dv + c);
+      }
+    }
+    if (GATE != LNX_GATE_NONE && tid < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + tid];
+  };
+  auto commit = [&]() {
+    if (tid < 64) sG[tid] = rG;
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
+      *reinterpret_cast<V16*>(sK + r * LDK + c) = rK[i];
+      const int rt = idx / (64 / VN), ct = (idx % (64 / VN)) * VN;
+      *reinterpret_cast<V16*>(sQT + rt * LDC + ct) = rQ[i];
+      *reinterpret_cast<V16*>(sWT + rt * LDC + ct) = rW[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NO; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < BV * 64 / VN) {
+        const int r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
+        *reinterpret_cast<V16*>(sdOT + r * LDC + c) = rO[i];
+        const int r2 = idx / (BV / VN), c2 = (idx % (BV / VN)) * VN;
+        *reinterpret_cast<V16*>(sdDl + r2 * LDU + c2) = rD[i];
+      }
+    }
+  };
+
+  if (c0 < c1) fetch(c1 - 1);
+  for (int n = c1 - 1; n >= c0; --n) {
+    const int64_t slot = (int64_t)row * N + n;
+    commit();
+    // dS (gradient of the state leaving chunk n) -> LDS transposed, and -> workspace row-major
+    frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
+    frag_store<T, 1, NT>(dS, wsp<T>(p, p.off.dSn) + slot * DK * p.dv + (int64_t)srow * p.dv + v0 + scol, p.dv, lane);
+    __syncthreads();
+    if (n > c0) fetch(n - 1);
+
+    const float gl = (GATE == LNX_GATE_NONE) ? 0.f : sG[63];
+    // dD = dD_loc + r_j (K dS)_j
+    if (has_tile) {
+      floatx16 d[1][1];
+      frag_zero(d);
+      mma_nt<T, 1, 1>(d, sK + 32 * wi * LDK, LDK, sdST + 32 * wj * LDK, LDK, DK, lane);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+        const float rj = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
+        d[0][0][e] = to_f32(sdDl[r * LDU + c]) + rj * d[0][0][e];
+      }
+      frag_store<T, 1, 1>(d, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
+      frag_store_t<T, 1, 1>(d, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)(v0 + 32 * wj) * 64 + 32 * wi, 64, lane);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) d[0][0][e] = -d[0][0][e];
+      frag_store_t<T, 1, 1>(d, sdDT + 32 * wj * LDC + 32 * wi, LDC, lane);
+    }
+    __syncthreads();
+
+    // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD
+    if (GATE != LNX_GATE_NONE) {
+      const float dec = __expf(gl);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dS[0][j][e] *= dec;
+    }
+    mma_nt<T, 1, NT>(dS, sQT + srow * LDC, LDC, sdOT + scol * LDC, LDC, 64, lane);
+    mma_nt<T, 1, NT>(dS, sWT + srow * LDC, LDC, sdDT + scol * LDC, LDC, 64, lane);
+    __syncthreads();
+  }
+  if (p.ds0) {
+    float* out = p.ds0 + (int64_t)sidx * DK * p.dv + v0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        out[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = dS[0][j][e];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// bwd_dqk
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct DqkCfg {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD;
+  // loop phase: dO, D, dD slabs [64][LDC] and S_n, dS_n slabs [DK][LDC]
+  // epilogue:   dPe, dPe^T [64][LDC] and K^T, Q^T [DK][LDC]   (same footprint minus one tile)
+  static constexpr int kTile = 64 * LDC, kWide = DK * LDC;
+  static constexpr size_t bytes = sizeof(T) * (3 * kTile + 2 * kWide) + sizeof(float) * (64 * LNX_LDA + 64 * 4);
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
+  typedef DqkCfg<T, DK> L;
+  typedef RowTiles<DK> RTl;
+  constexpr int LDC = L::LDC, MT = RTl::MT;
+  extern __shared__ __align__(16) char smem[];
+  T* sdO = reinterpret_cast<T*>(smem);
+  T* sD = sdO + L::kTile;
+  T* sdD = sD + L::kTile;
+  T* sSn = sdD + L::kTile;
+  T* sdSn = sSn + L::kWide;
+  float* sR = reinterpret_cast<float*>(sdSn + L::kWide);  // [64][LNX_LDA]
+  float* sG = sR + 64 * LNX_LDA;
+  float* sdG = sG + 64;     // per-row gate-gradient accumulator
+  float* sTj = sdG + 64;    // r_j <dKr_j, k_j>
+  float* sMisc = sTj + 64;  // [0] = <dS_n, S_n>
+  // epilogue overlays
+  T* sPe = sdO;
+  T* sPeT = sD;
+  T* sKT = sSn;
+  T* sQT = sdSn;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const int wi = wave >> 1, wj = wave & 1;
+  const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
+
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : wsp<float>(p, p.off.G)[slot * 64 + tid];
+    sdG[tid] = 0.f;
+    sTj[tid] = 0.f;
+    if (tid == 0) sMisc[0] = 0.f;
+  }
+
+  floatx16 aP[1][1], aQ[MT][1], aW[MT][1], aK[MT][1];
+  frag_zero(aP);
+  frag_zero(aQ);
+  frag_zero(aW);
+  frag_zero(aK);
+  float ss = 0.f;  // partial <dS_n, S_n>
+  for (int v0 = 0; v0 < p.dv; v0 += 64) {
+    __syncthreads();
+    stage_rows<T>(sdO, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, 64, len, 64, tid);
+    stage_rows<T>(sD, LDC, wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
+    stage_rows<T>(sdD, LDC, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
+    stage_rows_t<T>(sSn, LDC, wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, 64, 64, DK, tid, UnitScale());
+    stage_rows<T>(sdSn, LDC, wsp<T>(p, p.off.dSn) + slot * DK * p.dv + v0, p.dv, DK, DK, 64, tid);
+    __syncthreads();
+    mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDC, LDC, sD + 32 * wj * LDC, LDC, 64, lane);
+    mma_nt<T, MT, 1>(aQ, sdO + r0 * LDC, LDC, sSn + c0 * LDC, LDC, 64, lane);
+    mma_nt<T, MT, 1>(aW, sdD + r0 * LDC, LDC, sSn + c0 * LDC, LDC, 64, lane);
+    mma_nt<T, MT, 1>(aK, sD + r0 * LDC, LDC, sdSn + c0 * LDC, LDC, 64, lane);
+    if (GATE != LNX_GATE_NONE)
+      for (int idx = tid; idx < DK * 64; idx += 256) {
+        const int r = idx >> 6, c = idx & 63;
+        ss += to_f32(sSn[r * LDC + c]) * to_f32(sdSn[r * LDC + c]);
+      }
+  }
+  if (GATE != LNX_GATE_NONE) {
+    ss = wave_sum(ss);
+    if (lane == 0) atomicAdd(&sMisc[0], ss);
+  }
+  __syncthreads();  // slabs are dead from here on; sG, sdG initialised
+
+  // dW = -dD S_n^T to the workspace
+  {
+    floatx16 t[MT][1];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) t[i][0][e] = -aW[i][0][e];
+    frag_store<T, MT, 1>(t, wsp<T>(p, p.off.dW) + slot * 64 * DK + (int64_t)r0 * DK + c0, DK, lane);
+  }
+  // dP -> dPe = scale E dP (both orientations) and R = dP * P for the gate gradient
+  {
+    const T* Pg = wsp<T>(p, p.off.P) + slot * 64 * 64;
+    floatx16 pe[1][1];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      const float dp = (i >= j) ? aP[0][0][e] : 0.f;
+      pe[0][0][e] = p.scale * dec * dp;
+      if (GATE != LNX_GATE_NONE) sR[i * LNX_LDA + j] = dp * to_f32(Pg[i * 64 + j]);
+    }
+    frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+  }
+  // inter-chunk parts: dq = scale e^{G_i} dQg,  dk = r_j dKr, and their gate terms
+  const float gl = sG[63];
+  if (GATE != LNX_GATE_NONE) {
+    frag_rowdot<MT>(aQ, r0, c0, lane, sdG, [&](int r, int c) {
+      return (r < len) ? p.scale * __expf(sG[r]) * to_f32(qg[(int64_t)r * DK + c]) : 0.f;
+    });
+    frag_rowdot<MT>(aK, r0, c0, lane, sTj, [&](int r, int c) {
+      return (r < len) ? __expf(fminf(gl - sG[r], 0.f)) * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
+    });
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = r0 + 32 * i + frag_row(e, lane);
+      const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
+      const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
+      aQ[i][0][e] *= gq;
+      aK[i][0][e] *= gk;
+    }
+  stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
+  stage_rows_t<T>(sQT, LDC, qg, DK, 64, len, DK, tid, UnitScale());
+  __syncthreads();
+  // intra-chunk parts: dq += dPe K,  dk += dPe^T Q
+  mma_nt<T, MT, 1>(aQ, sPe + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
+  mma_nt<T, MT, 1>(aK, sPeT + r0 * LDC, LDC, sQT + c0 * LDC, LDC, 64, lane);
+  frag_store<T, MT, 1>(aQ, reinterpret_cast<T*>(p.dq) + (tbase + r0) * DK + c0, DK, lane, len - r0);
+  frag_store<T, MT, 1>(aK, reinterpret_cast<T*>(p.dk) + (tbase + r0) * DK + c0, DK, lane, len - r0);
+  // partial gate gradient wrt the cumulative gate G (row t); the chunk-end terms go to row 63
+  if (GATE != LNX_GATE_NONE && tid < 64) {
+    float rs = 0.f, cs = 0.f, tot = 0.f;
+    for (int j = 0; j < 64; ++j) {
+      rs += sR[tid * LNX_LDA + j];
+      cs += sR[j * LNX_LDA + tid];
+      tot += sTj[j];
+    }
+    float d = sdG[tid] + rs - cs - sTj[tid];
+    if (tid == 63) d += tot + __expf(gl) * sMisc[0];
+    wsp<float>(p, p.off.dG)[slot * 64 + tid] = d;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// bwd_wy
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct WyCfg {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD;
+  static constexpr int kR1 = 64 * LDC;                                   // Tm^T, later Y
+  static constexpr int kR2 = (128 * LDC > 64 * LDK) ? 128 * LDC : 64 * LDK;  // dW^T | dD^T + dBu | dBw | K^T
+  static constexpr int kR3 = 64 * LDK;                                   // U slab | W | K
+  static constexpr size_t bytes = sizeof(T) * (kR1 + kR2 + kR3) + sizeof(float) * (64 * LNX_LDA + 64 * 4);
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
+  typedef WyCfg<T, DK> L;
+  typedef RowTiles<DK> RTl;
+  constexpr int LDK = L::LDK, LDC = L::LDC, MT = RTl::MT;
+  extern __shared__ __align__(16) char smem[];
+  T* R1 = reinterpret_cast<T*>(smem);
+  T* R2 = R1 + L::kR1;
+  T* R3 = R2 + L::kR2;
+  float* sR = reinterpret_cast<float*>(R3 + L::kR3);  // [64][LNX_LDA]: dA * X
+  float* sG = sR + 64 * LNX_LDA;
+  float* sBeta = sG + 64;
+  float* sdB = sBeta + 64;  // dbeta accumulator
+  float* sdG = sdB + 64;    // gate-gradient accumulator (wrt cumulative G)
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+  const int wi = wave >> 1, wj = wave & 1;
+  const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
+
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : wsp<float>(p, p.off.G)[slot * 64 + tid];
+    sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+    sdB[tid] = 0.f;
+    sdG[tid] = 0.f;
+  }
+  // phase 1: dBw = Tm^T dW
+  T* sTmT = R1;
+  T* sdWT = R2;
+  stage_rows<T>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, 64, 64, tid);
+  stage_rows_t<T>(sdWT, LDC, wsp<T>(p, p.off.dW) + slot * 64 * DK, DK, 64, 64, DK, tid, UnitScale());
+  __syncthreads();
+  floatx16 aBw[MT][1], aM[1][1];
+  frag_zero(aBw);
+  frag_zero(aM);
+  mma_nt<T, MT, 1>(aBw, sTmT + r0 * LDC, LDC, sdWT + c0 * LDC, LDC, 64, lane);
+
+  // phase 2: per dv slab, dBu = Tm^T dD;  dv = beta dBu;  dbeta += <dBu, v>;  dM += dBu U^T
+  T* sdDT = R2;
+  T* sdBu = R2 + 64 * LDC;
+  T* sU = R3;
+  for (int v0 = 0; v0 < p.dv; v0 += 64) {
+    __syncthreads();
+    stage_rows<T>(sdDT, LDC, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, 64, 64, tid);
+    stage_rows<T>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
+    __syncthreads();
+    floatx16 bu[1][1];
+    frag_zero(bu);
+    mma_nt<T, 1, 1>(bu, sTmT + 32 * wi * LDC, LDC, sdDT + 32 * wj * LDC, LDC, 64, lane);
+    frag_store<T, 1, 1>(bu, sdBu + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_rowdot<1>(bu, 32 * wi, 32 * wj, lane, sdB, [&](int r, int c) {
+      return (r < len) ? to_f32(vg[(int64_t)r * p.dv + v0 + c]) : 0.f;
+    });
+#pragma unroll
+    for (int e = 0; e < 16; ++e) bu[0][0][e] *= sBeta[32 * wi + frag_row(e, lane)];
+    frag_store<T, 1, 1>(bu, reinterpret_cast<T*>(p.dv_out) + (tbase + 32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane,
+                        len - 32 * wi);
+    __syncthreads();
+    mma_nt<T, 1, 1>(aM, sdBu + 32 * wi * LDC, LDC, sU + 32 * wj * LDC, LDC, 64, lane);
+  }
+  __syncthreads();
+
+  // phase 3: dM += dBw W^T
+  T* sdBw = R2;
+  T* sW = R3;
+  frag_store<T, MT, 1>(aBw, sdBw + r0 * LDK + c0, LDK, lane);
+  stage_rows<T>(sW, LDK, wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, 64, DK, tid);
+  __syncthreads();
+  mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
+  __syncthreads();
+
+  // phase 4: X = K K^T (recomputed), dA = -tril(dM, -1), Y = sym(beta dA E), R = dA * E X
+  T* sK = R3;
+  T* sY = R1;
+  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
+  __syncthreads();
+  {
+    floatx16 x[1][1];
+    frag_zero(x);
+    if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(x, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      const float da = (i > j) ? -aM[0][0][e] : 0.f;
+      sR[i * LNX_LDA + j] = da * dec * x[0][0][e];
+      const T y = from_f32<T>(sBeta[i] * da * dec);
+      if (i > j) {
+        sY[i * LDC + j] = y;
+        sY[j * LDC + i] = y;
+      } else if (i == j) {
+        sY[i * LDC + j] = from_f32<T>(0.f);
+      }
+    }
+  }
+  // dk (row-type part through B_w): beta e^{G} dBw, with its dbeta / gate terms
+  frag_rowdot<MT>(aBw, r0, c0, lane, sdG, [&](int r, int c) {
+    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
+    return (r < len) ? gm * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
+  });
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = r0 + 32 * i + frag_row(e, lane);
+      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
+      aBw[i][0][e] *= sBeta[r] * gm;
+    }
+  __syncthreads();  // sdBw (R2) no longer read; sY, sR complete
+
+  // phase 5: dk += Y K, added to the partial dk of bwd_dqk
+  T* sKT = R2;
+  stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
+  __syncthreads();
+  mma_nt<T, MT, 1>(aBw, sY + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
+  {
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
+        if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + aBw[i][0][e]);
+      }
+  }
+  // dbeta and dg
+  if (wave == 0) {
+    const int t = lane;
+    float rs = 0.f, cs = 0.f;
+    for (int j = 0; j < 64; ++j) {
+      rs += sR[t * LNX_LDA + j];
+      cs += sBeta[j] * sR[j * LNX_LDA + t];
+    }
+    // sdG[t] holds e^{G_t} <dBw_t, k_t>
+    const float w = sdG[t];
+    if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
+    if (GATE != LNX_GATE_NONE) {
+      float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - cs;
+      // reverse inclusive cumsum over the chunk
+#pragma unroll
+      for (int s = 1; s < 64; s <<= 1) {
+        const float y = __shfl_down(d, s, LNX_WAVE);
+        if (t + s < 64) d += y;
+      }
+      if (t < len) p.dg[tbase + t] = d;
+    }
+  }
+}
+
+template <typename T, int DK, int GATE>
+int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
+  const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
+  auto k1 = bwd_scan_kernel<T, DK, GATE>;
+  auto k2 = bwd_dqk_kernel<T, DK, GATE>;
+  auto k3 = bwd_wy_kernel<T, DK, GATE>;
+  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK>::bytes, b3 = WyCfg<T, DK>::bytes;
+  hipError_t e;
+  if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
+      (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
+      (e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b3)) != hipSuccess)
+    return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(bwd_local_kernel<T>, dim3((unsigned)slots, (unsigned)(p.dv / 64)), dim3(256), 0, st, p);
+  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(256), b1, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)slots), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k3, dim3((unsigned)slots), dim3(256), b3, st, p);
+  return LNX_OK;
+}
+
+template <typename T, int DK>
+int launch_bwd_gate(int gate, const BwdParams& p, int nstate, hipStream_t st) {
+  switch (gate) {
+    case LNX_GATE_NONE: return launch_bwd<T, DK, LNX_GATE_NONE>(p, nstate, st);
+    case LNX_GATE_SCALAR: return launch_bwd<T, DK, LNX_GATE_SCALAR>(p, nstate, st);
+    default: return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels: gate kind %d is not supported yet", gate);
+  }
+}
+
+__global__ void copy_dstate_kernel(const float* src, float* dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src ? src[i] : 0.f;
+}
+
+}  // namespace
+
+extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   int rc = lnx_chunk_check(a, true);
   if (rc != LNX_OK) return rc;
-  return lnx_set_error(LNX_ERR_SHAPE, "chunk backward not built");
+  hipStream_t st = (hipStream_t)stream;
+  const bool packed = a->cu_seqlens != nullptr;
+  const int nstate = packed ? a->nseq : a->B;
+  if (nstate == 0) return LNX_OK;
+  if (a->T == 0) {
+    if (a->d_initial_state) {
+      const int64_t n = (int64_t)nstate * a->H * a->dk * a->dv;
+      hipLaunchKernelGGL(copy_dstate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a->d_final_state,
+                         a->d_initial_state, n);
+    }
+    return LNX_OK;
+  }
+  const ChunkWs w = lnx_chunk_ws_layout(a);
+  if (!a->workspace || a->workspace_bytes < w.total)
+    return lnx_set_error(LNX_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)w.total,
+                         (unsigned long long)a->workspace_bytes);
+  BwdParams p;
+  p.geom.H = a->H; p.geom.T = a->T; p.geom.N = lnx_chunk_slots(a); p.geom.nseq = a->nseq;
+  p.geom.rows = packed ? a->H : a->B * a->H;
+  p.geom.cu = a->cu_seqlens;
+  p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
+  p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.d_o = a->d_o; p.d_sT = a->d_final_state;
+  p.dq = a->d_q; p.dk = a->d_k; p.dv_out = a->d_v; p.dbeta = a->d_beta; p.dg = a->d_g; p.ds0 = a->d_initial_state;
+  p.dv = a->dv; p.scale = a->scale;
+  p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
+  if (a->dtype == LNX_BF16)
+    rc = (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+  else
+    rc = (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st) : launch_bwd_gate<float, 64>(a->gate, p, nstate, st);
+  if (rc != LNX_OK) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk backward launch: %s", hipGetErrorString(e));
+  return LNX_OK;
 }

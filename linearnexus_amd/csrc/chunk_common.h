@@ -12,11 +12,12 @@
 //   W    [64][dk]   (I + A)^-1 diag(beta) (K * exp(G))
 //   U    [64][dv]   (I + A)^-1 diag(beta) V
 //   KT   [dk][64]   K^T (scalar / no gate) or (K * exp(G_last - G))^T (vector gate)
+//   WT   [dk][64]   W^T            QgT [dk][64]  (scale * Q * exp(G))^T
 //   TmT  [64][64]   ((I + A)^-1)^T, used by the backward pass
 //   D    [64][dv]   U - W S            DT [dv][64] its transpose
 //   SnT  [dv][dk]   transpose of the state entering the chunk
 // Backward adds dOT [dv][64], dD [64][dv], dDT [dv][64], dSn [dk][dv] (gradient of the state
-// leaving the chunk) and dW [64][dk].
+// leaving the chunk), dW [64][dk] and dG (fp32 partial gradient of the cumulative gate).
 #pragma once
 
 #include "mma_tiles.h"
@@ -49,7 +50,7 @@ __device__ __forceinline__ void seq_chunks(const ChunkGeom& g, int s, int& c0, i
 }
 
 struct ChunkWs {
-  uint64_t tab, G, P, W, U, KT, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, total;
+  uint64_t tab, G, P, W, WT, QgT, U, KT, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, dG, total;
 };
 
 inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
@@ -70,6 +71,8 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.G = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
   w.W = take(slots * C * dk * es);
+  w.WT = take(slots * dk * C * es);
+  w.QgT = take(slots * dk * C * es);
   w.U = take(slots * C * dv * es);
   w.KT = take(slots * dk * C * es);
   w.TmT = take(slots * C * C * es);
@@ -81,6 +84,7 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.dDT = take(slots * dv * C * es);
   w.dSn = take(slots * dk * dv * es);
   w.dW = take(slots * C * dk * es);
+  w.dG = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
   w.total = off;
   return w;
 }

@@ -57,7 +57,7 @@ template <typename T, int DK> struct PrepSmem {
   static constexpr int LDC = LNX_C + PAD;   // transposed [d][64] tiles and [64][64] tiles
   static constexpr int kK = 64 * LDK;                       // sK, later sTw
   static constexpr int kKT = DK * LDC;                      // sKT
-  static constexpr int kQ = (64 * LDK > 64 * LDC) ? 64 * LDK : 64 * LDC;  // sQ, later a V^T slab
+  static constexpr int kQ = (64 * LDK > DK * LDC) ? 64 * LDK : DK * LDC;  // sQ, later Qg^T, then V^T slabs
   static constexpr size_t bytes = sizeof(T) * (kK + kKT + kQ) + sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36 + 128);
 };
 
@@ -121,7 +121,12 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
     }
   }
   __syncthreads();
+  // (scale * Q * e^G)^T for the backward scan, staged through the sQ region
+  stage_rows_t<T>(sQ, LDC, qg, DK, 64, len, DK, tid, [&](int r) {
+    return (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
+  });
   tri_inverse_64(sA, sT, sX, tid);
+  unstage_rows<T>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, 64, tid);
 
   // Tw = Tm * diag(beta e^G) (into the sK region), Tu = Tm * diag(beta) (into the sA region),
   // Tm^T to the workspace.
@@ -154,6 +159,7 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
       frag_zero(acc);
       mma_nt<T, 1, 1>(acc, sTw + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
       frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
+      frag_store_t<T, 1, 1>(acc, ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)(c0 + 32 * wj) * 64 + 32 * wi, 64, lane);
     }
     // K^T for the scan kernel
     unstage_rows<T>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, 64, tid);
