@@ -1,0 +1,214 @@
+"""Benchmark of the chunked delta-rule scan on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode]
+
+Default workload: Gated DeltaNet chunked forward+backward at B=8, H=16, T=4096, dk=dv=128,
+bf16 q/k/v/dO, fp32 beta/g, chunk 64 (benchmark configuration 2).  One "step" is one forward
+plus one backward pass through the public ops (``gated_delta_rule_chunkwise`` + autograd),
+inputs resident in HBM.  Prints ONE JSON line; ``value`` is tokens/s = B*T / step time.
+
+``roofline`` describes the kernel with the largest share of the step, timed with HIP events
+recorded by the library on the launch stream during the timed steps; ``achieved`` is that
+kernel's algorithmic FLOP/s (or bytes/s).  ``cpu_baseline`` times the CPU restatement of the
+same chunk algorithm (torch, all host cores) on a bounded sample of the workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+C = 64
+PEAK_BF16 = 2500.0  # TFLOP/s, dense bf16 MFMA, MI355X
+PEAK_HBM = 8000.0   # GB/s
+
+
+def chunk_flops(dk, dv):
+    """Algorithmic dense-product FLOPs per (batch, head, chunk), split by kernel.  The forward
+    terms add up to F_chunk = 2C^2(3dk+2dv) + 6C*dk*dv and the backward terms to 2*F_chunk."""
+    cc, cd = 2 * C * C, 2 * C * dk * dv
+    return {
+        "chunk_prepare": cc * (3 * dk + dv),          # K K^T, Q K^T, Tm(beta K), Tm(beta V)
+        "chunk_scan": 2 * cd,                         # W S, K^T D
+        "chunk_output": cd + cc * dv,                 # Q S, P D
+        "bwd_local": cc * dv,                         # P^T dO
+        "bwd_scan": 3 * cd,                           # K dS, Q^T dO, W^T dD
+        "bwd_dqk": cc * dv + 3 * cd + 2 * cc * dk,    # dO D^T, dO S^T, dD S^T, D dS^T, dPe K, dPe^T Q
+        "bwd_wy": cc * (4 * dk + 2 * dv),             # Tm^T dW, Tm^T dD, dBw W^T + dBu U^T, K K^T, Y K
+    }
+
+
+def make_gdn_inputs(torch, B, H, T, d, seed, device):
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    nrm = lambda x: x / (x.norm(dim=-1, keepdim=True) + 1e-6)
+    q, k = nrm(rn(B, H, T, d)), nrm(rn(B, H, T, d))
+    v = rn(B, H, T, d)
+    beta = torch.sigmoid(rn(B, H, T))
+    g = -torch.nn.functional.softplus(rn(B, H, T)) * 0.1
+    dO = rn(B, H, T, d)
+    return {n: t.to(device) for n, t in dict(q=q, k=k, v=v, beta=beta, g=g, dO=dO).items()}
+
+
+def cpu_baseline_chunk(torch, B, H, T, d, seed):
+    """fwd+bwd of the CPU restatement (chunk form + autograd) on a bounded sample: B_s batch rows."""
+    from oracle import torch_ref as tr
+
+    threads = torch.get_num_threads()
+    Bs = max(1, B // 2)
+    x = make_gdn_inputs(torch, Bs, H, T, d, seed, "cpu")
+
+    def run(xs):
+        inp = {"q": xs["q"], "k": xs["k"], "v": xs["v"], "beta": xs["beta"], "g": xs["g"], "initial_state": None}
+        tr.grads(tr.chunkwise, inp, xs["dO"], None, use_qk_l2norm=False)
+
+    run({n: t[:1, :2] for n, t in x.items()})  # warm-up
+    t0 = time.perf_counter()
+    run(x)
+    dt = time.perf_counter() - t0
+    return {"value": Bs * T / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"B={Bs} of {B} batch rows, H={H}, T={T}, d={d}, fp32, one timed pass ({dt:.1f} s)"}
+
+
+def bench_gdn_chunk(args, torch, la, _lib):
+    B, H, T, d = 8, 16, 4096, 128
+    dev = "cuda:0"
+    x = make_gdn_inputs(torch, B, H, T, d, 2, dev)
+    q, k, v, dO = (x[n].to(torch.bfloat16) for n in ("q", "k", "v", "dO"))
+    beta, g = x["beta"], x["g"]
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    beta.requires_grad_(True), g.requires_grad_(True)
+
+    def step():
+        for t in (q, k, v, beta, g):
+            t.grad = None
+        o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, use_qk_l2norm=False)
+        o.backward(dO)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    per_kernel = {}
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step()
+        if (i + 1) % 512 == 0:  # the library keeps a bounded number of event marks
+            for name, ms in _lib.profile_read():
+                per_kernel.setdefault(name, []).append(ms)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    for name, ms in _lib.profile_read():
+        per_kernel.setdefault(name, []).append(ms)
+    _lib.profile_enable(False)
+
+    nchunks = B * H * (T // C)
+    fl = chunk_flops(d, d)
+    avg = {n: sum(v_) / len(v_) for n, v_ in per_kernel.items()}
+    dom = max(avg, key=avg.get)
+    achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
+    total_fl = 3 * (2 * C * C * (3 * d + 2 * d) + 6 * C * d * d) * nchunks
+    out = {
+        "metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
+        "value": B * T / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "gated_deltanet_chunk_fwd_bwd", "B": B, "H": H, "T": T, "dk": d, "dv": d, "chunk": C,
+                   "use_qk_l2norm": False, "inputs": "q,k pre-normalised; bf16 q/k/v/dO, fp32 beta/g"},
+        "tflops_algorithmic": total_fl / dt / 1e12,
+        "mfma_peak_frac": total_fl / dt / 1e12 / PEAK_BF16,
+        "kernel_ms": {n: round(t, 4) for n, t in avg.items()},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16, "traffic": None},
+    }
+    return out, (B, H, T, d)
+
+
+def bench_decode(args, torch, la, _lib, steps=None):
+    """Gated DeltaNet decode step at B=256, H=32, dk=dv=128: fp32 state updated in place."""
+    B, H, d = 256, 32, 128
+    dev = "cuda:0"
+    gen = torch.Generator(device="cpu").manual_seed(4)
+    rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    nrm = lambda x: x / (x.norm(dim=-1, keepdim=True) + 1e-6)
+    S = (rn(B, H, d, d) * 0.02).to(dev)
+    q, k = nrm(rn(B, H, d)).to(dev).bfloat16(), nrm(rn(B, H, d)).to(dev).bfloat16()
+    v = rn(B, H, d).to(dev).bfloat16()
+    beta = torch.sigmoid(rn(B, H)).to(dev)
+    g = (-torch.nn.functional.softplus(rn(B, H)) * 0.1).to(dev)
+    steps = steps or 1000
+
+    def step():
+        la.gated_delta_rule_step(q, k, v, g, beta, S, use_qk_l2norm=False, inplace=True)
+
+    for _ in range(20):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    kern = []
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step()
+        if (i + 1) % 2048 == 0:
+            kern += [ms for _, ms in _lib.profile_read()]
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    kern += [ms for _, ms in _lib.profile_read()]
+    _lib.profile_enable(False)
+    nbytes = 2 * S.numel() * 4 + 4 * B * H * d * 2 + 2 * B * H * 4
+    kms = sum(kern) / len(kern)
+    return {
+        "workload": "gated_deltanet_decode_step", "B": B, "H": H, "dk": d, "dv": d, "steps": steps,
+        "ms_per_step": dt * 1e3, "tokens_per_s": B / dt, "bytes_per_step": nbytes,
+        "roofline": {"bound": "hbm", "kernel": "decode_step", "achieved": nbytes / (kms * 1e-3) / 1e9, "peak": PEAK_HBM,
+                     "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: the scan needs no collective and every figure here is "
+              "single-GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import linearnexus_amd as la
+    from linearnexus_amd import _lib
+
+    _lib.load()  # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
+        sys.exit(2)
+
+    if args.workload == "decode":
+        dec = bench_decode(args, torch, la, _lib, steps=max(args.steps, 100))
+        out = {"metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
+               "value": dec["roofline"]["achieved"], "unit": "GB/s", "n_gpus": 1, "steps": dec["steps"],
+               "warmup": 20, "ms_per_step": dec["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+               "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+               "config": {k_: dec[k_] for k_ in ("workload", "B", "H", "dk", "dv")}, "roofline": dec["roofline"]}
+        print(json.dumps(out))
+        return
+
+    out, (B, H, T, d) = bench_gdn_chunk(args, torch, la, _lib)
+    out["decode_step"] = bench_decode(args, torch, la, _lib)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_chunk(torch, B, H, T, d, 2)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -120,6 +120,17 @@ int lnx_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t d, int32_t dtyp
 int lnx_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_t d, int32_t dtype,
                    void* hip_stream);
 
+/*
+ * Optional per-kernel timing for benchmarks (no counterpart in the reference; its micro-benchmark
+ * times whole jitted ops, bench_kda_kernels.py:216-249).  While enabled (process-wide),
+ * every entry point records HIP events around each kernel it launches, on the caller's stream.
+ * lnx_profile_read waits for them, returns the number of kernels timed since the last read and
+ * fills up to `capacity` (name, milliseconds) pairs.  At most 8192 marks (one per kernel plus one
+ * per entry-point call) are kept between reads.
+ */
+int lnx_profile_enable(int on);
+int lnx_profile_read(int capacity, const char** names, float* ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,6 +16,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
+    "lnx_profile_enable", "lnx_profile_read",
 )
 
 
@@ -61,8 +62,25 @@ def load() -> C.CDLL:
     lib.lnx_l2norm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
     lib.lnx_l2norm_bwd.restype = C.c_int
     lib.lnx_l2norm_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lnx_profile_enable.restype = C.c_int
+    lib.lnx_profile_enable.argtypes = [C.c_int]
+    lib.lnx_profile_read.restype = C.c_int
+    lib.lnx_profile_read.argtypes = [C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_float)]
     _lib = lib
     return lib
+
+
+def profile_enable(on: bool) -> None:
+    """Turns per-kernel HIP-event timing on or off for the calling thread."""
+    load().lnx_profile_enable(int(on))
+
+
+def profile_read(capacity: int = 8192):
+    """Returns [(kernel name, milliseconds), ...] for the kernels launched since the last read."""
+    names = (C.c_char_p * capacity)()
+    ms = (C.c_float * capacity)()
+    n = load().lnx_profile_read(capacity, names, ms)
+    return [(names[i].decode(), float(ms[i])) for i in range(min(n, capacity))]
 
 
 class HipKernelError(RuntimeError):

@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "lnx_common.h"
 
 namespace {
@@ -20,6 +22,57 @@ int lnx_set_error(int code, const char* fmt, ...) {
 extern "C" const char* lnx_last_error(void) { return g_error; }
 extern "C" int lnx_abi_version(void) { return 1; }
 
+// ---- optional per-kernel timing with HIP events on the caller's stream.  Process-wide (one
+// mutex-guarded list) because a framework may run the backward entry point on another thread. ----
+namespace {
+struct Profile {
+  bool on = false;
+  int n = 0;  // events recorded
+  hipEvent_t ev[LNX_PROFILE_MAX + 1];
+  const char* name[LNX_PROFILE_MAX];
+  int created = 0;
+};
+Profile g_prof;
+std::mutex g_prof_mutex;
+}  // namespace
+
+void lnx_profile_mark(const char* kernel_name, hipStream_t st) {
+  Profile& P = g_prof;
+  if (!P.on) return;  // unguarded fast path: timing is off in normal use
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  if (!P.on || P.n > LNX_PROFILE_MAX) return;
+  if (kernel_name != nullptr && P.n == LNX_PROFILE_MAX) return;  // keep one slot for the closing mark
+  if (P.created <= P.n) {
+    if (hipEventCreate(&P.ev[P.created]) != hipSuccess) return;
+    ++P.created;
+  }
+  if (hipEventRecord(P.ev[P.n], st) != hipSuccess) return;
+  if (P.n < LNX_PROFILE_MAX) P.name[P.n] = kernel_name;
+  ++P.n;
+}
+
+extern "C" int lnx_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof.on = on != 0;
+  g_prof.n = 0;
+  return LNX_OK;
+}
+
+extern "C" int lnx_profile_read(int capacity, const char** names, float* ms) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  Profile& P = g_prof;
+  int out = 0;
+  for (int i = 0; i + 1 < P.n && i < LNX_PROFILE_MAX; ++i) {
+    if (P.name[i] == nullptr) continue;  // a closing mark: the gap to the next entry point
+    if (hipEventSynchronize(P.ev[i + 1]) != hipSuccess) break;
+    float t = 0.f;
+    if (hipEventElapsedTime(&t, P.ev[i], P.ev[i + 1]) != hipSuccess) break;
+    if (out < capacity) { names[out] = P.name[i]; ms[out] = t; }
+    ++out;
+  }
+  P.n = 0;
+  return out;
+}
 namespace {
 
 // One wavefront per row: y = x / (|x| + eps).

@@ -414,9 +414,13 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b3)) != hipSuccess)
     return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  lnx_profile_mark("chunk_prepare", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
+  lnx_profile_mark("chunk_scan", st);
   hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / 64)), dim3(256), b2, st, p);
+  lnx_profile_mark("chunk_output", st);
   hipLaunchKernelGGL(k3, dim3((unsigned)slots, (unsigned)(p.dv / 64)), dim3(256), b3, st, p);
+  lnx_profile_mark(nullptr, st);
   return LNX_OK;
 }
 

@@ -21,6 +21,11 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // Host side: records a message for lnx_last_error() and returns `code`.
 int lnx_set_error(int code, const char* fmt, ...);
 
+// Host side: when per-kernel timing is enabled (lnx_profile_enable), records a HIP event on
+// `st` before the kernel named `kernel_name`; a NULL name closes the current entry point.
+#define LNX_PROFILE_MAX 8192
+void lnx_profile_mark(const char* kernel_name, hipStream_t st);
+
 __device__ __forceinline__ float to_f32(float x) { return x; }
 __device__ __forceinline__ float to_f32(bf16_t x) { return (float)x; }
 

@@ -244,8 +244,10 @@ int token_entry(bool decode, const lnx_scan_args* a, void* stream) {
   p.H = a->H; p.T = a->T; p.dv = a->dv; p.scale = a->scale; p.l2norm = a->use_qk_l2norm; p.o_dtype = a->o_dtype;
   dim3 grid((unsigned)(nstate * a->H), (unsigned)((a->dv + (decode ? 127 : 31)) / (decode ? 128 : 32)));
   hipStream_t st = (hipStream_t)stream;
+  lnx_profile_mark(decode ? "decode_step" : "recurrent_fwd", st);
   int rc = (a->dtype == LNX_BF16) ? launch_dk<bf16_t>(decode, a->dk, a->gate, p, grid, st)
                                   : launch_dk<float>(decode, a->dk, a->gate, p, grid, st);
+  lnx_profile_mark(nullptr, st);
   if (rc != LNX_OK) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "token kernel launch: %s", hipGetErrorString(e));
