@@ -14,6 +14,7 @@
 //   KT   [dk][64]   K^T (scalar / no gate) or (K * exp(G_last - G))^T (vector gate)
 //   WT   [dk][64]   W^T            QgT [dk][64]  (scale * Q * exp(G))^T
 //   TmT  [64][64]   ((I + A)^-1)^T, used by the backward pass
+//   X    [64][64]   <k_i, k_j>_E, i > j, and  Kr [64][dk] = K * exp(G_last - G)   (vector gate only)
 //   D    [64][dv]   U - W S            DT [dv][64] its transpose
 //   SnT  [dv][dk]   transpose of the state entering the chunk
 // Backward adds dOT [dv][64], dD [64][dv], dDT [dv][64], dSn [dk][dv] (gradient of the state
@@ -50,7 +51,7 @@ __device__ __forceinline__ void seq_chunks(const ChunkGeom& g, int s, int& c0, i
 }
 
 struct ChunkWs {
-  uint64_t tab, G, P, W, WT, QgT, U, KT, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, dG, total;
+  uint64_t tab, G, P, X, W, WT, QgT, U, KT, Kr, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, dG, total;
 };
 
 inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
@@ -70,11 +71,13 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.tab = take(a->cu_seqlens ? (2 * N + a->nseq + 1) * 4 : 0);
   w.G = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
+  w.X = take(a->gate == LNX_GATE_VECTOR ? slots * C * C * es : 0);
   w.W = take(slots * C * dk * es);
   w.WT = take(slots * dk * C * es);
   w.QgT = take(slots * dk * C * es);
   w.U = take(slots * C * dv * es);
   w.KT = take(slots * dk * C * es);
+  w.Kr = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * es : 0);
   w.TmT = take(slots * C * C * es);
   w.D = take(slots * C * dv * es);
   w.DT = take(slots * dv * C * es);
@@ -94,3 +97,43 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward);
 
 // Builds the packed-batch chunk table (no-op for dense batches).
 void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st);
+
+// ---------------------------------------------------------------------------------------
+// Vector-gate (KDA) helpers: per-channel decays E_ij[c] = prod_{m=j+1..i} alpha_m[c] are applied
+// with a multiplicative recurrence along the token index, so no exponent of a positive number
+// is ever taken (the property kda.py:426-434 protects with its blocked factorisation).
+// Tiles live in LDS: M [64][LNX_LDA] fp32, al (alpha) and out [64][ldf] fp32, operands [64][ldb].
+// A wavefront owns a token row (or column), its lanes the channels.
+// ---------------------------------------------------------------------------------------
+
+// out[i][c] += mul * sum_{j <= i (j < i if STRICT)} M[i][j] * E_ij[c] * b[j][c]
+template <typename T, int DK, bool STRICT>
+__device__ __forceinline__ void pair_row(float* out, const float* M, const float* al, int ldf, const T* b, int ldb,
+                                         float mul, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int i = wave; i < 64; i += 4)
+    for (int c = lane; c < DK; c += 64) {
+      float e = 1.f, acc = 0.f;
+      for (int j = i; j >= 0; --j) {
+        if (!(STRICT && j == i)) acc += M[i * LNX_LDA + j] * e * to_f32(b[j * ldb + c]);
+        e *= al[j * ldf + c];
+      }
+      out[i * ldf + c] += mul * acc;
+    }
+}
+
+// out[j][c] += mul * sum_{i >= j (i > j if STRICT)} M[i][j] * E_ij[c] * a[i][c]
+template <typename T, int DK, bool STRICT>
+__device__ __forceinline__ void pair_col(float* out, const float* M, const float* al, int ldf, const T* a, int lda,
+                                         float mul, int tid) {
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int j = wave; j < 64; j += 4)
+    for (int c = lane; c < DK; c += 64) {
+      float e = 1.f, acc = 0.f;
+      for (int i = j; i < 64; ++i) {
+        if (i > j) e *= al[i * ldf + c];
+        if (!(STRICT && i == j)) acc += M[i * LNX_LDA + j] * e * to_f32(a[i * lda + c]);
+      }
+      out[j * ldf + c] += mul * acc;
+    }
+}

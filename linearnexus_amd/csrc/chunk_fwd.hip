@@ -181,6 +181,162 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
+// kda_prepare: chunk_prepare for a per-channel (vector) gate.  The pairwise products carry the
+// decay inside the dk sum, X_ij = sum_c k_i[c] k_j[c] exp(G_i[c] - G_j[c]); they are evaluated
+// on the VALU with exponents of non-positive numbers only (i >= j), as the reference does for
+// its diagonal blocks (kda.py:483-502).  Everything after A is the same MFMA pipeline, with the
+// decays folded element-wise into the staged operands.
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct KdaPrepSmem {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
+  static constexpr int kK = 64 * LDK;                                     // sK, later the T-typed copy of Tm
+  static constexpr int kQ = (64 * LDK > DK * LDC) ? 64 * LDK : DK * LDC;  // sQ, later transposed staging
+  static constexpr size_t bytes =
+      sizeof(T) * (kK + kQ) + sizeof(float) * (64 * LDF + 2 * 64 * LNX_LDA + 32 * 36 + 64);
+};
+
+template <typename T, int DK>
+__global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
+  typedef KdaPrepSmem<T, DK> L;
+  constexpr int LDK = L::LDK, LDC = L::LDC, LDF = L::LDF;
+  extern __shared__ __align__(16) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);
+  T* sQ = sK + L::kK;
+  float* sG = reinterpret_cast<float*>(sQ + L::kQ);  // [64][LDF] cumulative gate
+  float* sA = sG + 64 * LDF;
+  float* sT = sA + 64 * LNX_LDA;
+  float* sX = sT + 64 * LNX_LDA;
+  float* sBeta = sX + 32 * 36;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+
+  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
+  stage_rows<T>(sQ, LDK, qg, DK, 64, len, DK, tid);
+  for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
+    const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+    floatx4 x = {0.f, 0.f, 0.f, 0.f};
+    if (r < len) x = load4(p.g + (tbase + r) * DK + c);
+    store4(sG + r * LDF + c, x);
+  }
+  if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+  __syncthreads();
+  if (tid < DK) {
+    float acc = 0.f;
+    for (int r = 0; r < 64; ++r) {
+      acc += sG[r * LDF + tid];
+      sG[r * LDF + tid] = acc;
+    }
+  }
+  __syncthreads();
+  {
+    float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
+    T* Krg = ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK;
+    for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
+      const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+      const floatx4 gr = load4(sG + r * LDF + c), gl = load4(sG + 63 * LDF + c), kk = load4(sK + r * LDK + c);
+      store4(Gg + r * DK + c, gr);
+      floatx4 kr;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) kr[e] = kk[e] * __expf(fminf(gl[e] - gr[e], 0.f));
+      store4(Krg + r * DK + c, kr);
+    }
+  }
+  // pairwise products with the decay inside the channel sum
+  {
+    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
+    T* Xg = ws_ptr<T>(p, p.off.X) + slot * 64 * 64;
+    for (int idx = tid; idx < 64 * 64; idx += 256) {
+      const int i = idx >> 6, j = idx & 63;
+      float x = 0.f, pp = 0.f;
+      if (j <= i) {
+        for (int c = 0; c < DK; c += 4) {
+          const floatx4 gi = load4(sG + i * LDF + c), gj = load4(sG + j * LDF + c);
+          const floatx4 ki = load4(sK + i * LDK + c), kj = load4(sK + j * LDK + c), qi = load4(sQ + i * LDK + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float ee = __expf(fminf(gi[e] - gj[e], 0.f)) * kj[e];
+            x += ki[e] * ee;
+            pp += qi[e] * ee;
+          }
+        }
+      }
+      x = (j < i) ? x : 0.f;
+      sA[i * LNX_LDA + j] = sBeta[i] * x;
+      Xg[idx] = from_f32<T>(x);
+      Pg[idx] = from_f32<T>(p.scale * pp);
+    }
+  }
+  __syncthreads();
+  // (scale * Q * e^G)^T through the sQ region
+  stage_rows_t_elem<T>(sQ, LDC, qg, DK, 64, len, DK, tid,
+                       [&](int r, int c) { return p.scale * __expf(sG[r * LDF + c]); });
+  tri_inverse_64(sA, sT, sX, tid);
+  unstage_rows<T>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, 64, tid);
+
+  T* sTm = sK;                         // T-typed copy of Tm (bf16); fp32 reads sT in place
+  T* sTu = reinterpret_cast<T*>(sA);   // Tm * diag(beta)
+  {
+    T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
+    for (int idx = tid; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
+      TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
+      const float t = sT[r * LNX_LDA + c];
+      sTu[r * LDC + c] = from_f32<T>(t * sBeta[c]);
+      if (sizeof(T) == 2) sTm[r * LDC + c] = from_f32<T>(t);
+    }
+  }
+  const T* tm_op = (sizeof(T) == 4) ? reinterpret_cast<const T*>(sT) : sTm;
+  __syncthreads();
+  // W = Tm (beta e^G K): transposed, scaled K through the sQ region
+  T* sKT = sQ;
+  stage_rows_t_elem<T>(sKT, LDC, kg, DK, 64, len, DK, tid,
+                       [&](int r, int c) { return sBeta[r] * __expf(sG[r * LDF + c]); });
+  __syncthreads();
+  const int wi = wave >> 1, wj = wave & 1;
+  {
+    T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
+    for (int c0 = 0; c0 < DK; c0 += 64) {
+      floatx16 acc[1][1];
+      frag_zero(acc);
+      mma_nt<T, 1, 1>(acc, tm_op + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
+      frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
+      frag_store_t<T, 1, 1>(acc, ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)(c0 + 32 * wj) * 64 + 32 * wi, 64, lane);
+    }
+  }
+  __syncthreads();
+  // (K * e^{G_last - G})^T for the scan kernel
+  stage_rows_t_elem<T>(sKT, LDC, kg, DK, 64, len, DK, tid,
+                       [&](int r, int c) { return __expf(fminf(sG[63 * LDF + c] - sG[r * LDF + c], 0.f)); });
+  __syncthreads();
+  unstage_rows<T>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, 64, tid);
+  // U = Tu V
+  {
+    T* sVT = sQ;
+    T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
+    for (int c0 = 0; c0 < p.dv; c0 += 64) {
+      __syncthreads();
+      stage_rows_t<T>(sVT, LDC, vg + c0, p.dv, 64, len, 64, tid, UnitScale());
+      __syncthreads();
+      floatx16 acc[1][1];
+      frag_zero(acc);
+      mma_nt<T, 1, 1>(acc, sTu + 32 * wi * LDC, LDC, sVT + 32 * wj * LDC, LDC, 64, lane);
+      frag_store<T, 1, 1>(acc, Ug + 32 * wi * p.dv + c0 + 32 * wj, p.dv, lane);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // chunk_scan
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct ScanSmem {
@@ -189,7 +345,7 @@ template <typename T, int DK> struct ScanSmem {
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int BV = 64;
   static constexpr int kW = 64 * LDK, kKT = DK * LDC, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
-  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 64;
+  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
@@ -248,7 +404,8 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
       rU[i] = *reinterpret_cast<const V16*>(Ug + (int64_t)r * p.dv + c);
     }
-    if (GATE != LNX_GATE_NONE && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
+    if (GATE == LNX_GATE_SCALAR && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
+    if (GATE == LNX_GATE_VECTOR && tid < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];  // G_last[c]
   };
   auto commit = [&]() {
 #pragma unroll
@@ -266,7 +423,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
       *reinterpret_cast<V16*>(sU + r * LDU + c) = rU[i];
     }
-    if (tid < 64) sG[tid] = rG;
+    if (tid < 128) sG[tid] = rG;
   };
 
   if (c0 < c1) fetch(c0);
@@ -284,7 +441,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     floatx16 d[1][1];
     frag_zero(d);
     mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
-    const float gl = (GATE == LNX_GATE_NONE) ? 0.f : sG[63];
+    const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
@@ -294,7 +451,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
                         p.dv, lane);
     frag_store_t<T, 1, 1>(d, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)(v0 + 32 * wj) * 64 + 32 * wi, 64,
                           lane);
-    if (GATE != LNX_GATE_NONE) {
+    if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
     }
@@ -302,12 +459,18 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     __syncthreads();
 
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
-    if (GATE != LNX_GATE_NONE) {
+    if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) S[0][j][e] *= dec;
+    }
+    if (GATE == LNX_GATE_VECTOR) {  // per state row (key channel)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
     mma_nt<T, 1, NT>(S, sKT + srow * LDC, LDC, sDT + scol * LDC, LDC, 64, lane);
     __syncthreads();
@@ -353,11 +516,27 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   if (len <= 0) return;
   const int64_t tbase = (int64_t)row * p.geom.T + tok0;
 
-  stage_rows<T>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, 64, len, DK, tid);
+  if (GATE == LNX_GATE_VECTOR) {
+    constexpr int VN = Vec16<T>::N;
+    const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
+    const float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
+    for (int idx = tid; idx < 64 * DK / VN; idx += 256) {
+      const int r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
+      typename Vec16<T>::V x = vec_zero<T>();
+      if (r < len) {
+        x = *reinterpret_cast<const typename Vec16<T>::V*>(qg + (int64_t)r * DK + c);
+#pragma unroll
+        for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * p.scale * __expf(Gg[r * DK + c + e]));
+      }
+      *reinterpret_cast<typename Vec16<T>::V*>(sQ + r * LDK + c) = x;
+    }
+  } else {
+    stage_rows<T>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, 64, len, DK, tid);
+  }
   stage_rows<T>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, BV, DK, tid);
   stage_rows<T>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, 64, 64, tid);
   stage_rows<T>(sDT, LDC, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, BV, BV, 64, tid);
-  if (tid < 64) sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
+  if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
   __syncthreads();
 
   const int wi = wave >> 1, wj = wave & 1;
@@ -366,7 +545,7 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   mma_nt<T, 1, 1>(acc, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
-    const float gm = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+    const float gm = (GATE == LNX_GATE_VECTOR) ? 1.f : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
     acc[0][0][e] *= gm;
   }
   mma_nt<T, 1, 1>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj * LDC, LDC, 64, lane);
@@ -402,13 +581,22 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* 
   }
 }
 
+template <typename T, int DK, int GATE> struct PrepSelect {
+  static constexpr size_t bytes = PrepSmem<T, DK>::bytes;
+  static auto kernel() { return chunk_prepare_kernel<T, DK, GATE>; }
+};
+template <typename T, int DK> struct PrepSelect<T, DK, LNX_GATE_VECTOR> {
+  static constexpr size_t bytes = KdaPrepSmem<T, DK>::bytes;
+  static auto kernel() { return kda_prepare_kernel<T, DK>; }
+};
+
 template <typename T, int DK, int GATE>
 int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
-  auto k1 = chunk_prepare_kernel<T, DK, GATE>;
+  auto k1 = PrepSelect<T, DK, GATE>::kernel();
   auto k2 = chunk_scan_kernel<T, DK, GATE>;
   auto k3 = chunk_output_kernel<T, DK, GATE>;
-  const size_t b1 = PrepSmem<T, DK>::bytes, b2 = ScanSmem<T, DK>::bytes, b3 = OutSmem<T, DK>::bytes;
+  const size_t b1 = PrepSelect<T, DK, GATE>::bytes, b2 = ScanSmem<T, DK>::bytes, b3 = OutSmem<T, DK>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
@@ -429,7 +617,8 @@ int launch_fwd_gate(int gate, const FwdParams& p, int nstate, hipStream_t st) {
   switch (gate) {
     case LNX_GATE_NONE: return launch_fwd<T, DK, LNX_GATE_NONE>(p, nstate, st);
     case LNX_GATE_SCALAR: return launch_fwd<T, DK, LNX_GATE_SCALAR>(p, nstate, st);
-    default: return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels: gate kind %d is not supported yet", gate);
+    case LNX_GATE_VECTOR: return launch_fwd<T, DK, LNX_GATE_VECTOR>(p, nstate, st);
+    default: return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", gate);
   }
 }
 

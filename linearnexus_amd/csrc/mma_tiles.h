@@ -177,6 +177,31 @@ __device__ __forceinline__ void stage_rows_t(T* dst, int ld, const T* src, int64
   }
 }
 
+// As stage_rows_t with a per-element factor f(r, c).
+template <typename T, typename F>
+__device__ __forceinline__ void stage_rows_t_elem(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
+                                                  int cols, int tid, F elem_scale) {
+  constexpr int N = Vec16<T>::N;
+  const int vpr = cols / N;
+  for (int idx = tid; idx < (rows / 4) * vpr; idx += 256) {
+    const int rg = idx / vpr, c = (idx - rg * vpr) * N;
+    typename Vec16<T>::V x[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * rg + i;
+      x[i] = vec_zero<T>();
+      if (r < valid) x[i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      floatx4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = to_f32(x[i][e]) * elem_scale(4 * rg + i, c + e);
+      store4(dst + (c + e) * ld + 4 * rg, y);
+    }
+  }
+}
+
 struct UnitScale {
   __device__ __forceinline__ float operator()(int) const { return 1.f; }
 };
