@@ -101,7 +101,7 @@ template <typename T, int DK> struct BScanCfg {
   static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDU = BV + PAD;
   static constexpr int kK = 64 * LDK, kQT = DK * LDC, kWT = DK * LDC, kdOT = BV * LDC, kdDl = 64 * LDU,
                        kdST = BV * LDK, kdDT = BV * LDC;
-  static constexpr size_t bytes = sizeof(T) * (kK + kQT + kWT + kdOT + kdDl + kdST + kdDT) + sizeof(float) * 64;
+  static constexpr size_t bytes = sizeof(T) * (kK + kQT + kWT + kdOT + kdDl + kdST + kdDT) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
@@ -154,7 +154,10 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
     int tok0, len;
     chunk_span(p.geom, n, tok0, len);
     const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-    const T* Kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+    // vector gate: K * e^{G_last - G} was stored by the forward pass (all 64 rows defined)
+    const T* Kg = (GATE == LNX_GATE_VECTOR) ? wsp<T>(p, p.off.Kr) + slot * 64 * DK
+                                            : reinterpret_cast<const T*>(p.k) + tbase * DK;
+    if (GATE == LNX_GATE_VECTOR) len = 64;
     const T* Wg = wsp<T>(p, p.off.WT) + slot * DK * 64;
     const T* Qg = wsp<T>(p, p.off.QgT) + slot * DK * 64;
 #pragma unroll
@@ -176,10 +179,11 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
         rD[i] = *reinterpret_cast<const V16*>(Dg + (int64_t)r * p.dv + c);
       }
     }
-    if (GATE != LNX_GATE_NONE && tid < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + tid];
+    if (GATE == LNX_GATE_SCALAR && tid < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + tid];
+    if (GATE == LNX_GATE_VECTOR && tid < DK) rG = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];
   };
   auto commit = [&]() {
-    if (tid < 64) sG[tid] = rG;
+    if (tid < 128) sG[tid] = rG;
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
     __syncthreads();
     if (n > c0) fetch(n - 1);
 
-    const float gl = (GATE == LNX_GATE_NONE) ? 0.f : sG[63];
+    const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
     // dD = dD_loc + r_j (K dS)_j
     if (has_tile) {
       floatx16 d[1][1];
@@ -219,7 +223,7 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        const float rj = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
+        const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[r], 0.f)) : 1.f;
         d[0][0][e] = to_f32(sdDl[r * LDU + c]) + rj * d[0][0][e];
       }
       frag_store<T, 1, 1>(d, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
@@ -231,12 +235,18 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
     __syncthreads();
 
     // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD
-    if (GATE != LNX_GATE_NONE) {
+    if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) dS[0][j][e] *= dec;
+    }
+    if (GATE == LNX_GATE_VECTOR) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dS[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
     mma_nt<T, 1, NT>(dS, sQT + srow * LDC, LDC, sdOT + scol * LDC, LDC, 64, lane);
     mma_nt<T, 1, NT>(dS, sWT + srow * LDC, LDC, sdDT + scol * LDC, LDC, 64, lane);
@@ -255,36 +265,37 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
 // ---------------------------------------------------------------------------------------
 // bwd_dqk
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct DqkCfg {
+template <typename T, int DK, int GATE> struct DqkCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD;
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
   // loop phase: dO, D, dD slabs [64][LDC] and S_n, dS_n slabs [DK][LDC]
-  // epilogue:   dPe, dPe^T [64][LDC] and K^T, Q^T [DK][LDC]   (same footprint minus one tile)
+  // epilogue (scalar / no gate): dPe, dPe^T [64][LDC] and K^T, Q^T [DK][LDC] overlaid on the slabs
+  // epilogue (vector gate): alpha, out [64][LDF] fp32 and K, Q [64][LDK] overlaid on the slabs
   static constexpr int kTile = 64 * LDC, kWide = DK * LDC;
-  static constexpr size_t bytes = sizeof(T) * (3 * kTile + 2 * kWide) + sizeof(float) * (64 * LNX_LDA + 64 * 4);
+  static constexpr size_t loop_bytes = sizeof(T) * (3 * kTile + 2 * kWide);
+  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 2 * 64 * LDK;
+  static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > loop_bytes) ? vec_bytes : loop_bytes;
+  static constexpr int kSmall = 64 * LNX_LDA + 64 * 4 + DK;  // floats: sR, sG, sdG, sTj, sMisc, sSS
+  static constexpr size_t bytes = sizeof(float) * kSmall + big;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
-  typedef DqkCfg<T, DK> L;
+  typedef DqkCfg<T, DK, GATE> L;
   typedef RowTiles<DK> RTl;
-  constexpr int LDC = L::LDC, MT = RTl::MT;
+  constexpr int LDC = L::LDC, LDK = L::LDK, LDF = L::LDF, MT = RTl::MT;
   extern __shared__ __align__(16) char smem[];
-  T* sdO = reinterpret_cast<T*>(smem);
-  T* sD = sdO + L::kTile;
-  T* sdD = sD + L::kTile;
-  T* sSn = sdD + L::kTile;
-  T* sdSn = sSn + L::kWide;
-  float* sR = reinterpret_cast<float*>(sdSn + L::kWide);  // [64][LNX_LDA]
+  float* sR = reinterpret_cast<float*>(smem);  // [64][LNX_LDA]
   float* sG = sR + 64 * LNX_LDA;
   float* sdG = sG + 64;     // per-row gate-gradient accumulator
   float* sTj = sdG + 64;    // r_j <dKr_j, k_j>
   float* sMisc = sTj + 64;  // [0] = <dS_n, S_n>
-  // epilogue overlays
-  T* sPe = sdO;
-  T* sPeT = sD;
-  T* sKT = sSn;
-  T* sQT = sdSn;
+  float* sSS = sMisc + 64;  // [DK] per key channel: sum_v dS_n[c][v] S_n[c][v]   (vector gate)
+  T* sdO = reinterpret_cast<T*>(sSS + DK);
+  T* sD = sdO + L::kTile;
+  T* sdD = sD + L::kTile;
+  T* sSn = sdD + L::kTile;
+  T* sdSn = sSn + L::kWide;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -300,11 +311,12 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
   const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
 
   if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : wsp<float>(p, p.off.G)[slot * 64 + tid];
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
     sdG[tid] = 0.f;
     sTj[tid] = 0.f;
     if (tid == 0) sMisc[0] = 0.f;
   }
+  if (tid < DK) sSS[tid] = 0.f;
 
   floatx16 aP[1][1], aQ[MT][1], aW[MT][1], aK[MT][1];
   frag_zero(aP);
@@ -325,15 +337,13 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
     mma_nt<T, MT, 1>(aW, sdD + r0 * LDC, LDC, sSn + c0 * LDC, LDC, 64, lane);
     mma_nt<T, MT, 1>(aK, sD + r0 * LDC, LDC, sdSn + c0 * LDC, LDC, 64, lane);
     if (GATE != LNX_GATE_NONE)
-      for (int idx = tid; idx < DK * 64; idx += 256) {
-        const int r = idx >> 6, c = idx & 63;
-        ss += to_f32(sSn[r * LDC + c]) * to_f32(sdSn[r * LDC + c]);
+      for (int r = wave; r < DK; r += 4) {  // one key channel per wavefront, lanes over the slab
+        const float t = wave_sum(to_f32(sSn[r * LDC + lane]) * to_f32(sdSn[r * LDC + lane]));
+        if (GATE == LNX_GATE_VECTOR) { if (lane == 0) sSS[r] += t; }
+        else ss += t;
       }
   }
-  if (GATE != LNX_GATE_NONE) {
-    ss = wave_sum(ss);
-    if (lane == 0) atomicAdd(&sMisc[0], ss);
-  }
+  if (GATE == LNX_GATE_SCALAR && lane == 0) atomicAdd(&sMisc[0], ss);
   __syncthreads();  // slabs are dead from here on; sG, sdG initialised
 
   // dW = -dD S_n^T to the workspace
@@ -345,89 +355,165 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
       for (int e = 0; e < 16; ++e) t[i][0][e] = -aW[i][0][e];
     frag_store<T, MT, 1>(t, wsp<T>(p, p.off.dW) + slot * 64 * DK + (int64_t)r0 * DK + c0, DK, lane);
   }
-  // dP -> dPe = scale E dP (both orientations) and R = dP * P for the gate gradient
-  {
-    const T* Pg = wsp<T>(p, p.off.P) + slot * 64 * 64;
-    floatx16 pe[1][1];
+
+  if constexpr (GATE == LNX_GATE_VECTOR) {
+    // ---- per-channel gate: element-wise decays, pair terms on the VALU ----
+    float* sAl = reinterpret_cast<float*>(sdO);  // [64][LDF] alpha_j[c] = exp(g_j[c])
+    float* sOut = sAl + 64 * LDF;                // [64][LDF]
+    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDK]
+    T* sQr = sKr + 64 * LDK;                         // Q rows
+    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
+    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      const float dp = (i >= j) ? aP[0][0][e] : 0.f;
-      pe[0][0][e] = p.scale * dec * dp;
-      if (GATE != LNX_GATE_NONE) sR[i * LNX_LDA + j] = dp * to_f32(Pg[i * 64 + j]);
+      sR[i * LNX_LDA + j] = (i >= j) ? aP[0][0][e] : 0.f;
     }
-    frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
-    frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
-  }
-  // inter-chunk parts: dq = scale e^{G_i} dQg,  dk = r_j dKr, and their gate terms
-  const float gl = sG[63];
-  if (GATE != LNX_GATE_NONE) {
-    frag_rowdot<MT>(aQ, r0, c0, lane, sdG, [&](int r, int c) {
-      return (r < len) ? p.scale * __expf(sG[r]) * to_f32(qg[(int64_t)r * DK + c]) : 0.f;
-    });
-    frag_rowdot<MT>(aK, r0, c0, lane, sTj, [&](int r, int c) {
-      return (r < len) ? __expf(fminf(gl - sG[r], 0.f)) * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
-    });
-  }
+    stage_rows<T>(sKr, LDK, kg, DK, 64, len, DK, tid);
+    stage_rows<T>(sQr, LDK, qg, DK, 64, len, DK, tid);
+    for (int idx = tid; idx < 64 * DK; idx += 256) {
+      const int r = idx / DK, c = idx % DK;
+      const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
+      sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
+    }
+    // dq = scale e^G dQg (+ intra-chunk part)
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = r0 + 32 * i + frag_row(e, lane);
-      const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
-      const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
-      aQ[i][0][e] *= gq;
-      aK[i][0][e] *= gk;
+      for (int e = 0; e < 16; ++e) {
+        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
+        sOut[r * LDF + c] = aQ[i][0][e] * p.scale * __expf(Gg[r * DK + c]);
+      }
+    __syncthreads();
+    pair_row<T, DK, false>(sOut, sR, sAl, LDF, sKr, LDK, p.scale, tid);
+    __syncthreads();
+    T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK;
+    for (int idx = tid; idx < 64 * DK; idx += 256) {
+      const int r = idx / DK, c = idx % DK;
+      const float v = sOut[r * LDF + c];
+      if (r < len) dqg[(int64_t)r * DK + c] = from_f32<T>(v);
+      dGg[idx] = to_f32(sQr[r * LDK + c]) * v;
     }
-  stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
-  stage_rows_t<T>(sQT, LDC, qg, DK, 64, len, DK, tid, UnitScale());
-  __syncthreads();
-  // intra-chunk parts: dq += dPe K,  dk += dPe^T Q
-  mma_nt<T, MT, 1>(aQ, sPe + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
-  mma_nt<T, MT, 1>(aK, sPeT + r0 * LDC, LDC, sQT + c0 * LDC, LDC, 64, lane);
-  frag_store<T, MT, 1>(aQ, reinterpret_cast<T*>(p.dq) + (tbase + r0) * DK + c0, DK, lane, len - r0);
-  frag_store<T, MT, 1>(aK, reinterpret_cast<T*>(p.dk) + (tbase + r0) * DK + c0, DK, lane, len - r0);
-  // partial gate gradient wrt the cumulative gate G (row t); the chunk-end terms go to row 63
-  if (GATE != LNX_GATE_NONE && tid < 64) {
-    float rs = 0.f, cs = 0.f, tot = 0.f;
-    for (int j = 0; j < 64; ++j) {
-      rs += sR[tid * LNX_LDA + j];
-      cs += sR[j * LNX_LDA + tid];
-      tot += sTj[j];
+    __syncthreads();
+    // dk (column-type parts): e^{G_last - G} dKr (+ P part); chunk-end gate term from the Kr part
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
+        sOut[r * LDF + c] = aK[i][0][e] * __expf(fminf(Gg[63 * DK + c] - Gg[r * DK + c], 0.f));
+      }
+    __syncthreads();
+    float dgc = 0.f;
+    if (tid < DK) {
+      for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDK + tid]);
+      dgc += __expf(Gg[63 * DK + tid]) * sSS[tid];
     }
-    float d = sdG[tid] + rs - cs - sTj[tid];
-    if (tid == 63) d += tot + __expf(gl) * sMisc[0];
-    wsp<float>(p, p.off.dG)[slot * 64 + tid] = d;
+    __syncthreads();
+    pair_col<T, DK, false>(sOut, sR, sAl, LDF, sQr, LDK, p.scale, tid);
+    __syncthreads();
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
+    for (int idx = tid; idx < 64 * DK; idx += 256) {
+      const int r = idx / DK, c = idx % DK;
+      const float v = sOut[r * LDF + c];
+      if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(v);
+      dGg[idx] -= to_f32(sKr[r * LDK + c]) * v;
+    }
+    __syncthreads();
+    if (tid < DK) dGg[63 * DK + tid] += dgc;
+  } else {
+    // ---- scalar / no gate ----
+    T* sPe = sdO;
+    T* sPeT = sD;
+    T* sKT = sSn;
+    T* sQT = sdSn;
+    // dP -> dPe = scale E dP (both orientations) and R = dP * P for the gate gradient
+    {
+      const T* Pg = wsp<T>(p, p.off.P) + slot * 64 * 64;
+      floatx16 pe[1][1];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+        const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+        const float dp = (i >= j) ? aP[0][0][e] : 0.f;
+        pe[0][0][e] = p.scale * dec * dp;
+        if (GATE != LNX_GATE_NONE) sR[i * LNX_LDA + j] = dp * to_f32(Pg[i * 64 + j]);
+      }
+      frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
+      frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+    }
+    // inter-chunk parts: dq = scale e^{G_i} dQg,  dk = r_j dKr, and their gate terms
+    const float gl = sG[63];
+    if (GATE != LNX_GATE_NONE) {
+      frag_rowdot<MT>(aQ, r0, c0, lane, sdG, [&](int r, int c) {
+        return (r < len) ? p.scale * __expf(sG[r]) * to_f32(qg[(int64_t)r * DK + c]) : 0.f;
+      });
+      frag_rowdot<MT>(aK, r0, c0, lane, sTj, [&](int r, int c) {
+        return (r < len) ? __expf(fminf(gl - sG[r], 0.f)) * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
+      });
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = r0 + 32 * i + frag_row(e, lane);
+        const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
+        const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
+        aQ[i][0][e] *= gq;
+        aK[i][0][e] *= gk;
+      }
+    stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
+    stage_rows_t<T>(sQT, LDC, qg, DK, 64, len, DK, tid, UnitScale());
+    __syncthreads();
+    // intra-chunk parts: dq += dPe K,  dk += dPe^T Q
+    mma_nt<T, MT, 1>(aQ, sPe + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
+    mma_nt<T, MT, 1>(aK, sPeT + r0 * LDC, LDC, sQT + c0 * LDC, LDC, 64, lane);
+    frag_store<T, MT, 1>(aQ, reinterpret_cast<T*>(p.dq) + (tbase + r0) * DK + c0, DK, lane, len - r0);
+    frag_store<T, MT, 1>(aK, reinterpret_cast<T*>(p.dk) + (tbase + r0) * DK + c0, DK, lane, len - r0);
+    // partial gate gradient wrt the cumulative gate G (row t); the chunk-end terms go to row 63
+    if (GATE != LNX_GATE_NONE && tid < 64) {
+      float rs = 0.f, cs = 0.f, tot = 0.f;
+      for (int j = 0; j < 64; ++j) {
+        rs += sR[tid * LNX_LDA + j];
+        cs += sR[j * LNX_LDA + tid];
+        tot += sTj[j];
+      }
+      float d = sdG[tid] + rs - cs - sTj[tid];
+      if (tid == 63) d += tot + __expf(gl) * sMisc[0];
+      wsp<float>(p, p.off.dG)[slot * 64 + tid] = d;
+    }
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // bwd_wy
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct WyCfg {
+template <typename T, int DK, int GATE> struct WyCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD;
-  static constexpr int kR1 = 64 * LDC;                                   // Tm^T, later Y
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
+  static constexpr int kR1 = 64 * LDC;                                       // Tm^T, later Y
   static constexpr int kR2 = (128 * LDC > 64 * LDK) ? 128 * LDC : 64 * LDK;  // dW^T | dD^T + dBu | dBw | K^T
-  static constexpr int kR3 = 64 * LDK;                                   // U slab | W | K
-  static constexpr size_t bytes = sizeof(T) * (kR1 + kR2 + kR3) + sizeof(float) * (64 * LNX_LDA + 64 * 4);
+  static constexpr int kR3 = 64 * LDK;                                       // U slab | W | K
+  static constexpr size_t mma_bytes = sizeof(T) * (kR1 + kR2 + kR3);
+  static constexpr size_t vec_bytes = sizeof(float) * 3 * 64 * LDF + sizeof(T) * 64 * LDK;  // alpha, out+, out-, K
+  static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > mma_bytes) ? vec_bytes : mma_bytes;
+  static constexpr size_t bytes = sizeof(float) * (64 * LNX_LDA + 64 * 4) + big;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
-  typedef WyCfg<T, DK> L;
+  typedef WyCfg<T, DK, GATE> L;
   typedef RowTiles<DK> RTl;
-  constexpr int LDK = L::LDK, LDC = L::LDC, MT = RTl::MT;
+  constexpr int LDK = L::LDK, LDC = L::LDC, LDF = L::LDF, MT = RTl::MT;
   extern __shared__ __align__(16) char smem[];
-  T* R1 = reinterpret_cast<T*>(smem);
-  T* R2 = R1 + L::kR1;
-  T* R3 = R2 + L::kR2;
-  float* sR = reinterpret_cast<float*>(R3 + L::kR3);  // [64][LNX_LDA]: dA * X
+  float* sR = reinterpret_cast<float*>(smem);  // [64][LNX_LDA]: dA * X (scalar) or dA, then beta dA (vector)
   float* sG = sR + 64 * LNX_LDA;
   float* sBeta = sG + 64;
   float* sdB = sBeta + 64;  // dbeta accumulator
   float* sdG = sdB + 64;    // gate-gradient accumulator (wrt cumulative G)
+  T* R1 = reinterpret_cast<T*>(sdG + 64);
+  T* R2 = R1 + L::kR1;
+  T* R3 = R2 + L::kR2;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -443,7 +529,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
 
   if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_NONE) ? 0.f : wsp<float>(p, p.off.G)[slot * 64 + tid];
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
     sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
     sdB[tid] = 0.f;
     sdG[tid] = 0.f;
@@ -493,80 +579,148 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
   __syncthreads();
 
-  // phase 4: X = K K^T (recomputed), dA = -tril(dM, -1), Y = sym(beta dA E), R = dA * E X
-  T* sK = R3;
-  T* sY = R1;
-  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
-  __syncthreads();
-  {
-    floatx16 x[1][1];
-    frag_zero(x);
-    if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(x, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+  if constexpr (GATE == LNX_GATE_VECTOR) {
+    // ---- per-channel gate ----
+    float* sAl = reinterpret_cast<float*>(R1);  // [64][LDF]
+    float* sOp = sAl + 64 * LDF;                // row-type part of dk (through B_w and the rows of X)
+    float* sOm = sOp + 64 * LDF;                // column-type part of dk (columns of X)
+    T* sKr = reinterpret_cast<T*>(sOm + 64 * LDF);
+    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
+    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
+    const T* Xg = wsp<T>(p, p.off.X) + slot * 64 * 64;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      const float da = (i > j) ? -aM[0][0][e] : 0.f;
-      sR[i * LNX_LDA + j] = da * dec * x[0][0][e];
-      const T y = from_f32<T>(sBeta[i] * da * dec);
-      if (i > j) {
-        sY[i * LDC + j] = y;
-        sY[j * LDC + i] = y;
-      } else if (i == j) {
-        sY[i * LDC + j] = from_f32<T>(0.f);
-      }
+      sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
     }
-  }
-  // dk (row-type part through B_w): beta e^{G} dBw, with its dbeta / gate terms
-  frag_rowdot<MT>(aBw, r0, c0, lane, sdG, [&](int r, int c) {
-    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
-    return (r < len) ? gm * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
-  });
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = r0 + 32 * i + frag_row(e, lane);
-      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
-      aBw[i][0][e] *= sBeta[r] * gm;
+    stage_rows<T>(sKr, LDK, kg, DK, 64, len, DK, tid);
+    for (int idx = tid; idx < 64 * DK; idx += 256) {
+      const int r = idx / DK, c = idx % DK;
+      const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
+      sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
+      sOm[r * LDF + c] = 0.f;
     }
-  __syncthreads();  // sdBw (R2) no longer read; sY, sR complete
-
-  // phase 5: dk += Y K, added to the partial dk of bwd_dqk
-  T* sKT = R2;
-  stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
-  __syncthreads();
-  mma_nt<T, MT, 1>(aBw, sY + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
-  {
-    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
-        if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + aBw[i][0][e]);
+        sOp[r * LDF + c] = aBw[i][0][e] * __expf(Gg[r * DK + c]);  // e^G dBw
       }
-  }
-  // dbeta and dg
-  if (wave == 0) {
-    const int t = lane;
-    float rs = 0.f, cs = 0.f;
-    for (int j = 0; j < 64; ++j) {
-      rs += sR[t * LNX_LDA + j];
-      cs += sBeta[j] * sR[j * LNX_LDA + t];
+    __syncthreads();
+    if (tid < 64) {  // dbeta += sum_j dA_ij X_ij
+      float rs = 0.f;
+      for (int j = 0; j < tid; ++j) rs += sR[tid * LNX_LDA + j] * to_f32(Xg[tid * 64 + j]);
+      atomicAdd(&sdB[tid], rs);
     }
-    // sdG[t] holds e^{G_t} <dBw_t, k_t>
-    const float w = sdG[t];
-    if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
-    if (GATE != LNX_GATE_NONE) {
-      float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - cs;
-      // reverse inclusive cumsum over the chunk
-#pragma unroll
-      for (int s = 1; s < 64; s <<= 1) {
-        const float y = __shfl_down(d, s, LNX_WAVE);
-        if (t + s < 64) d += y;
+    for (int r = wave; r < 64; r += 4) {  // dbeta += <e^G dBw, k>;  out+ = beta e^G dBw
+      float t = 0.f;
+      for (int c = lane; c < DK; c += 64) {
+        t += sOp[r * LDF + c] * to_f32(sKr[r * LDK + c]);
+        sOp[r * LDF + c] *= sBeta[r];
       }
-      if (t < len) p.dg[tbase + t] = d;
+      t = wave_sum(t);
+      if (lane == 0) atomicAdd(&sdB[r], t);
+    }
+    __syncthreads();
+    for (int idx = tid; idx < 64 * 64; idx += 256) sR[(idx >> 6) * LNX_LDA + (idx & 63)] *= sBeta[idx >> 6];  // dX
+    __syncthreads();
+    pair_row<T, DK, true>(sOp, sR, sAl, LDF, sKr, LDK, 1.f, tid);
+    pair_col<T, DK, true>(sOm, sR, sAl, LDF, sKr, LDK, 1.f, tid);
+    __syncthreads();
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
+    for (int idx = tid; idx < 64 * DK; idx += 256) {
+      const int r = idx / DK, c = idx % DK;
+      const float up = sOp[r * LDF + c], um = sOm[r * LDF + c];
+      if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + up + um);
+      dGg[idx] += to_f32(sKr[r * LDK + c]) * (up - um);
+    }
+    __syncthreads();
+    if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
+    if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
+      float acc = 0.f;
+      for (int r = 63; r >= 0; --r) {
+        acc += dGg[r * DK + tid];
+        if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
+      }
+    }
+  } else {
+    // ---- scalar / no gate ----
+    // phase 4: X = K K^T (recomputed), dA = -tril(dM, -1), Y = sym(beta dA E), R = dA * E X
+    T* sK = R3;
+    T* sY = R1;
+    stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
+    __syncthreads();
+    {
+      floatx16 x[1][1];
+      frag_zero(x);
+      if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(x, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+        const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+        const float da = (i > j) ? -aM[0][0][e] : 0.f;
+        sR[i * LNX_LDA + j] = da * dec * x[0][0][e];
+        const T y = from_f32<T>(sBeta[i] * da * dec);
+        if (i > j) {
+          sY[i * LDC + j] = y;
+          sY[j * LDC + i] = y;
+        } else if (i == j) {
+          sY[i * LDC + j] = from_f32<T>(0.f);
+        }
+      }
+    }
+    // dk (row-type part through B_w): beta e^{G} dBw, with its dbeta / gate terms
+    frag_rowdot<MT>(aBw, r0, c0, lane, sdG, [&](int r, int c) {
+      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
+      return (r < len) ? gm * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
+    });
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = r0 + 32 * i + frag_row(e, lane);
+        const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
+        aBw[i][0][e] *= sBeta[r] * gm;
+      }
+    __syncthreads();  // sdBw (R2) no longer read; sY, sR complete
+
+    // phase 5: dk += Y K, added to the partial dk of bwd_dqk
+    T* sKT = R2;
+    stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
+    __syncthreads();
+    mma_nt<T, MT, 1>(aBw, sY + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
+    {
+      T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
+          if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + aBw[i][0][e]);
+        }
+    }
+    // dbeta and dg
+    if (wave == 0) {
+      const int t = lane;
+      float rs = 0.f, cs = 0.f;
+      for (int j = 0; j < 64; ++j) {
+        rs += sR[t * LNX_LDA + j];
+        cs += sBeta[j] * sR[j * LNX_LDA + t];
+      }
+      // sdG[t] holds e^{G_t} <dBw_t, k_t>
+      const float w = sdG[t];
+      if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
+      if (GATE != LNX_GATE_NONE) {
+        float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - cs;
+        // reverse inclusive cumsum over the chunk
+#pragma unroll
+        for (int s_ = 1; s_ < 64; s_ <<= 1) {
+          const float y = __shfl_down(d, s_, LNX_WAVE);
+          if (t + s_ < 64) d += y;
+        }
+        if (t < len) p.dg[tbase + t] = d;
+      }
     }
   }
 }
@@ -577,7 +731,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   auto k1 = bwd_scan_kernel<T, DK, GATE>;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
   auto k3 = bwd_wy_kernel<T, DK, GATE>;
-  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK>::bytes, b3 = WyCfg<T, DK>::bytes;
+  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = WyCfg<T, DK, GATE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
@@ -600,7 +754,8 @@ int launch_bwd_gate(int gate, const BwdParams& p, int nstate, hipStream_t st) {
   switch (gate) {
     case LNX_GATE_NONE: return launch_bwd<T, DK, LNX_GATE_NONE>(p, nstate, st);
     case LNX_GATE_SCALAR: return launch_bwd<T, DK, LNX_GATE_SCALAR>(p, nstate, st);
-    default: return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels: gate kind %d is not supported yet", gate);
+    case LNX_GATE_VECTOR: return launch_bwd<T, DK, LNX_GATE_VECTOR>(p, nstate, st);
+    default: return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", gate);
   }
 }
 
