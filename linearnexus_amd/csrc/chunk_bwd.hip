@@ -29,7 +29,7 @@ struct BwdParams {
   float* dbeta;
   float* dg;
   float* ds0;
-  int dv;
+  int dv, gate;
   float scale;
   char* ws;
   ChunkWs off;
@@ -52,16 +52,13 @@ template <int DK> struct RowTiles {
 template <int MT, typename F>
 __device__ __forceinline__ void frag_rowdot(const floatx16 (&acc)[MT][1], int row0, int col0, int lane, float* rows,
                                             F partner) {
+  float v[16 * MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = row0 + 32 * i + frag_row(e, lane), c = col0 + frag_col(lane);
-      float s = acc[i][0][e] * partner(r, c);
-#pragma unroll
-      for (int m = 1; m < 32; m <<= 1) s += __shfl_xor(s, m, LNX_WAVE);
-      if ((lane & 31) == 0) atomicAdd(&rows[r], s);
-    }
+    for (int e = 0; e < 16; ++e)
+      v[16 * i + e] = acc[i][0][e] * partner(row0 + 32 * i + frag_row(e, lane), col0 + frag_col(lane));
+  rows_reduce_add<MT>(v, row0, lane, rows);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -81,10 +78,11 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-  stage_rows_t<T>(sPT, LDC, wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, 64, 64, tid, UnitScale());
-  stage_rows_t<T>(sdOT, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, 64, len, 64, tid, UnitScale());
+  if (v0 == 0 && tid < 64 && p.gate == LNX_GATE_SCALAR) wsp<float>(p, p.off.dG)[slot * 64 + tid] = 0.f;  // accumulated by bwd_dqk
+  stage_tile_t<T, 64, 64>(sPT, LDC, wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
+  stage_tile_t<T, 64, 64>(sdOT, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
   __syncthreads();
-  unstage_rows<T>(wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdOT, LDC, 64, 64, tid);
+  unstage_tile<T, 64, 64>(wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdOT, LDC, 64, tid);
   const int wi = wave >> 1, wj = wave & 1;
   floatx16 acc[1][1];
   frag_zero(acc);
@@ -263,224 +261,247 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
-// bwd_dqk
+// bwd_dqk: one workgroup per (chunk, 64-channel half of dk).  Loop over 64-column slabs of dv
+// with the next slab prefetched into registers; every product is one 32x32 tile per wave.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK, int GATE> struct DqkCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
-  // loop phase: dO, D, dD slabs [64][LDC] and S_n, dS_n slabs [DK][LDC]
-  // epilogue (scalar / no gate): dPe, dPe^T [64][LDC] and K^T, Q^T [DK][LDC] overlaid on the slabs
-  // epilogue (vector gate): alpha, out [64][LDF] fp32 and K, Q [64][LDK] overlaid on the slabs
-  static constexpr int kTile = 64 * LDC, kWide = DK * LDC;
-  static constexpr size_t loop_bytes = sizeof(T) * (3 * kTile + 2 * kWide);
-  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 2 * 64 * LDK;
+  static constexpr int LDC = LNX_C + PAD, LDF = 64 + 4;
+  static constexpr int kTile = 64 * LDC;
+  // loop phase: dO, D, dD, S_n, dS_n tiles; scalar epilogue: dPe, dPe^T, K^T, Q^T + one staging tile
+  static constexpr size_t loop_bytes = sizeof(T) * 5 * kTile;
+  // vector epilogue: alpha, out (fp32 [64][LDF]) and K, Q rows, plus dP in fp32
+  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 2 * kTile;
   static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > loop_bytes) ? vec_bytes : loop_bytes;
-  static constexpr int kSmall = 64 * LNX_LDA + 64 * 4 + DK;  // floats: sR, sG, sdG, sTj, sMisc, sSS
+  static constexpr int kSmall = 64 * 4 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0);  // floats
   static constexpr size_t bytes = sizeof(float) * kSmall + big;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
   typedef DqkCfg<T, DK, GATE> L;
-  typedef RowTiles<DK> RTl;
-  constexpr int LDC = L::LDC, LDK = L::LDK, LDF = L::LDF, MT = RTl::MT;
+  constexpr int LDC = L::LDC, LDF = L::LDF;
   extern __shared__ __align__(16) char smem[];
-  float* sR = reinterpret_cast<float*>(smem);  // [64][LNX_LDA]
-  float* sG = sR + 64 * LNX_LDA;
+  float* sG = reinterpret_cast<float*>(smem);
   float* sdG = sG + 64;     // per-row gate-gradient accumulator
-  float* sTj = sdG + 64;    // r_j <dKr_j, k_j>
-  float* sMisc = sTj + 64;  // [0] = <dS_n, S_n>
-  float* sSS = sMisc + 64;  // [DK] per key channel: sum_v dS_n[c][v] S_n[c][v]   (vector gate)
-  T* sdO = reinterpret_cast<T*>(sSS + DK);
+  float* sSS = sdG + 64;    // vector gate: per key channel sum_v dS_n[c][v] S_n[c][v]
+  float* sMisc = sSS + 64;  // [0] = sum_j r_j <dKr_j, k_j>, [1] = <dS_n, S_n>
+  float* sR = sMisc + 64;   // vector gate only: dP [64][LNX_LDA]
+  T* sdO = reinterpret_cast<T*>(sMisc + 64 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0));
   T* sD = sdO + L::kTile;
   T* sdD = sD + L::kTile;
   T* sSn = sdD + L::kTile;
-  T* sdSn = sSn + L::kWide;
+  T* sdSn = sSn + L::kTile;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
   const int64_t slot = blockIdx.x;
+  const int ch0 = blockIdx.y * 64;  // first key channel of this half
   const int row = (int)(slot / N), n = (int)(slot % N);
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
-  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK + ch0;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK + ch0;
   const int wi = wave >> 1, wj = wave & 1;
-  const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
 
   if (tid < 64) {
     sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
     sdG[tid] = 0.f;
-    sTj[tid] = 0.f;
-    if (tid == 0) sMisc[0] = 0.f;
+    sSS[tid] = 0.f;
+    sMisc[tid] = 0.f;
   }
-  if (tid < DK) sSS[tid] = 0.f;
 
-  floatx16 aP[1][1], aQ[MT][1], aW[MT][1], aK[MT][1];
+  TileRegs<T, 64, 64> rdO, rD, rdD, rdSn;
+  TileRegsT<T, 64, 64> rSn;
+  auto fetch = [&](int v0) {
+    rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
+    rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+    rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+    rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, 64, tid);
+    rdSn.load(wsp<T>(p, p.off.dSn) + slot * DK * p.dv + (int64_t)ch0 * p.dv + v0, p.dv, 64, tid);
+  };
+  floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
   frag_zero(aP);
   frag_zero(aQ);
   frag_zero(aW);
   frag_zero(aK);
-  float ss = 0.f;  // partial <dS_n, S_n>
+  float ss = 0.f;
+  fetch(0);
   for (int v0 = 0; v0 < p.dv; v0 += 64) {
     __syncthreads();
-    stage_rows<T>(sdO, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, 64, len, 64, tid);
-    stage_rows<T>(sD, LDC, wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
-    stage_rows<T>(sdD, LDC, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
-    stage_rows_t<T>(sSn, LDC, wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, 64, 64, DK, tid, UnitScale());
-    stage_rows<T>(sdSn, LDC, wsp<T>(p, p.off.dSn) + slot * DK * p.dv + v0, p.dv, DK, DK, 64, tid);
+    rdO.store(sdO, LDC, tid);
+    rD.store(sD, LDC, tid);
+    rdD.store(sdD, LDC, tid);
+    rSn.store(sSn, LDC, tid);
+    rdSn.store(sdSn, LDC, tid);
     __syncthreads();
+    if (v0 + 64 < p.dv) fetch(v0 + 64);
     mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDC, LDC, sD + 32 * wj * LDC, LDC, 64, lane);
-    mma_nt<T, MT, 1>(aQ, sdO + r0 * LDC, LDC, sSn + c0 * LDC, LDC, 64, lane);
-    mma_nt<T, MT, 1>(aW, sdD + r0 * LDC, LDC, sSn + c0 * LDC, LDC, 64, lane);
-    mma_nt<T, MT, 1>(aK, sD + r0 * LDC, LDC, sdSn + c0 * LDC, LDC, 64, lane);
-    if (GATE != LNX_GATE_NONE)
-      for (int r = wave; r < DK; r += 4) {  // one key channel per wavefront, lanes over the slab
-        const float t = wave_sum(to_f32(sSn[r * LDC + lane]) * to_f32(sdSn[r * LDC + lane]));
-        if (GATE == LNX_GATE_VECTOR) { if (lane == 0) sSS[r] += t; }
-        else ss += t;
+    mma_nt<T, 1, 1>(aQ, sdO + 32 * wi * LDC, LDC, sSn + 32 * wj * LDC, LDC, 64, lane);
+    mma_nt<T, 1, 1>(aW, sdD + 32 * wi * LDC, LDC, sSn + 32 * wj * LDC, LDC, 64, lane);
+    mma_nt<T, 1, 1>(aK, sD + 32 * wi * LDC, LDC, sdSn + 32 * wj * LDC, LDC, 64, lane);
+    if (GATE != LNX_GATE_NONE) {  // thread = (channel row tid / 4, quarter of the slab)
+      const int r = tid >> 2, q4 = (tid & 3) * 16;
+      float t = 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; e += 4) {
+        const floatx4 x = load4(sSn + r * LDC + q4 + e), y = load4(sdSn + r * LDC + q4 + e);
+        t += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
       }
+      ss += t;
+    }
   }
-  if (GATE == LNX_GATE_SCALAR && lane == 0) atomicAdd(&sMisc[0], ss);
-  __syncthreads();  // slabs are dead from here on; sG, sdG initialised
-
-  // dW = -dD S_n^T to the workspace
-  {
-    floatx16 t[MT][1];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) t[i][0][e] = -aW[i][0][e];
-    frag_store<T, MT, 1>(t, wsp<T>(p, p.off.dW) + slot * 64 * DK + (int64_t)r0 * DK + c0, DK, lane);
+  if (GATE == LNX_GATE_VECTOR) {
+    ss += __shfl_xor(ss, 1, LNX_WAVE);
+    ss += __shfl_xor(ss, 2, LNX_WAVE);
+    if ((tid & 3) == 0) sSS[tid >> 2] = ss;
+  } else if (GATE == LNX_GATE_SCALAR) {
+    ss = wave_sum(ss);
+    if (lane == 0) atomicAdd(&sMisc[1], ss);
   }
+  __syncthreads();  // slab tiles are dead from here on
 
   if constexpr (GATE == LNX_GATE_VECTOR) {
-    // ---- per-channel gate: element-wise decays, pair terms on the VALU ----
-    float* sAl = reinterpret_cast<float*>(sdO);  // [64][LDF] alpha_j[c] = exp(g_j[c])
-    float* sOut = sAl + 64 * LDF;                // [64][LDF]
-    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDK]
-    T* sQr = sKr + 64 * LDK;                         // Q rows
-    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
-    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
+    // ---- per-channel gate: element-wise decays, pair terms on the VALU (64 channels) ----
+    float* sAl = reinterpret_cast<float*>(sdO);      // [64][LDF] alpha_j[c] = exp(g_j[c])
+    float* sOut = sAl + 64 * LDF;                    // [64][LDF]
+    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC] (this half's channels)
+    T* sQr = sKr + L::kTile;
+    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK + ch0;
+    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK + ch0;
+    TileRegs<T, 64, 64> rk, rq;
+    rk.load(kg, DK, len, tid);
+    rq.load(qg, DK, len, tid);
+    // dW half through sOut (fp32) -> global
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       sR[i * LNX_LDA + j] = (i >= j) ? aP[0][0][e] : 0.f;
+      sOut[i * LDF + j] = -aW[0][0][e];
     }
-    stage_rows<T>(sKr, LDK, kg, DK, 64, len, DK, tid);
-    stage_rows<T>(sQr, LDK, qg, DK, 64, len, DK, tid);
-    for (int idx = tid; idx < 64 * DK; idx += 256) {
-      const int r = idx / DK, c = idx % DK;
+    rk.store(sKr, LDC, tid);
+    rq.store(sQr, LDC, tid);
+    for (int idx = tid; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
       const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
       sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
     }
-    // dq = scale e^G dQg (+ intra-chunk part)
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
-        sOut[r * LDF + c] = aQ[i][0][e] * p.scale * __expf(Gg[r * DK + c]);
+    __syncthreads();
+    {
+      T* dWg = wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0;
+      for (int idx = tid; idx < 64 * 16; idx += 256) {
+        const int r = idx >> 4, c = (idx & 15) * 4;
+        store4(dWg + (int64_t)r * DK + c, load4(sOut + r * LDF + c));
       }
-    __syncthreads();
-    pair_row<T, DK, false>(sOut, sR, sAl, LDF, sKr, LDK, p.scale, tid);
-    __syncthreads();
-    T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK;
-    for (int idx = tid; idx < 64 * DK; idx += 256) {
-      const int r = idx / DK, c = idx % DK;
-      const float v = sOut[r * LDF + c];
-      if (r < len) dqg[(int64_t)r * DK + c] = from_f32<T>(v);
-      dGg[idx] = to_f32(sQr[r * LDK + c]) * v;
     }
     __syncthreads();
-    // dk (column-type parts): e^{G_last - G} dKr (+ P part); chunk-end gate term from the Kr part
+    // dq = scale e^G dQg + intra-chunk part
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+      sOut[r * LDF + c] = aQ[0][0][e] * p.scale * __expf(Gg[r * DK + c]);
+    }
+    __syncthreads();
+    pair_row<T, 64, false>(sOut, sR, sAl, LDF, sKr, LDC, p.scale, tid);
+    __syncthreads();
+    T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK + ch0;
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int r = idx >> 4, c = (idx & 15) * 4;
+      const floatx4 v = load4(sOut + r * LDF + c), qq = load4(sQr + r * LDC + c);
+      if (r < len) store4(dqg + (int64_t)r * DK + c, v);
+      store4(dGg + r * DK + c, qq * v);
+    }
+    __syncthreads();
+    // dk (column-type parts): e^{G_last - G} dKr + P part; chunk-end gate term from the Kr part
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
-        sOut[r * LDF + c] = aK[i][0][e] * __expf(fminf(Gg[63 * DK + c] - Gg[r * DK + c], 0.f));
-      }
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+      sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(Gg[63 * DK + c] - Gg[r * DK + c], 0.f));
+    }
     __syncthreads();
     float dgc = 0.f;
-    if (tid < DK) {
-      for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDK + tid]);
+    if (tid < 64) {
+      for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDC + tid]);
       dgc += __expf(Gg[63 * DK + tid]) * sSS[tid];
     }
     __syncthreads();
-    pair_col<T, DK, false>(sOut, sR, sAl, LDF, sQr, LDK, p.scale, tid);
+    pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
     __syncthreads();
-    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
-    for (int idx = tid; idx < 64 * DK; idx += 256) {
-      const int r = idx / DK, c = idx % DK;
-      const float v = sOut[r * LDF + c];
-      if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(v);
-      dGg[idx] -= to_f32(sKr[r * LDK + c]) * v;
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + ch0;
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int r = idx >> 4, c = (idx & 15) * 4;
+      const floatx4 v = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
+      if (r < len) store4(dkg + (int64_t)r * DK + c, v);
+      store4(dGg + r * DK + c, load4(dGg + r * DK + c) - kk * v);
     }
     __syncthreads();
-    if (tid < DK) dGg[63 * DK + tid] += dgc;
+    if (tid < 64) dGg[63 * DK + tid] += dgc;
   } else {
     // ---- scalar / no gate ----
     T* sPe = sdO;
     T* sPeT = sD;
-    T* sKT = sSn;
-    T* sQT = sdSn;
-    // dP -> dPe = scale E dP (both orientations) and R = dP * P for the gate gradient
+    T* sKT = sdD;
+    T* sQT = sSn;
+    T* sOut = sdSn;
+    TileRegs<T, 64, 64> rKT;
+    TileRegsT<T, 64, 64> rQT;
+    rKT.load(wsp<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)ch0 * 64, 64, 64, tid);
+    rQT.load(qg, DK, len, tid);
     {
-      const T* Pg = wsp<T>(p, p.off.P) + slot * 64 * 64;
-      floatx16 pe[1][1];
+      floatx16 pe[1][1], nw[1][1];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
         const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-        const float dp = (i >= j) ? aP[0][0][e] : 0.f;
-        pe[0][0][e] = p.scale * dec * dp;
-        if (GATE != LNX_GATE_NONE) sR[i * LNX_LDA + j] = dp * to_f32(Pg[i * 64 + j]);
+        pe[0][0][e] = (i >= j) ? p.scale * dec * aP[0][0][e] : 0.f;
+        nw[0][0][e] = -aW[0][0][e];
       }
       frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
       frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+      frag_store<T, 1, 1>(nw, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
     }
-    // inter-chunk parts: dq = scale e^{G_i} dQg,  dk = r_j dKr, and their gate terms
+    rKT.store(sKT, LDC, tid);
+    rQT.store(sQT, LDC, tid);
+    __syncthreads();
+    unstage_tile<T, 64, 64>(wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0, DK, sOut, LDC, 64, tid);
+    // inter-chunk parts scaled, then the intra-chunk products on top
     const float gl = sG[63];
-    if (GATE != LNX_GATE_NONE) {
-      frag_rowdot<MT>(aQ, r0, c0, lane, sdG, [&](int r, int c) {
-        return (r < len) ? p.scale * __expf(sG[r]) * to_f32(qg[(int64_t)r * DK + c]) : 0.f;
-      });
-      frag_rowdot<MT>(aK, r0, c0, lane, sTj, [&](int r, int c) {
-        return (r < len) ? __expf(fminf(gl - sG[r], 0.f)) * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
-      });
-    }
+    float tot = 0.f;
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+      const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
+      const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
+      aQ[0][0][e] *= gq;
+      aK[0][0][e] *= gk;
+      tot += aK[0][0][e] * to_f32(sKT[c * LDC + r]);
+    }
+    mma_nt<T, 1, 1>(aQ, sPe + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
+    mma_nt<T, 1, 1>(aK, sPeT + 32 * wi * LDC, LDC, sQT + 32 * wj * LDC, LDC, 64, lane);
+    if (GATE != LNX_GATE_NONE) {
+      // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts)
+      float v[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int r = r0 + 32 * i + frag_row(e, lane);
-        const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
-        const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
-        aQ[i][0][e] *= gq;
-        aK[i][0][e] *= gk;
+        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+        v[e] = aQ[0][0][e] * to_f32(sQT[c * LDC + r]) - aK[0][0][e] * to_f32(sKT[c * LDC + r]);
       }
-    stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
-    stage_rows_t<T>(sQT, LDC, qg, DK, 64, len, DK, tid, UnitScale());
+      rows_reduce_add<1>(v, 32 * wi, lane, sdG);
+      tot = wave_sum(tot);
+      if (lane == 0) atomicAdd(&sMisc[0], tot);
+    }
+    __syncthreads();  // all reads of sPe / sPeT / sOut done
+    frag_store<T, 1, 1>(aQ, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store<T, 1, 1>(aK, sPeT + 32 * wi * LDC + 32 * wj, LDC, lane);
     __syncthreads();
-    // intra-chunk parts: dq += dPe K,  dk += dPe^T Q
-    mma_nt<T, MT, 1>(aQ, sPe + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
-    mma_nt<T, MT, 1>(aK, sPeT + r0 * LDC, LDC, sQT + c0 * LDC, LDC, 64, lane);
-    frag_store<T, MT, 1>(aQ, reinterpret_cast<T*>(p.dq) + (tbase + r0) * DK + c0, DK, lane, len - r0);
-    frag_store<T, MT, 1>(aK, reinterpret_cast<T*>(p.dk) + (tbase + r0) * DK + c0, DK, lane, len - r0);
-    // partial gate gradient wrt the cumulative gate G (row t); the chunk-end terms go to row 63
+    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, DK, sPe, LDC, len, tid);
+    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sPeT, LDC, len, tid);
     if (GATE != LNX_GATE_NONE && tid < 64) {
-      float rs = 0.f, cs = 0.f, tot = 0.f;
-      for (int j = 0; j < 64; ++j) {
-        rs += sR[tid * LNX_LDA + j];
-        cs += sR[j * LNX_LDA + tid];
-        tot += sTj[j];
-      }
-      float d = sdG[tid] + rs - cs - sTj[tid];
-      if (tid == 63) d += tot + __expf(gl) * sMisc[0];
-      wsp<float>(p, p.off.dG)[slot * 64 + tid] = d;
+      float d = sdG[tid];
+      if (tid == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
+      atomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + tid], d);
     }
   }
 }
@@ -537,8 +558,8 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   // phase 1: dBw = Tm^T dW
   T* sTmT = R1;
   T* sdWT = R2;
-  stage_rows<T>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, 64, 64, tid);
-  stage_rows_t<T>(sdWT, LDC, wsp<T>(p, p.off.dW) + slot * 64 * DK, DK, 64, 64, DK, tid, UnitScale());
+  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
+  stage_tile_t<T, 64, DK>(sdWT, LDC, wsp<T>(p, p.off.dW) + slot * 64 * DK, DK, 64, tid);
   __syncthreads();
   floatx16 aBw[MT][1], aM[1][1];
   frag_zero(aBw);
@@ -551,8 +572,8 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   T* sU = R3;
   for (int v0 = 0; v0 < p.dv; v0 += 64) {
     __syncthreads();
-    stage_rows<T>(sdDT, LDC, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, 64, 64, tid);
-    stage_rows<T>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, 64, 64, tid);
+    stage_tile<T, 64, 64>(sdDT, LDC, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, tid);
+    stage_tile<T, 64, 64>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     __syncthreads();
     floatx16 bu[1][1];
     frag_zero(bu);
@@ -574,7 +595,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   T* sdBw = R2;
   T* sW = R3;
   frag_store<T, MT, 1>(aBw, sdBw + r0 * LDK + c0, LDK, lane);
-  stage_rows<T>(sW, LDK, wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, 64, DK, tid);
+  stage_tile<T, 64, DK>(sW, LDK, wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
   __syncthreads();
   mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
   __syncthreads();
@@ -593,7 +614,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
     }
-    stage_rows<T>(sKr, LDK, kg, DK, 64, len, DK, tid);
+    stage_tile<T, 64, DK>(sKr, LDK, kg, DK, len, tid);
     for (int idx = tid; idx < 64 * DK; idx += 256) {
       const int r = idx / DK, c = idx % DK;
       const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
@@ -649,7 +670,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     // phase 4: X = K K^T (recomputed), dA = -tril(dM, -1), Y = sym(beta dA E), R = dA * E X
     T* sK = R3;
     T* sY = R1;
-    stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
+    stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
     __syncthreads();
     {
       floatx16 x[1][1];
@@ -687,7 +708,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
 
     // phase 5: dk += Y K, added to the partial dk of bwd_dqk
     T* sKT = R2;
-    stage_rows<T>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, DK, 64, tid);
+    stage_tile<T, DK, 64>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, tid);
     __syncthreads();
     mma_nt<T, MT, 1>(aBw, sY + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
     {
@@ -742,7 +763,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("bwd_scan", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(256), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
-  hipLaunchKernelGGL(k2, dim3((unsigned)slots), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)slots, (unsigned)(DK / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("bwd_wy", st);
   hipLaunchKernelGGL(k3, dim3((unsigned)slots), dim3(256), b3, st, p);
   lnx_profile_mark(nullptr, st);
@@ -792,7 +813,7 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.d_o = a->d_o; p.d_sT = a->d_final_state;
   p.dq = a->d_q; p.dk = a->d_k; p.dv_out = a->d_v; p.dbeta = a->d_beta; p.dg = a->d_g; p.ds0 = a->d_initial_state;
-  p.dv = a->dv; p.scale = a->scale;
+  p.dv = a->dv; p.gate = a->gate; p.scale = a->scale;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);

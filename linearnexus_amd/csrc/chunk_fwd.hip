@@ -87,9 +87,9 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
 
-  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
-  stage_rows_t<T>(sKT, LDC, kg, DK, 64, len, DK, tid, UnitScale());
-  stage_rows<T>(sQ, LDK, qg, DK, 64, len, DK, tid);
+  stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
+  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid);
+  stage_tile<T, 64, DK>(sQ, LDK, qg, DK, len, tid);
   if (wave == 0) {
     const bool ok = lane < len;
     sBeta[lane] = ok ? p.beta[tbase + lane] : 0.f;
@@ -122,11 +122,11 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
   }
   __syncthreads();
   // (scale * Q * e^G)^T for the backward scan, staged through the sQ region
-  stage_rows_t<T>(sQ, LDC, qg, DK, 64, len, DK, tid, [&](int r) {
+  stage_tile_t<T, 64, DK>(sQ, LDC, qg, DK, len, tid, [&](int r, int) {
     return (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
   });
   tri_inverse_64(sA, sT, sX, tid);
-  unstage_rows<T>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, 64, tid);
+  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, tid);
 
   // Tw = Tm * diag(beta e^G) (into the sK region), Tu = Tm * diag(beta) (into the sA region),
   // Tm^T to the workspace.
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
       frag_store_t<T, 1, 1>(acc, ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)(c0 + 32 * wj) * 64 + 32 * wi, 64, lane);
     }
     // K^T for the scan kernel
-    unstage_rows<T>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, 64, tid);
+    unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, tid);
   }
   // U = Tu V, one transposed 64-column slab of V at a time (slab overlays sQ)
   {
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
     T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
     for (int c0 = 0; c0 < p.dv; c0 += 64) {
       __syncthreads();
-      stage_rows_t<T>(sVT, LDC, vg + c0, p.dv, 64, len, 64, tid, UnitScale());
+      stage_tile_t<T, 64, 64>(sVT, LDC, vg + c0, p.dv, len, tid);
       __syncthreads();
       floatx16 acc[1][1];
       frag_zero(acc);
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
 
-  stage_rows<T>(sK, LDK, kg, DK, 64, len, DK, tid);
-  stage_rows<T>(sQ, LDK, qg, DK, 64, len, DK, tid);
+  stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
+  stage_tile<T, 64, DK>(sQ, LDK, qg, DK, len, tid);
   for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
     const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
     floatx4 x = {0.f, 0.f, 0.f, 0.f};
@@ -279,10 +279,9 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   }
   __syncthreads();
   // (scale * Q * e^G)^T through the sQ region
-  stage_rows_t_elem<T>(sQ, LDC, qg, DK, 64, len, DK, tid,
-                       [&](int r, int c) { return p.scale * __expf(sG[r * LDF + c]); });
+  stage_tile_t<T, 64, DK>(sQ, LDC, qg, DK, len, tid, [&](int r, int c) { return p.scale * __expf(sG[r * LDF + c]); });
   tri_inverse_64(sA, sT, sX, tid);
-  unstage_rows<T>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, 64, tid);
+  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, tid);
 
   T* sTm = sK;                         // T-typed copy of Tm (bf16); fp32 reads sT in place
   T* sTu = reinterpret_cast<T*>(sA);   // Tm * diag(beta)
@@ -300,8 +299,7 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   __syncthreads();
   // W = Tm (beta e^G K): transposed, scaled K through the sQ region
   T* sKT = sQ;
-  stage_rows_t_elem<T>(sKT, LDC, kg, DK, 64, len, DK, tid,
-                       [&](int r, int c) { return sBeta[r] * __expf(sG[r * LDF + c]); });
+  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid, [&](int r, int c) { return sBeta[r] * __expf(sG[r * LDF + c]); });
   __syncthreads();
   const int wi = wave >> 1, wj = wave & 1;
   {
@@ -316,17 +314,16 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   }
   __syncthreads();
   // (K * e^{G_last - G})^T for the scan kernel
-  stage_rows_t_elem<T>(sKT, LDC, kg, DK, 64, len, DK, tid,
-                       [&](int r, int c) { return __expf(fminf(sG[63 * LDF + c] - sG[r * LDF + c], 0.f)); });
+  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid, [&](int r, int c) { return __expf(fminf(sG[63 * LDF + c] - sG[r * LDF + c], 0.f)); });
   __syncthreads();
-  unstage_rows<T>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, 64, tid);
+  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, tid);
   // U = Tu V
   {
     T* sVT = sQ;
     T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
     for (int c0 = 0; c0 < p.dv; c0 += 64) {
       __syncthreads();
-      stage_rows_t<T>(sVT, LDC, vg + c0, p.dv, 64, len, 64, tid, UnitScale());
+      stage_tile_t<T, 64, 64>(sVT, LDC, vg + c0, p.dv, len, tid);
       __syncthreads();
       floatx16 acc[1][1];
       frag_zero(acc);
@@ -531,11 +528,11 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
       *reinterpret_cast<typename Vec16<T>::V*>(sQ + r * LDK + c) = x;
     }
   } else {
-    stage_rows<T>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, 64, len, DK, tid);
+    stage_tile<T, 64, DK>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, len, tid);
   }
-  stage_rows<T>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, BV, DK, tid);
-  stage_rows<T>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, 64, 64, tid);
-  stage_rows<T>(sDT, LDC, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, BV, BV, 64, tid);
+  stage_tile<T, BV, DK>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, tid);
+  stage_tile<T, 64, 64>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
+  stage_tile<T, BV, 64>(sDT, LDC, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, BV, tid);
   if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
   __syncthreads();
 

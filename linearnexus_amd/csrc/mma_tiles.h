@@ -137,85 +137,143 @@ __device__ __forceinline__ typename Vec16<T>::V vec_zero() {
   return z;
 }
 
-// dst[r][c] = src[r * stride + c] for r < rows (rows >= valid are zero-filled); cols % VEC == 0.
-template <typename T>
-__device__ __forceinline__ void stage_rows(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
-                                           int cols, int tid) {
-  constexpr int N = Vec16<T>::N;
-  const int vpr = cols / N;
-  for (int idx = tid; idx < rows * vpr; idx += 256) {
-    const int r = idx / vpr, c = (idx - r * vpr) * N;
-    typename Vec16<T>::V x = vec_zero<T>();
-    if (r < valid) x = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
-    *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = x;
-  }
-}
-
-// dst[c][r] = f(r) * src[r * stride + c]: transposed staging through 4-row x N-column register
-// micro-tiles (coalesced 16-byte global loads, 4-element LDS stores).  rows % 4 == 0.
-template <typename T, typename F>
-__device__ __forceinline__ void stage_rows_t(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
-                                             int cols, int tid, F row_scale) {
-  constexpr int N = Vec16<T>::N;
-  const int vpr = cols / N;
-  for (int idx = tid; idx < (rows / 4) * vpr; idx += 256) {
-    const int rg = idx / vpr, c = (idx - rg * vpr) * N;
-    typename Vec16<T>::V x[4];
-    float s[4];
+// A [ROWS x COLS] tile held in registers between its global loads and its LDS stores, so that a
+// kernel can issue the loads of all tiles of a phase before it waits for any of them.
+// Rows >= valid are zero-filled.  COLS % VEC == 0.
+template <typename T, int ROWS, int COLS> struct TileRegs {
+  static constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = (TOTAL + 255) / 256;
+  typename Vec16<T>::V x[IT];
+  __device__ __forceinline__ void load(const T* src, int64_t stride, int valid, int tid) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 4 * rg + i;
-      x[i] = vec_zero<T>();
-      if (r < valid) x[i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
-      s[i] = row_scale(r);
-    }
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-      floatx4 y = {to_f32(x[0][e]) * s[0], to_f32(x[1][e]) * s[1], to_f32(x[2][e]) * s[2], to_f32(x[3][e]) * s[3]};
-      store4(dst + (c + e) * ld + 4 * rg, y);
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+      x[it] = vec_zero<T>();
+      if (idx < TOTAL && r < valid) x[it] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
     }
   }
-}
-
-// As stage_rows_t with a per-element factor f(r, c).
-template <typename T, typename F>
-__device__ __forceinline__ void stage_rows_t_elem(T* dst, int ld, const T* src, int64_t stride, int rows, int valid,
-                                                  int cols, int tid, F elem_scale) {
-  constexpr int N = Vec16<T>::N;
-  const int vpr = cols / N;
-  for (int idx = tid; idx < (rows / 4) * vpr; idx += 256) {
-    const int rg = idx / vpr, c = (idx - rg * vpr) * N;
-    typename Vec16<T>::V x[4];
+  __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 4 * rg + i;
-      x[i] = vec_zero<T>();
-      if (r < valid) x[i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
-    }
-#pragma unroll
-    for (int e = 0; e < N; ++e) {
-      floatx4 y;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) y[i] = to_f32(x[i][e]) * elem_scale(4 * rg + i, c + e);
-      store4(dst + (c + e) * ld + 4 * rg, y);
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+      if (idx < TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = x[it];
     }
   }
-}
-
-struct UnitScale {
-  __device__ __forceinline__ float operator()(int) const { return 1.f; }
 };
 
-// Copies an LDS tile [rows][cols] (leading dimension ld) to global memory with 16-byte vectors.
-template <typename T>
-__device__ __forceinline__ void unstage_rows(T* dst, int64_t stride, const T* src, int ld, int rows, int cols, int tid) {
-  constexpr int N = Vec16<T>::N;
-  const int vpr = cols / N;
-  for (int idx = tid; idx < rows * vpr; idx += 256) {
-    const int r = idx / vpr, c = (idx - r * vpr) * N;
-    *reinterpret_cast<typename Vec16<T>::V*>(dst + r * stride + c) =
-        *reinterpret_cast<const typename Vec16<T>::V*>(src + r * ld + c);
+// The same for a tile that goes to LDS transposed (dst[c][r] = f(r, c) * src[r][c]): each thread
+// holds 4-row x N-column micro-tiles (coalesced 16-byte loads, 4-element LDS stores). ROWS % 4 == 0.
+template <typename T, int ROWS, int COLS> struct TileRegsT {
+  static constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = (ROWS / 4) * VPR, IT = (TOTAL + 255) / 256;
+  typename Vec16<T>::V x[IT][4];
+  __device__ __forceinline__ void load(const T* src, int64_t stride, int valid, int tid) {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 4 * rg + i;
+        x[it][i] = vec_zero<T>();
+        if (idx < TOTAL && r < valid) x[it][i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
+      }
+    }
   }
+  template <typename F>
+  __device__ __forceinline__ void store(T* dst, int ld, int tid, F elem_scale) const {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
+      if (idx < TOTAL) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          floatx4 y;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) y[i] = to_f32(x[it][i][e]) * elem_scale(4 * rg + i, c + e);
+          store4(dst + (c + e) * ld + 4 * rg, y);
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
+      if (idx < TOTAL) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          typename Mma<T>::Quad y = {x[it][0][e], x[it][1][e], x[it][2][e], x[it][3][e]};
+          *reinterpret_cast<typename Mma<T>::Quad*>(dst + (c + e) * ld + 4 * rg) = y;
+        }
+      }
+    }
+  }
+};
+
+// One-shot forms (load, then store) for single tiles.
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void stage_tile(T* dst, int ld, const T* src, int64_t stride, int valid, int tid) {
+  TileRegs<T, ROWS, COLS> t;
+  t.load(src, stride, valid, tid);
+  t.store(dst, ld, tid);
+}
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void stage_tile_t(T* dst, int ld, const T* src, int64_t stride, int valid, int tid) {
+  TileRegsT<T, ROWS, COLS> t;
+  t.load(src, stride, valid, tid);
+  t.store(dst, ld, tid);
+}
+template <typename T, int ROWS, int COLS, typename F>
+__device__ __forceinline__ void stage_tile_t(T* dst, int ld, const T* src, int64_t stride, int valid, int tid, F f) {
+  TileRegsT<T, ROWS, COLS> t;
+  t.load(src, stride, valid, tid);
+  t.store(dst, ld, tid, f);
+}
+
+// LDS tile [ROWS][COLS] (leading dimension ld) -> global, 16-byte vectors, rows < valid only.
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void unstage_tile(T* dst, int64_t stride, const T* src, int ld, int valid, int tid) {
+  constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = (TOTAL + 255) / 256;
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+    if (idx < TOTAL && r < valid)
+      *reinterpret_cast<typename Vec16<T>::V*>(dst + r * stride + c) =
+          *reinterpret_cast<const typename Vec16<T>::V*>(src + r * ld + c);
+  }
+}
+
+// Sums f(e) * acc[i][0][e] over the 32 lanes that share rows, for all 16*MT rows of a wave's
+// fragments at once, by a transpose-reduce (31 shuffles per 32 values instead of 160), then adds
+// the row totals into rows[] (LDS) with one atomic per row and wave.
+template <int MT>
+__device__ __forceinline__ void rows_reduce_add(float (&v)[16 * MT], int row0, int lane, float* rows) {
+  // after the step with mask m, v[t] (t < n/2) holds the partial for value index t + (lane & m ? n/2 : 0)
+  static_assert(MT == 1 || MT == 2, "one or two row tiles");
+  constexpr int NV = 16 * MT;
+  int n = NV;
+  // reduce value count down to 1 using lane bits 4,3,2,1 (and 0 when NV == 32); remaining lane bits by plain xor-adds
+  constexpr int STEPS = (MT == 2) ? 5 : 4;
+  int masks[5] = {16, 8, 4, 2, 1};
+#pragma unroll
+  for (int s_ = 0; s_ < STEPS; ++s_) {
+    const int m = masks[s_];
+    const int half = NV >> (s_ + 1);
+    const bool hi = (lane & m) != 0;
+#pragma unroll
+    for (int t = 0; t < half; ++t) {
+      const float a = v[t], b = v[t + half];
+      const float send = hi ? a : b, keep = hi ? b : a;
+      v[t] = keep + __shfl_xor(send, m, LNX_WAVE);
+    }
+  }
+  (void)n;
+  float total = v[0];
+  if (MT == 1) total += __shfl_xor(total, 1, LNX_WAVE);  // 16 values: lane bit 0 still unreduced
+  // value index owned by this lane: bits (4,3,2,1[,0]) of the lane select the halves kept
+  int idx = 0;
+#pragma unroll
+  for (int s_ = 0; s_ < STEPS; ++s_) idx |= ((lane & masks[s_]) ? (NV >> (s_ + 1)) : 0);
+  const int i = idx >> 4, e = idx & 15;
+  if (MT == 2 || (lane & 1) == 0) atomicAdd(&rows[row0 + 32 * i + frag_row(e, lane)], total);
 }
 
 // ---------------------------------------------------------------------------------------
