@@ -746,13 +746,224 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// bwd_wy2 (no gate / scalar gate): bwd_wy as one loop over 64-column slabs of [dk | dv] with the
+// next slab's tiles prefetched into registers, every product one 32x32 tile per wave, row and
+// column sums taken from the fragments, results stored through LDS with 16-byte vectors.
+// ---------------------------------------------------------------------------------------
+template <typename T, int DK> struct Wy2Cfg {
+  static constexpr int PAD = Mma<T>::PAD;
+  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int kTile = 64 * LDC;
+  static constexpr size_t bytes = sizeof(T) * 5 * kTile + sizeof(float) * 64 * 6;
+};
+
+template <typename T, int DK, int GATE>
+__global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
+  typedef Wy2Cfg<T, DK> L;
+  constexpr int LDC = L::LDC, NKS = DK / 64;
+  extern __shared__ __align__(16) char smem[];
+  float* sG = reinterpret_cast<float*>(smem);
+  float* sBeta = sG + 64;
+  float* sdB = sBeta + 64;   // dbeta: <dBu, v>
+  float* sdGk = sdB + 64;    // e^{G} <dBw, k>
+  float* sRow = sdGk + 64;   // sum_j dA_ij E_ij X_ij
+  float* sCol = sRow + 64;   // sum_i beta_i dA_ij E_ij X_ij
+  T* sTmT = reinterpret_cast<T*>(sCol + 64);
+  T* sIn = sTmT + L::kTile;   // dW^T / dD^T slab  [col][token]
+  T* sWU = sIn + L::kTile;    // W / U slab        [token][col]
+  T* sdBt = sWU + L::kTile;   // dB slab           [token][col]
+  T* sKs = sdBt + L::kTile;   // K / V slab        [token][col]
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+  const int wi = wave >> 1, wj = wave & 1;
+  const int nslab = NKS + p.dv / 64;
+
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
+    sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+    sdB[tid] = 0.f;
+    sdGk[tid] = 0.f;
+    sRow[tid] = 0.f;
+    sCol[tid] = 0.f;
+  }
+  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
+
+  TileRegsT<T, 64, 64> rInT;        // dW slab, transposed on the way to LDS
+  TileRegs<T, 64, 64> rIn, rWU, rKs;
+  auto fetch = [&](int s_) {
+    if (s_ < NKS) {
+      const int c0 = 64 * s_;
+      rInT.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
+      rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
+      rKs.load(kg + c0, DK, len, tid);
+    } else {
+      const int v0 = 64 * (s_ - NKS);
+      rIn.load(wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, tid);
+      rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+      rKs.load(vg + v0, p.dv, len, tid);
+    }
+  };
+  floatx16 aBw[NKS][1][1], aM[1][1], aX[1][1];
+#pragma unroll
+  for (int s_ = 0; s_ < NKS; ++s_) frag_zero(aBw[s_]);
+  frag_zero(aM);
+  frag_zero(aX);
+
+  fetch(0);
+#pragma unroll 1
+  for (int s_ = 0; s_ < nslab; ++s_) {
+    const bool is_k = s_ < NKS;
+    __syncthreads();
+    if (is_k) rInT.store(sIn, LDC, tid); else rIn.store(sIn, LDC, tid);
+    rWU.store(sWU, LDC, tid);
+    rKs.store(sKs, LDC, tid);
+    __syncthreads();
+    if (s_ + 1 < nslab) fetch(s_ + 1);
+    floatx16 b[1][1];
+    frag_zero(b);
+    mma_nt<T, 1, 1>(b, sTmT + 32 * wi * LDC, LDC, sIn + 32 * wj * LDC, LDC, 64, lane);
+    frag_store<T, 1, 1>(b, sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
+    {
+      float v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+        v[e] = b[0][0][e] * to_f32(sKs[r * LDC + c]);
+      }
+      rows_reduce_add<1>(v, 32 * wi, lane, is_k ? sdGk : sdB);
+    }
+    if (is_k) {
+#pragma unroll
+      for (int u = 0; u < NKS; ++u)
+        if (u == s_) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) aBw[u][0][0][e] = b[0][0][e];
+        }
+      if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
+    }
+    __syncthreads();
+    mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
+    if (!is_k) {  // dv = beta dBu, 16-byte stores
+      constexpr int VN = Vec16<T>::N;
+      T* dvg = reinterpret_cast<T*>(p.dv_out) + tbase * p.dv + 64 * (s_ - NKS);
+      for (int idx = tid; idx < 64 * 64 / VN; idx += 256) {
+        const int r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
+        if (r < len) {
+          typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBt + r * LDC + c);
+#pragma unroll
+          for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * sBeta[r]);
+          *reinterpret_cast<typename Vec16<T>::V*>(dvg + (int64_t)r * p.dv + c) = x;
+        }
+      }
+    }
+  }
+  // K^T slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
+  TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
+#pragma unroll
+  for (int u = 0; u < NKS; ++u) {
+    rKT[u].load(wsp<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)(64 * u) * 64, 64, 64, tid);
+    rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, DK, len, tid);
+  }
+  __syncthreads();  // loop tiles dead
+  T* sYa = sIn;   // beta dA E (strictly lower)
+  T* sYb = sWU;   // its transpose
+  {
+    floatx16 y[1][1];
+    float v[16], cs = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      const float da = (i > j) ? -aM[0][0][e] * dec : 0.f;
+      v[e] = da * aX[0][0][e];
+      cs += sBeta[i] * v[e];
+      y[0][0][e] = sBeta[i] * da;
+    }
+    frag_store<T, 1, 1>(y, sYa + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store_t<T, 1, 1>(y, sYb + 32 * wj * LDC + 32 * wi, LDC, lane);
+    rows_reduce_add<1>(v, 32 * wi, lane, sRow);
+    cs += __shfl_xor(cs, 32, LNX_WAVE);
+    if (lane < 32) atomicAdd(&sCol[32 * wj + lane], cs);
+  }
+#pragma unroll
+  for (int u = 0; u < NKS; ++u) {
+    T* sKT = (u == 0) ? sKs : sTmT;
+    rKT[u].store(sKT, LDC, tid);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < NKS; ++u) {
+    const T* sKT = (u == 0) ? sKs : sTmT;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane);
+      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
+      aBw[u][0][0][e] *= sBeta[r] * gm;
+    }
+    mma_nt<T, 1, 1>(aBw[u], sYa + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
+    mma_nt<T, 1, 1>(aBw[u], sYb + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
+    if (u > 0) __syncthreads();
+    frag_store<T, 1, 1>(aBw[u], sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
+    __syncthreads();
+    {
+      constexpr int VN = Vec16<T>::N, VPR = 64 / VN;
+      T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + 64 * u;
+#pragma unroll
+      for (int it = 0; it < TileRegs<T, 64, 64>::IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / VPR, c = (idx % VPR) * VN;
+        if (r < len) {
+          typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBt + r * LDC + c);
+#pragma unroll
+          for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) + to_f32(rdk[u].x[it][e]));
+          *reinterpret_cast<typename Vec16<T>::V*>(dkg + (int64_t)r * DK + c) = x;
+        }
+      }
+    }
+  }
+  // dbeta and dg
+  if (wave == 0) {
+    const int t = lane;
+    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[t]);
+    const float w = gm * sdGk[t], rs = sRow[t];
+    if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
+    if (GATE != LNX_GATE_NONE) {
+      float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - sCol[t];
+#pragma unroll
+      for (int s_ = 1; s_ < 64; s_ <<= 1) {
+        const float y = __shfl_down(d, s_, LNX_WAVE);
+        if (t + s_ < 64) d += y;
+      }
+      if (t < len) p.dg[tbase + t] = d;
+    }
+  }
+}
+
+template <typename T, int DK, int GATE> struct WySelect {
+  static constexpr size_t bytes = Wy2Cfg<T, DK>::bytes;
+  static auto kernel() { return bwd_wy2_kernel<T, DK, GATE>; }
+};
+template <typename T, int DK> struct WySelect<T, DK, LNX_GATE_VECTOR> {
+  static constexpr size_t bytes = WyCfg<T, DK, LNX_GATE_VECTOR>::bytes;
+  static auto kernel() { return bwd_wy_kernel<T, DK, LNX_GATE_VECTOR>; }
+};
+
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   auto k1 = bwd_scan_kernel<T, DK, GATE>;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
-  auto k3 = bwd_wy_kernel<T, DK, GATE>;
-  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = WyCfg<T, DK, GATE>::bytes;
+  auto k3 = WySelect<T, DK, GATE>::kernel();
+  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = WySelect<T, DK, GATE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
