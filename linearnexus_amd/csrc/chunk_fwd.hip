@@ -1,6 +1,6 @@
 // Chunked (WY) delta-rule forward on gfx950 MFMA, three kernels per call:
 //
-//   chunk_prepare  (one workgroup per 64-token chunk, all chunks in parallel)
+//   chunk_prepare2 (one workgroup per 64-token chunk, all chunks in parallel; kda_prepare for a vector gate)
 //       A = tril(diag(beta) K K^T * E, -1);  Tm = (I + A)^-1 (fp32, block forward substitution +
 //       MFMA block merges);  W = Tm diag(beta e^G) K;  U = Tm diag(beta) V;
 //       P = scale * tril(Q K^T * E);  also K^T and Tm^T for later kernels.
@@ -49,30 +49,35 @@ __device__ __forceinline__ float wave_cumsum(float x, int lane) {
 }
 
 // ---------------------------------------------------------------------------------------
-// chunk_prepare
+// chunk_prepare2 (no gate / scalar gate): the same computation as chunk_prepare, organised as
+// slab loops with register prefetch so that two workgroups fit a CU: K K^T and Q K^T over
+// 64-channel slabs, the fp32 inverse, then one 64-column slab of [dk | dv] at a time for
+// W / W^T / K^T / Qg^T and U, every result leaving through LDS with 16-byte stores.
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct PrepSmem {
+template <typename T, int DK> struct Prep2Cfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD;      // row-major [64][DK] tiles
-  static constexpr int LDC = LNX_C + PAD;   // transposed [d][64] tiles and [64][64] tiles
-  static constexpr int kK = 64 * LDK;                       // sK, later sTw
-  static constexpr int kKT = DK * LDC;                      // sKT
-  static constexpr int kQ = (64 * LDK > DK * LDC) ? 64 * LDK : DK * LDC;  // sQ, later Qg^T, then V^T slabs
-  static constexpr size_t bytes = sizeof(T) * (kK + kKT + kQ) + sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36 + 128);
+  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int kTile = 64 * LDC;
+  static constexpr size_t f32_bytes = sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36);
+  static constexpr size_t regionF = (4 * kTile * sizeof(T) > f32_bytes) ? 4 * kTile * sizeof(T) : f32_bytes;
+  static constexpr size_t bytes = regionF + 2 * kTile * sizeof(T) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
-  typedef PrepSmem<T, DK> L;
-  constexpr int LDK = L::LDK, LDC = L::LDC;
+__global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
+  typedef Prep2Cfg<T, DK> L;
+  constexpr int LDC = L::LDC, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
-  T* sK = reinterpret_cast<T*>(smem);
-  T* sKT = sK + L::kK;
-  T* sQ = sKT + L::kKT;
-  float* sA = reinterpret_cast<float*>(sQ + L::kQ);
+  float* sA = reinterpret_cast<float*>(smem);
   float* sT = sA + 64 * LNX_LDA;
   float* sX = sT + 64 * LNX_LDA;
-  float* sBeta = sX + 32 * 36;
+  T* sIn = reinterpret_cast<T*>(smem);  // overlays the fp32 matrices once Tw / Tu exist
+  T* sOut = sIn + L::kTile;
+  T* sOut2 = sOut + L::kTile;
+  T* sQg = sOut2 + L::kTile;
+  T* sKa = reinterpret_cast<T*>(smem + L::regionF);  // K slab, then Tw
+  T* sQa = sKa + L::kTile;                           // Q slab, then Tu
+  float* sBeta = reinterpret_cast<float*>(sQa + L::kTile);
   float* sG = sBeta + 64;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -86,10 +91,11 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+  const int wi = wave >> 1, wj = wave & 1;
 
-  stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
-  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid);
-  stage_tile<T, 64, DK>(sQ, LDK, qg, DK, len, tid);
+  TileRegs<T, 64, 64> rK, rQ;
+  rK.load(kg, DK, len, tid);
+  rQ.load(qg, DK, len, tid);
   if (wave == 0) {
     const bool ok = lane < len;
     sBeta[lane] = ok ? p.beta[tbase + lane] : 0.f;
@@ -99,48 +105,57 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
     sG[lane] = gv;
     ws_ptr<float>(p, p.off.G)[slot * 64 + lane] = gv;
   }
-  __syncthreads();
-
-  // X = K K^T and Q K^T, one 32x32 tile per wave (the upper-right tile is all zero)
-  {
-    const int wi = wave >> 1, wj = wave & 1;
-    floatx16 ax[1][1], ap[1][1];
-    frag_zero(ax);
-    frag_zero(ap);
-    if (!(wi == 0 && wj == 1)) {
-      mma_nt<T, 1, 1>(ax, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
-      mma_nt<T, 1, 1>(ap, sQ + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
+  floatx16 ax[1][1], ap[1][1];
+  frag_zero(ax);
+  frag_zero(ap);
+#pragma unroll 1
+  for (int s_ = 0; s_ < NKS; ++s_) {
+    __syncthreads();
+    rK.store(sKa, LDC, tid);
+    rQ.store(sQa, LDC, tid);
+    __syncthreads();
+    if (s_ + 1 < NKS) {
+      rK.load(kg + 64 * (s_ + 1), DK, len, tid);
+      rQ.load(qg + 64 * (s_ + 1), DK, len, tid);
     }
-    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
+    if (!(wi == 0 && wj == 1)) {
+      mma_nt<T, 1, 1>(ax, sKa + 32 * wi * LDC, LDC, sKa + 32 * wj * LDC, LDC, 64, lane);
+      mma_nt<T, 1, 1>(ap, sQa + 32 * wi * LDC, LDC, sKa + 32 * wj * LDC, LDC, 64, lane);
+    }
+  }
+  // first slab of the second loop, in flight during the inverse
+  TileRegsT<T, 64, 64> rInT, rQT;
+  auto fetch = [&](int s_) {
+    if (s_ < NKS) {
+      rInT.load(kg + 64 * s_, DK, len, tid);
+      rQT.load(qg + 64 * s_, DK, len, tid);
+    } else {
+      rInT.load(vg + 64 * (s_ - NKS), p.dv, len, tid);
+    }
+  };
+  fetch(0);
+  __syncthreads();  // slab tiles dead
+  {
+    floatx16 pe[1][1];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
       sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * ax[0][0][e] : 0.f;
-      Pg[i * 64 + j] = from_f32<T>((i >= j) ? p.scale * dec * ap[0][0][e] : 0.f);
+      pe[0][0][e] = (i >= j) ? p.scale * dec * ap[0][0][e] : 0.f;
     }
+    frag_store<T, 1, 1>(pe, sKa + 32 * wi * LDC + 32 * wj, LDC, lane);
   }
   __syncthreads();
-  // (scale * Q * e^G)^T for the backward scan, staged through the sQ region
-  stage_tile_t<T, 64, DK>(sQ, LDC, qg, DK, len, tid, [&](int r, int) {
-    return (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
-  });
+  unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sKa, LDC, 64, tid);
   tri_inverse_64(sA, sT, sX, tid);
-  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, tid);
-
-  // Tw = Tm * diag(beta e^G) (into the sK region), Tu = Tm * diag(beta) (into the sA region),
-  // Tm^T to the workspace.
-  T* sTw = sK;
-  T* sTu = reinterpret_cast<T*>(sA);
   {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
+    T* sTw = sKa;
+    T* sTu = sQa;
     for (int idx = tid; idx < 64 * 64; idx += 256) {
       const int r = idx >> 6, c = idx & 63;
       TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
-    }
-    __syncthreads();  // everyone is done reading sA (inverse) and sK (products)
-    for (int idx = tid; idx < 64 * 64; idx += 256) {
-      const int r = idx >> 6, c = idx & 63;
       const float t = sT[r * LNX_LDA + c];
       const float bu = sBeta[c];
       const float bw = (GATE == LNX_GATE_NONE) ? bu : bu * __expf(sG[c]);
@@ -148,34 +163,30 @@ __global__ __launch_bounds__(256) void chunk_prepare_kernel(FwdParams p) {
       sTw[r * LDC + c] = from_f32<T>(t * bw);
     }
   }
-  __syncthreads();
-
-  const int wi = wave >> 1, wj = wave & 1;
-  // W = Tw K, 64 columns at a time
-  {
-    T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
-    for (int c0 = 0; c0 < DK; c0 += 64) {
-      floatx16 acc[1][1];
-      frag_zero(acc);
-      mma_nt<T, 1, 1>(acc, sTw + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
-      frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
-      frag_store_t<T, 1, 1>(acc, ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)(c0 + 32 * wj) * 64 + 32 * wi, 64, lane);
-    }
-    // K^T for the scan kernel
-    unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, tid);
-  }
-  // U = Tu V, one transposed 64-column slab of V at a time (slab overlays sQ)
-  {
-    T* sVT = sQ;
-    T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
-    for (int c0 = 0; c0 < p.dv; c0 += 64) {
-      __syncthreads();
-      stage_tile_t<T, 64, 64>(sVT, LDC, vg + c0, p.dv, len, tid);
-      __syncthreads();
-      floatx16 acc[1][1];
-      frag_zero(acc);
-      mma_nt<T, 1, 1>(acc, sTu + 32 * wi * LDC, LDC, sVT + 32 * wj * LDC, LDC, 64, lane);
-      frag_store<T, 1, 1>(acc, Ug + 32 * wi * p.dv + c0 + 32 * wj, p.dv, lane);
+  const int nslab = NKS + p.dv / 64;
+#pragma unroll 1
+  for (int s_ = 0; s_ < nslab; ++s_) {
+    const bool is_k = s_ < NKS;
+    __syncthreads();  // fp32 matrices / previous slab's tiles are dead
+    rInT.store(sIn, LDC, tid);
+    if (is_k)
+      rQT.store(sQg, LDC, tid, [&](int r, int) { return (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]); });
+    __syncthreads();
+    if (s_ + 1 < nslab) fetch(s_ + 1);
+    floatx16 acc[1][1];
+    frag_zero(acc);
+    mma_nt<T, 1, 1>(acc, (is_k ? sKa : sQa) + 32 * wi * LDC, LDC, sIn + 32 * wj * LDC, LDC, 64, lane);
+    frag_store<T, 1, 1>(acc, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
+    if (is_k) frag_store_t<T, 1, 1>(acc, sOut2 + 32 * wj * LDC + 32 * wi, LDC, lane);
+    __syncthreads();
+    if (is_k) {
+      const int c0 = 64 * s_;
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + c0, DK, sOut, LDC, 64, tid);
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sOut2, LDC, 64, tid);
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sIn, LDC, 64, tid);
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sQg, LDC, 64, tid);
+    } else {
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + 64 * (s_ - NKS), p.dv, sOut, LDC, 64, tid);
     }
   }
 }
@@ -579,8 +590,8 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* 
 }
 
 template <typename T, int DK, int GATE> struct PrepSelect {
-  static constexpr size_t bytes = PrepSmem<T, DK>::bytes;
-  static auto kernel() { return chunk_prepare_kernel<T, DK, GATE>; }
+  static constexpr size_t bytes = Prep2Cfg<T, DK>::bytes;
+  static auto kernel() { return chunk_prepare2_kernel<T, DK, GATE>; }
 };
 template <typename T, int DK> struct PrepSelect<T, DK, LNX_GATE_VECTOR> {
   static constexpr size_t bytes = KdaPrepSmem<T, DK>::bytes;
