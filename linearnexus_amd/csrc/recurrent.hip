@@ -132,11 +132,16 @@ __global__ __launch_bounds__(256) void decode_step_kernel(TokenParams p) {
   const int64_t sbase = (bh * DK + row0) * p.dv + col0;
   floatx4 S[RPL];
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) S[i] = load4(p.s_in + sbase + (int64_t)i * p.dv);
+  for (int i = 0; i < RPL; ++i) {
+    // streamed once: non-temporal, so the 512 MiB state does not churn L2 / the memory-side cache
+    S[i] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p.s_in + sbase + (int64_t)i * p.dv));
+  }
   const floatx4 v4 = load4(reinterpret_cast<const T*>(p.v) + bh * p.dv + col0);
   const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, p.beta[bh], v4, qk);
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) store4(p.s_out + sbase + (int64_t)i * p.dv, S[i]);
+  for (int i = 0; i < RPL; ++i) {
+    __builtin_nontemporal_store(S[i], reinterpret_cast<floatx4*>(p.s_out + sbase + (int64_t)i * p.dv));
+  }
   if ((lane >> 3) == 0) store_o4(p.o, bh * p.dv + col0, o4, p.o_dtype);
 }
 
