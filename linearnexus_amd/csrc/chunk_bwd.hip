@@ -71,9 +71,11 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   __shared__ __align__(16) T sdOT[64 * LDC];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
-  const int64_t slot = blockIdx.x;
+  int64_t slot;
+  int part;
+  if (!xcd_slot_part((int64_t)p.geom.rows * N, p.dv / 64, slot, part)) return;
   const int row = (int)(slot / N), n = (int)(slot % N);
-  const int v0 = blockIdx.y * 64;
+  const int v0 = part * 64;
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
@@ -295,8 +297,10 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
-  const int64_t slot = blockIdx.x;
-  const int ch0 = blockIdx.y * 64;  // first key channel of this half
+  int64_t slot;
+  int part;
+  if (!xcd_slot_part((int64_t)p.geom.rows * N, DK / 64, slot, part)) return;
+  const int ch0 = part * 64;  // first key channel of this half
   const int row = (int)(slot / N), n = (int)(slot % N);
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
@@ -970,11 +974,11 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
       (e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b3)) != hipSuccess)
     return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   lnx_profile_mark("bwd_local", st);
-  hipLaunchKernelGGL(bwd_local_kernel<T>, dim3((unsigned)slots, (unsigned)(p.dv / 64)), dim3(256), 0, st, p);
+  hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
   lnx_profile_mark("bwd_scan", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(256), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
-  hipLaunchKernelGGL(k2, dim3((unsigned)slots, (unsigned)(DK / 64)), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("bwd_wy", st);
   hipLaunchKernelGGL(k3, dim3((unsigned)slots), dim3(256), b3, st, p);
   lnx_profile_mark(nullptr, st);

@@ -50,6 +50,17 @@ __device__ __forceinline__ void seq_chunks(const ChunkGeom& g, int s, int& c0, i
   }
 }
 
+// 1-D launch of `parts` workgroups per chunk slot such that the parts of one slot run on the same
+// XCD (workgroups are dealt round-robin to the 8 XCDs, each with its own L2) and back to back, so
+// the tiles they share are read from HBM once.  Grid size: lnx_xcd_grid(slots, parts).
+__device__ __forceinline__ bool xcd_slot_part(int64_t slots, int parts, int64_t& slot, int& part) {
+  const int64_t bid = blockIdx.x, rest = bid >> 3;
+  part = (int)(rest % parts);
+  slot = (rest / parts) * 8 + (bid & 7);
+  return slot < slots;
+}
+inline unsigned lnx_xcd_grid(int64_t slots, int parts) { return (unsigned)(((slots + 7) / 8) * 8 * parts); }
+
 struct ChunkWs {
   uint64_t tab, G, P, X, W, WT, QgT, U, KT, Kr, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, dG, total;
 };

@@ -516,9 +516,11 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
-  const int64_t slot = blockIdx.x;
+  int64_t slot;
+  int part;
+  if (!xcd_slot_part((int64_t)p.geom.rows * N, p.dv / BV, slot, part)) return;
   const int row = (int)(slot / N), n = (int)(slot % N);
-  const int v0 = blockIdx.y * BV;
+  const int v0 = part * BV;
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
@@ -615,7 +617,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("chunk_scan", st);
   hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("chunk_output", st);
-  hipLaunchKernelGGL(k3, dim3((unsigned)slots, (unsigned)(p.dv / 64)), dim3(256), b3, st, p);
+  hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
   lnx_profile_mark(nullptr, st);
   return LNX_OK;
 }
