@@ -1,0 +1,129 @@
+"""Benchmark-shaped parity checks on the GPU.
+
+The fp64 oracle finishes in seconds only on slices, so at the full BASELINE shapes the checks
+are (a) the oracle on a slice of the (batch, head) rows of the very same launch and
+(b) size-independent properties: MFMA chunk path == fp32 token-by-token kernel, the adjoint
+identity <dO, o(v)> = <dv, v>, and var-len == per-sequence launches."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import recurrent as rc
+from oracle.inputs import make_cu_seqlens
+from conftest import max_rel
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _nrm(x):
+    return x / (x.norm(dim=-1, keepdim=True) + 1e-6)
+
+
+def _rel(a, b):
+    a, b = a.detach(), b.detach()
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max())
+
+
+def test_config3_kda_full_shape():
+    """KDA chunk fwd+bwd at B4 H16 T8192 d128 bf16, vector gate, random S0."""
+    import linearnexus_amd as la
+    torch.manual_seed(3)
+    B, H, T, d = 4, 16, 8192, 128
+    q = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16()
+    k = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16()
+    v = torch.randn(B, H, T, d, device=DEV).bfloat16().requires_grad_(True)
+    beta = torch.sigmoid(torch.randn(B, H, T, device=DEV))
+    g = -torch.nn.functional.softplus(torch.randn(B, H, T, d, device=DEV)) * 0.05
+    S0 = torch.randn(B, H, d, d, device=DEV) * 0.02
+    o1, S1 = la.kda_recurrent(q, k, v.detach(), g, beta, None, S0, False)
+    o2, S2 = la.kda_chunkwise(q, k, v, g, beta, None, S0, 64, False)
+    assert o2.dtype == torch.float32  # kda.py:655
+    assert _rel(o2, o1.float()) < 2e-2 and _rel(S2, S1) < 2e-2
+    # oracle on one (batch, head) row of the same launch, first 512 tokens
+    sl = lambda t: t.detach()[1:2, 3:4, :512].float().cpu().numpy()
+    o_ref, _ = rc.kda_recurrent(sl(q), sl(k), sl(v.detach()), sl(g), sl(beta), None, S0[1:2, 3:4].cpu().numpy(), False)
+    assert max_rel(o2.detach()[1:2, 3:4, :512].cpu().numpy(), o_ref) < 2e-2
+    # adjoint identity with S0 = 0 (o linear in v)
+    dO = torch.randn(B, H, T, d, device=DEV)
+    o3, _ = la.kda_chunkwise(q, k, v, g, beta, None, None, 64, False)
+    o3.backward(dO)
+    lhs = (o3.detach().double() * dO.bfloat16().double()).sum()
+    rhs = (v.grad.double() * v.detach().double()).sum()
+    assert abs(lhs - rhs) <= 5e-3 * abs(lhs), (float(lhs), float(rhs))
+
+
+def test_config5_deltanet_long_packed():
+    """DeltaNet chunk fwd+bwd at B1 H32 T32768 d128 bf16, 8 packed sequences in [1024, 8192]."""
+    import linearnexus_amd as la
+    torch.manual_seed(5)
+    H, T, d = 32, 32768, 128
+    cu = make_cu_seqlens(5, 8, T, 1024, 8192)
+    q = _nrm(torch.randn(1, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    k = _nrm(torch.randn(1, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    v = torch.randn(1, H, T, d, device=DEV).bfloat16().requires_grad_(True)
+    beta = torch.sigmoid(torch.randn(1, H, T, device=DEV)).requires_grad_(True)
+    S0 = (torch.randn(8, H, d, d, device=DEV) * 0.02).requires_grad_(True)
+    dO = torch.randn(1, H, T, d, device=DEV).bfloat16()
+    cu_t = torch.from_numpy(cu).to(DEV)
+    o, S = la.delta_rule_chunkwise(q, k, v, beta, S0, cu_seqlens=cu_t)
+    o.backward(dO)
+    assert tuple(S.shape) == (8, H, d, d) and all(t.grad is not None for t in (q, k, v, beta, S0))
+    # (a) packed == the token-by-token kernel on the packed batch
+    o_r, S_r = la.delta_rule_recurrent(q.detach(), k.detach(), v.detach(), beta.detach(), S0.detach(), cu_seqlens=cu_t)
+    assert _rel(o, o_r) < 2e-2 and _rel(S, S_r) < 2e-2
+    # (b) packed == one launch per sequence, outputs and every gradient (sequence 2 and the last)
+    for s in (2, 7):
+        a, b = int(cu[s]), int(cu[s + 1])
+        leaf = lambda t: t.detach()[:, :, a:b].clone().requires_grad_(True)
+        qs, ks, vs, bs = leaf(q), leaf(k), leaf(v), leaf(beta)
+        s0 = S0.detach()[s:s + 1].clone().requires_grad_(True)
+        o_s, S_s = la.delta_rule_chunkwise(qs, ks, vs, bs, s0)
+        o_s.backward(dO[:, :, a:b])
+        assert _rel(o[:, :, a:b], o_s) < 1e-3 and _rel(S[s:s + 1], S_s) < 1e-3
+        for full, part in ((q.grad, qs.grad), (k.grad, ks.grad), (v.grad, vs.grad), (beta.grad, bs.grad)):
+            assert _rel(full[:, :, a:b], part) < 1e-3
+        assert _rel(S0.grad[s:s + 1], s0.grad) < 1e-3
+    # (c) oracle on the first 300 tokens of sequence 0, head 5
+    a = int(cu[0])
+    sl = lambda t: t.detach()[:, 5:6, a:a + 300].float().cpu().numpy()
+    o_ref, _ = rc.delta_rule_recurrent(sl(q), sl(k), sl(v), sl(beta), S0.detach()[0:1, 5:6].cpu().numpy())
+    assert max_rel(o.detach()[:, 5:6, a:a + 300].float().cpu().numpy(), o_ref) < 2e-2
+
+
+def test_config4_decode_full_shape_one_step_and_1000_steps():
+    """Gated decode step at B256 H32 d128: one in-place step against the oracle on a slice of
+    the rows, then 1000 back-to-back steps on a smaller batch against the oracle scan."""
+    import linearnexus_amd as la
+    torch.manual_seed(4)
+    B, H, d = 256, 32, 128
+    S = torch.randn(B, H, d, d, device=DEV) * 0.02
+    S_before = S[:2, :4].clone()
+    q = _nrm(torch.randn(B, H, d, device=DEV)).bfloat16()
+    k = _nrm(torch.randn(B, H, d, device=DEV)).bfloat16()
+    v = torch.randn(B, H, d, device=DEV).bfloat16()
+    beta = torch.sigmoid(torch.randn(B, H, device=DEV))
+    g = -torch.nn.functional.softplus(torch.randn(B, H, device=DEV)) * 0.1
+    o, S2 = la.gated_delta_rule_step(q, k, v, g, beta, S, use_qk_l2norm=False, inplace=True)
+    assert S2.data_ptr() == S.data_ptr()
+    n = lambda t: t[:2, :4].float().cpu().numpy()
+    o_ref, S_ref = rc.gated_delta_rule_step(n(q), n(k), n(v), n(g), n(beta), S_before.cpu().numpy(), None, False)
+    assert max_rel(o[:2, :4].float().cpu().numpy(), o_ref) < 2e-2 and max_rel(S[:2, :4].cpu().numpy(), S_ref) < 2e-2
+    # 1000 steps, B=4 H=4
+    B, H, T = 4, 4, 1000
+    S = torch.randn(B, H, d, d, device=DEV) * 0.02
+    S0 = S.clone()
+    q = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16()
+    k = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16()
+    v = torch.randn(B, H, T, d, device=DEV).bfloat16()
+    beta = torch.sigmoid(torch.randn(B, H, T, device=DEV))
+    g = -torch.nn.functional.softplus(torch.randn(B, H, T, device=DEV)) * 0.1
+    outs = []
+    for t in range(T):
+        o, _ = la.gated_delta_rule_step(q[:, :, t], k[:, :, t], v[:, :, t], g[:, :, t], beta[:, :, t], S,
+                                        use_qk_l2norm=False, inplace=True)
+        outs.append(o)
+    o = torch.stack(outs, 2)
+    f = lambda t: t.float().cpu().numpy()
+    o_ref, S_ref = rc.gated_delta_rule_recurrent(f(q), f(k), f(v), f(g), f(beta), None, f(S0), False)
+    assert max_rel(f(o), o_ref) < 2e-2 and max_rel(f(S), S_ref) < 2e-2
