@@ -1,6 +1,7 @@
 """Benchmark of the chunked delta-rule scan on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload gdn_chunk|kda_chunk|deltanet_varlen|deltanet_fp32|decode]
 
 Default workload: Gated DeltaNet chunked forward+backward at B=8, H=16, T=4096, dk=dv=128,
 bf16 q/k/v/dO, fp32 beta/g, chunk 64 (benchmark configuration 2).  One "step" is one forward
@@ -27,6 +28,11 @@ if ROOT not in sys.path:
 C = 64
 PEAK_BF16 = 2500.0  # TFLOP/s, dense bf16 MFMA, MI355X
 PEAK_HBM = 8000.0   # GB/s
+PEAK_FP32_MFMA = 157.3  # TFLOP/s
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured for that (workload, kernel).
+TRAFFIC = {}
 
 
 def chunk_flops(dk, dv):
@@ -76,20 +82,52 @@ def cpu_baseline_chunk(torch, B, H, T, d, seed):
             "sample": f"B={Bs} of {B} batch rows, H={H}, T={T}, d={d}, fp32, one timed pass ({dt:.1f} s)"}
 
 
-def bench_gdn_chunk(args, torch, la, _lib):
-    B, H, T, d = 8, 16, 4096, 128
+CHUNK_CONFIGS = {
+    # name: (variant, B, H, T, d, packed sequences, random S0, backward)
+    "gdn_chunk": ("gated", 8, 16, 4096, 128, 0, False, True),        # configuration 2 (headline)
+    "kda_chunk": ("kda", 4, 16, 8192, 128, 0, True, True),           # configuration 3
+    "deltanet_varlen": ("delta", 1, 32, 32768, 128, 8, False, True),  # configuration 5
+    "deltanet_fp32": ("delta32", 2, 4, 512, 64, 0, False, False),     # configuration 1 (forward only)
+}
+
+
+def bench_chunk(args, torch, la, _lib, name):
+    variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
-    x = make_gdn_inputs(torch, B, H, T, d, 2, dev)
-    q, k, v, dO = (x[n].to(torch.bfloat16) for n in ("q", "k", "v", "dO"))
+    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5}[name]
+    x = make_gdn_inputs(torch, B, H, T, d, seed, dev)
+    dt = torch.float32 if variant == "delta32" else torch.bfloat16
+    q, k, v, dO = (x[n].to(dt) for n in ("q", "k", "v", "dO"))
     beta, g = x["beta"], x["g"]
-    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
-    beta.requires_grad_(True), g.requires_grad_(True)
+    gen = torch.Generator(device="cpu").manual_seed(seed + 100)
+    if variant == "kda":
+        g = (-torch.nn.functional.softplus(torch.randn(B, H, T, d, generator=gen)) * 0.05).to(dev)
+    cu = None
+    nstate = B
+    if nseq:
+        from oracle.inputs import make_cu_seqlens
+        cu_np = make_cu_seqlens(seed, nseq, T, 1024, 8192)
+        cu = torch.from_numpy(cu_np).to(dev)
+        nstate = nseq
+    s0 = (torch.randn(nstate, H, d, d, generator=gen) * 0.02).to(dev) if (with_s0 or nseq) else None
+    leaves = [q, k, v, beta] + ([g] if variant in ("gated", "kda") else []) + ([s0] if s0 is not None else [])
+    if backward:
+        for t in leaves:
+            t.requires_grad_(True)
+
+    def forward():
+        if variant == "gated":
+            return la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, s0, 64, False)
+        if variant == "kda":
+            return la.kda_chunkwise(q, k, v, g, beta, None, s0, 64, False)
+        return la.delta_rule_chunkwise(q, k, v, beta, s0, cu_seqlens=cu)
 
     def step():
-        for t in (q, k, v, beta, g):
+        for t in leaves:
             t.grad = None
-        o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, use_qk_l2norm=False)
-        o.backward(dO)
+        o, S = forward()
+        if backward:
+            o.backward(dO.to(o.dtype))
 
     for _ in range(args.warmup):
         step()
@@ -100,32 +138,37 @@ def bench_gdn_chunk(args, torch, la, _lib):
     for i in range(args.steps):
         step()
         if (i + 1) % 512 == 0:  # the library keeps a bounded number of event marks
-            for name, ms in _lib.profile_read():
-                per_kernel.setdefault(name, []).append(ms)
+            for kn, ms in _lib.profile_read():
+                per_kernel.setdefault(kn, []).append(ms)
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
-    for name, ms in _lib.profile_read():
-        per_kernel.setdefault(name, []).append(ms)
+    dtm = (time.perf_counter() - t0) / args.steps
+    for kn, ms in _lib.profile_read():
+        per_kernel.setdefault(kn, []).append(ms)
     _lib.profile_enable(False)
 
-    nchunks = B * H * (T // C)
+    if nseq:
+        nchunks = H * int(sum(-(-int(l) // C) for l in (cu_np[1:] - cu_np[:-1])))
+    else:
+        nchunks = B * H * (-(-T // C))
     fl = chunk_flops(d, d)
     avg = {n: sum(v_) / len(v_) for n, v_ in per_kernel.items()}
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
-    total_fl = 3 * (2 * C * C * (3 * d + 2 * d) + 6 * C * d * d) * nchunks
+    peak = PEAK_FP32_MFMA if variant == "delta32" else PEAK_BF16
+    total_fl = (3 if backward else 1) * (2 * C * C * (3 * d + 2 * d) + 6 * C * d * d) * nchunks
     out = {
         "metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
-        "value": B * T / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "gated_deltanet_chunk_fwd_bwd", "B": B, "H": H, "T": T, "dk": d, "dv": d, "chunk": C,
-                   "use_qk_l2norm": False, "inputs": "q,k pre-normalised; bf16 q/k/v/dO, fp32 beta/g"},
-        "tflops_algorithmic": total_fl / dt / 1e12,
-        "mfma_peak_frac": total_fl / dt / 1e12 / PEAK_BF16,
+        "value": B * T / dtm, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dtm * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if variant == "delta32" else "bf16", "data": "synthetic",
+        "config": {"workload": name + ("_fwd_bwd" if backward else "_fwd"), "variant": variant, "B": B, "H": H, "T": T,
+                   "dk": d, "dv": d, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
+                   "use_qk_l2norm": False, "inputs": "q,k pre-normalised; fp32 beta/g"},
+        "tflops_algorithmic": total_fl / dtm / 1e12,
+        "mfma_peak_frac": total_fl / dtm / 1e12 / peak,
         "kernel_ms": {n: round(t, 4) for n, t in avg.items()},
-        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16, "traffic": None},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                     "frac": achieved / peak, "traffic": TRAFFIC.get((name, dom))},
     }
     return out, (B, H, T, d)
 
@@ -176,7 +219,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -203,9 +246,10 @@ def main():
         print(json.dumps(out))
         return
 
-    out, (B, H, T, d) = bench_gdn_chunk(args, torch, la, _lib)
-    out["decode_step"] = bench_decode(args, torch, la, _lib)
-    if not args.no_cpu_baseline:
+    out, (B, H, T, d) = bench_chunk(args, torch, la, _lib, args.workload)
+    if args.workload == "gdn_chunk":
+        out["decode_step"] = bench_decode(args, torch, la, _lib)
+    if not args.no_cpu_baseline and args.workload == "gdn_chunk":
         out["cpu_baseline"] = cpu_baseline_chunk(torch, B, H, T, d, 2)
     print(json.dumps(out))
 

@@ -4,7 +4,7 @@
 // linearnexus/train/sft.py:126-127); this is the hand-derived adjoint of the chunk algorithm of
 // gated_deltanet.py:444-523.  Four kernels:
 //
-//   bwd_local  (chunk x dv-slab parallel)   dD_loc = P^T dO;  also stores dO^T
+//   bwd_local  (chunk x dv-slab parallel)   dD_loc = P^T dO
 //   bwd_scan   (sequential, reverse)        dD = dD_loc + (K r) dS;  dS <- e^{G_last} dS + (Q~ e^G)^T dO - W^T dD
 //   bwd_dqk    (chunk parallel)             dP, dq, the P/K^r parts of dk, dW = -dD S^T, gate terms
 //   bwd_wy     (chunk parallel)             through W = Tm B_w, U = Tm B_u and Tm = (I + A)^-1:
@@ -67,8 +67,8 @@ __device__ __forceinline__ void frag_rowdot(const floatx16 (&acc)[MT][1], int ro
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   constexpr int LDC = LNX_C + Mma<T>::PAD;
-  __shared__ __align__(16) T sPT[64 * LDC];
-  __shared__ __align__(16) T sdOT[64 * LDC];
+  __shared__ __align__(16) T sP[64 * LDC];    // P  [i][j]
+  __shared__ __align__(16) T sdO[64 * LDC];   // dO [i][v]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
   int64_t slot;
@@ -81,14 +81,17 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   if (len <= 0) return;
   const int64_t tbase = (int64_t)row * p.geom.T + tok0;
   if (v0 == 0 && tid < 64 && p.gate == LNX_GATE_SCALAR) wsp<float>(p, p.off.dG)[slot * 64 + tid] = 0.f;  // accumulated by bwd_dqk
-  stage_tile_t<T, 64, 64>(sPT, LDC, wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
-  stage_tile_t<T, 64, 64>(sdOT, LDC, reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
+  TileRegs<T, 64, 64> rP, rdO;
+  rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
+  rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
+  rP.store(sP, LDC, tid);
+  rdO.store(sdO, LDC, tid);
   __syncthreads();
-  unstage_tile<T, 64, 64>(wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdOT, LDC, 64, tid);
   const int wi = wave >> 1, wj = wave & 1;
   floatx16 acc[1][1];
   frag_zero(acc);
-  mma_nt<T, 1, 1>(acc, sPT + 32 * wi * LDC, LDC, sdOT + 32 * wj * LDC, LDC, 64, lane);
+  // dD_loc[j][v] = sum_i P[i][j] dO[i][v]: both operands contract along the rows of their tiles
+  mma_x<T, 1, 1, true, true>(acc, sP + 32 * wi, LDC, sdO + 32 * wj, LDC, 64, lane);
   frag_store<T, 1, 1>(acc, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
 }
 
@@ -98,29 +101,30 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 template <typename T, int DK> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int BV = (sizeof(T) == 4 && DK == 128) ? 32 : 64;  // dv slab per workgroup
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDU = BV + PAD;
-  static constexpr int kK = 64 * LDK, kQT = DK * LDC, kWT = DK * LDC, kdOT = BV * LDC, kdDl = 64 * LDU,
-                       kdST = BV * LDK, kdDT = BV * LDC;
-  static constexpr size_t bytes = sizeof(T) * (kK + kQT + kWT + kdOT + kdDl + kdST + kdDT) + sizeof(float) * 128;
+  static constexpr int LDK = DK + PAD, LDU = BV + PAD;
+  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
+  // K, Q, W rows [token][dk];  dO, dD_loc slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk]
+  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
   typedef BScanCfg<T, DK> L;
   typedef typename Vec16<T>::V V16;
-  constexpr int LDK = L::LDK, LDC = L::LDC, LDU = L::LDU, BV = L::BV, VN = Vec16<T>::N;
+  constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV, VN = Vec16<T>::N;
   constexpr int CT = BV / 32;                      // column tiles of the slab
   constexpr int NT = (DK == 128) ? CT : 1;         // state tiles per wave (row tile = wave or wave & 1)
   static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
   T* sK = reinterpret_cast<T*>(smem);
-  T* sQT = sK + L::kK;
-  T* sWT = sQT + L::kQT;
-  T* sdOT = sWT + L::kWT;
-  T* sdDl = sdOT + L::kdOT;
-  T* sdST = sdDl + L::kdDl;
-  T* sdDT = sdST + L::kdST;
-  float* sG = reinterpret_cast<float*>(sdDT + L::kdDT);
+  T* sQ = sK + L::kRow;
+  T* sW = sQ + L::kRow;
+  T* sdO = sW + L::kRow;
+  T* sdDl = sdO + L::kSlab;
+  T* sdDT = sdDl + L::kSlab;
+  T* sdST = sdDT + L::kdDT;
+  float* sG = reinterpret_cast<float*>(sdST + L::kdST);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
@@ -147,36 +151,45 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
   }
 
   constexpr int NK = 64 * DK / VN / 256, NO = (BV * 64 / VN + 255) / 256;
-  V16 rK[NK], rQ[NK], rW[NK], rO[NO], rD[NO];  // K rows; (scale Q e^G)^T and W^T rows
+  V16 rK[NK], rQ[NK], rW[NK], rO[NO], rD[NO];
+  float rOs[NO];  // scale * e^{G_i} of the dO row each vector belongs to
   float rG = 0.f;
   auto fetch = [&](int n) {
     const int64_t slot = (int64_t)row * N + n;
     int tok0, len;
     chunk_span(p.geom, n, tok0, len);
     const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-    // vector gate: K * e^{G_last - G} was stored by the forward pass (all 64 rows defined)
+    // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)
     const T* Kg = (GATE == LNX_GATE_VECTOR) ? wsp<T>(p, p.off.Kr) + slot * 64 * DK
                                             : reinterpret_cast<const T*>(p.k) + tbase * DK;
-    if (GATE == LNX_GATE_VECTOR) len = 64;
-    const T* Wg = wsp<T>(p, p.off.WT) + slot * DK * 64;
-    const T* Qg = wsp<T>(p, p.off.QgT) + slot * DK * 64;
+    const T* Qg = (GATE == LNX_GATE_VECTOR) ? wsp<T>(p, p.off.Qg) + slot * 64 * DK
+                                            : reinterpret_cast<const T*>(p.q) + tbase * DK;
+    const T* Wg = wsp<T>(p, p.off.W) + slot * 64 * DK;
+    const int klen = (GATE == LNX_GATE_VECTOR) ? 64 : len;
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
       const int idx = tid + 256 * i, r = idx / (DK / VN);
       rK[i] = vec_zero<T>();
-      if (r < len) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
-      rQ[i] = *reinterpret_cast<const V16*>(Qg + (int64_t)idx * VN);
+      rQ[i] = vec_zero<T>();
+      if (r < klen) {
+        rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
+        rQ[i] = *reinterpret_cast<const V16*>(Qg + (int64_t)idx * VN);
+      }
       rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)idx * VN);
     }
-    const T* Og = wsp<T>(p, p.off.dOT) + slot * p.dv * 64 + (int64_t)v0 * 64;
+    const T* Og = reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0;
     const T* Dg = wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0;
 #pragma unroll
     for (int i = 0; i < NO; ++i) {
       const int idx = tid + 256 * i;
       if (idx < BV * 64 / VN) {
-        rO[i] = *reinterpret_cast<const V16*>(Og + (int64_t)idx * VN);
         const int r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
+        rO[i] = vec_zero<T>();
+        if (r < len) rO[i] = *reinterpret_cast<const V16*>(Og + (int64_t)r * p.dv + c);
         rD[i] = *reinterpret_cast<const V16*>(Dg + (int64_t)r * p.dv + c);
+        rOs[i] = (GATE == LNX_GATE_VECTOR) ? 1.f
+                 : (GATE == LNX_GATE_NONE) ? p.scale
+                                           : p.scale * __expf(wsp<float>(p, p.off.G)[slot * 64 + r]);
       }
     }
     if (GATE == LNX_GATE_SCALAR && tid < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + tid];
@@ -188,18 +201,21 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
     for (int i = 0; i < NK; ++i) {
       const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
       *reinterpret_cast<V16*>(sK + r * LDK + c) = rK[i];
-      const int rt = idx / (64 / VN), ct = (idx % (64 / VN)) * VN;
-      *reinterpret_cast<V16*>(sQT + rt * LDC + ct) = rQ[i];
-      *reinterpret_cast<V16*>(sWT + rt * LDC + ct) = rW[i];
+      *reinterpret_cast<V16*>(sQ + r * LDK + c) = rQ[i];
+      *reinterpret_cast<V16*>(sW + r * LDK + c) = rW[i];
     }
 #pragma unroll
     for (int i = 0; i < NO; ++i) {
       const int idx = tid + 256 * i;
       if (idx < BV * 64 / VN) {
-        const int r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
-        *reinterpret_cast<V16*>(sdOT + r * LDC + c) = rO[i];
-        const int r2 = idx / (BV / VN), c2 = (idx % (BV / VN)) * VN;
-        *reinterpret_cast<V16*>(sdDl + r2 * LDU + c2) = rD[i];
+        const int r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
+        V16 o = rO[i];
+        if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}: (scale Q e^G)^T dO = Q^T (that)
+#pragma unroll
+          for (int e = 0; e < VN; ++e) o[e] = from_f32<T>(to_f32(o[e]) * rOs[i]);
+        }
+        *reinterpret_cast<V16*>(sdO + r * LDU + c) = o;
+        *reinterpret_cast<V16*>(sdDl + r * LDU + c) = rD[i];
       }
     }
   };
@@ -227,14 +243,13 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
         d[0][0][e] = to_f32(sdDl[r * LDU + c]) + rj * d[0][0][e];
       }
       frag_store<T, 1, 1>(d, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
-      frag_store_t<T, 1, 1>(d, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)(v0 + 32 * wj) * 64 + 32 * wi, 64, lane);
 #pragma unroll
       for (int e = 0; e < 16; ++e) d[0][0][e] = -d[0][0][e];
       frag_store_t<T, 1, 1>(d, sdDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
     __syncthreads();
 
-    // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD
+    // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD   (token-contracted: rows of the tiles)
     if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
 #pragma unroll
@@ -248,8 +263,8 @@ __global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) dS[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
-    mma_nt<T, 1, NT>(dS, sQT + srow * LDC, LDC, sdOT + scol * LDC, LDC, 64, lane);
-    mma_nt<T, 1, NT>(dS, sWT + srow * LDC, LDC, sdDT + scol * LDC, LDC, 64, lane);
+    mma_x<T, 1, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+    mma_x<T, 1, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     __syncthreads();
   }
   if (p.ds0) {
@@ -317,8 +332,7 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
     sMisc[tid] = 0.f;
   }
 
-  TileRegs<T, 64, 64> rdO, rD, rdD, rdSn;
-  TileRegsT<T, 64, 64> rSn;
+  TileRegs<T, 64, 64> rdO, rD, rdD, rdSn, rSn;  // S_n slab stays [v][c]: contracted along its rows
   auto fetch = [&](int v0) {
     rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
     rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
@@ -343,16 +357,17 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
     __syncthreads();
     if (v0 + 64 < p.dv) fetch(v0 + 64);
     mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDC, LDC, sD + 32 * wj * LDC, LDC, 64, lane);
-    mma_nt<T, 1, 1>(aQ, sdO + 32 * wi * LDC, LDC, sSn + 32 * wj * LDC, LDC, 64, lane);
-    mma_nt<T, 1, 1>(aW, sdD + 32 * wi * LDC, LDC, sSn + 32 * wj * LDC, LDC, 64, lane);
+    mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDC, LDC, sSn + 32 * wj, LDC, 64, lane);
+    mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDC, LDC, sSn + 32 * wj, LDC, 64, lane);
     mma_nt<T, 1, 1>(aK, sD + 32 * wi * LDC, LDC, sdSn + 32 * wj * LDC, LDC, 64, lane);
     if (GATE != LNX_GATE_NONE) {  // thread = (channel row tid / 4, quarter of the slab)
       const int r = tid >> 2, q4 = (tid & 3) * 16;
       float t = 0.f;
 #pragma unroll
       for (int e = 0; e < 16; e += 4) {
-        const floatx4 x = load4(sSn + r * LDC + q4 + e), y = load4(sdSn + r * LDC + q4 + e);
-        t += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+        const floatx4 y = load4(sdSn + r * LDC + q4 + e);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t += to_f32(sSn[(q4 + e + u) * LDC + r]) * y[u];
       }
       ss += t;
     }
@@ -444,14 +459,13 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
     if (tid < 64) dGg[63 * DK + tid] += dgc;
   } else {
     // ---- scalar / no gate ----
-    T* sPe = sdO;
-    T* sPeT = sD;
-    T* sKT = sdD;
-    T* sQT = sSn;
+    T* sPe = sdO;     // scale E dP   [i][j]
+    T* sOut2 = sD;    // staging for dk
+    T* sKr = sdD;     // K rows of this half [token][c]
+    T* sQr = sSn;     // Q rows
     T* sOut = sdSn;
-    TileRegs<T, 64, 64> rKT;
-    TileRegsT<T, 64, 64> rQT;
-    rKT.load(wsp<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)ch0 * 64, 64, 64, tid);
+    TileRegs<T, 64, 64> rKT, rQT;
+    rKT.load(kg, DK, len, tid);
     rQT.load(qg, DK, len, tid);
     {
       floatx16 pe[1][1], nw[1][1];
@@ -463,11 +477,10 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
         nw[0][0][e] = -aW[0][0][e];
       }
       frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
-      frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
       frag_store<T, 1, 1>(nw, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
     }
-    rKT.store(sKT, LDC, tid);
-    rQT.store(sQT, LDC, tid);
+    rKT.store(sKr, LDC, tid);
+    rQT.store(sQr, LDC, tid);
     __syncthreads();
     unstage_tile<T, 64, 64>(wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0, DK, sOut, LDC, 64, tid);
     // inter-chunk parts scaled, then the intra-chunk products on top
@@ -480,28 +493,29 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
       const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
       aQ[0][0][e] *= gq;
       aK[0][0][e] *= gk;
-      tot += aK[0][0][e] * to_f32(sKT[c * LDC + r]);
+      tot += aK[0][0][e] * to_f32(sKr[r * LDC + c]);
     }
-    mma_nt<T, 1, 1>(aQ, sPe + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
-    mma_nt<T, 1, 1>(aK, sPeT + 32 * wi * LDC, LDC, sQT + 32 * wj * LDC, LDC, 64, lane);
+    // dq += dPe K,  dk += dPe^T Q: K, Q (and dPe for the second product) contracted along tile rows
+    mma_x<T, 1, 1, false, true>(aQ, sPe + 32 * wi * LDC, LDC, sKr + 32 * wj, LDC, 64, lane);
+    mma_x<T, 1, 1, true, true>(aK, sPe + 32 * wi, LDC, sQr + 32 * wj, LDC, 64, lane);
     if (GATE != LNX_GATE_NONE) {
       // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts)
       float v[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        v[e] = aQ[0][0][e] * to_f32(sQT[c * LDC + r]) - aK[0][0][e] * to_f32(sKT[c * LDC + r]);
+        v[e] = aQ[0][0][e] * to_f32(sQr[r * LDC + c]) - aK[0][0][e] * to_f32(sKr[r * LDC + c]);
       }
       rows_reduce_add<1>(v, 32 * wi, lane, sdG);
       tot = wave_sum(tot);
       if (lane == 0) atomicAdd(&sMisc[0], tot);
     }
-    __syncthreads();  // all reads of sPe / sPeT / sOut done
+    __syncthreads();  // all reads of sPe / sOut done
     frag_store<T, 1, 1>(aQ, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
-    frag_store<T, 1, 1>(aK, sPeT + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store<T, 1, 1>(aK, sOut2 + 32 * wi * LDC + 32 * wj, LDC, lane);
     __syncthreads();
     unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, DK, sPe, LDC, len, tid);
-    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sPeT, LDC, len, tid);
+    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sOut2, LDC, len, tid);
     if (GATE != LNX_GATE_NONE && tid < 64) {
       float d = sdG[tid];
       if (tid == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
@@ -576,7 +590,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   T* sU = R3;
   for (int v0 = 0; v0 < p.dv; v0 += 64) {
     __syncthreads();
-    stage_tile<T, 64, 64>(sdDT, LDC, wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, tid);
+    stage_tile_t<T, 64, 64>(sdDT, LDC, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     stage_tile<T, 64, 64>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     __syncthreads();
     floatx16 bu[1][1];
@@ -604,7 +618,8 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
   __syncthreads();
 
-  if constexpr (GATE == LNX_GATE_VECTOR) {
+  static_assert(GATE == LNX_GATE_VECTOR, "bwd_wy2 handles the other gate kinds");
+  {
     // ---- per-channel gate ----
     float* sAl = reinterpret_cast<float*>(R1);  // [64][LDF]
     float* sOp = sAl + 64 * LDF;                // row-type part of dk (through B_w and the rows of X)
@@ -669,84 +684,6 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
         if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
       }
     }
-  } else {
-    // ---- scalar / no gate ----
-    // phase 4: X = K K^T (recomputed), dA = -tril(dM, -1), Y = sym(beta dA E), R = dA * E X
-    T* sK = R3;
-    T* sY = R1;
-    stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
-    __syncthreads();
-    {
-      floatx16 x[1][1];
-      frag_zero(x);
-      if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(x, sK + 32 * wi * LDK, LDK, sK + 32 * wj * LDK, LDK, DK, lane);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-        const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-        const float da = (i > j) ? -aM[0][0][e] : 0.f;
-        sR[i * LNX_LDA + j] = da * dec * x[0][0][e];
-        const T y = from_f32<T>(sBeta[i] * da * dec);
-        if (i > j) {
-          sY[i * LDC + j] = y;
-          sY[j * LDC + i] = y;
-        } else if (i == j) {
-          sY[i * LDC + j] = from_f32<T>(0.f);
-        }
-      }
-    }
-    // dk (row-type part through B_w): beta e^{G} dBw, with its dbeta / gate terms
-    frag_rowdot<MT>(aBw, r0, c0, lane, sdG, [&](int r, int c) {
-      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
-      return (r < len) ? gm * to_f32(kg[(int64_t)r * DK + c]) : 0.f;
-    });
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = r0 + 32 * i + frag_row(e, lane);
-        const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
-        aBw[i][0][e] *= sBeta[r] * gm;
-      }
-    __syncthreads();  // sdBw (R2) no longer read; sY, sR complete
-
-    // phase 5: dk += Y K, added to the partial dk of bwd_dqk
-    T* sKT = R2;
-    stage_tile<T, DK, 64>(sKT, LDC, wsp<T>(p, p.off.KT) + slot * DK * 64, 64, DK, tid);
-    __syncthreads();
-    mma_nt<T, MT, 1>(aBw, sY + r0 * LDC, LDC, sKT + c0 * LDC, LDC, 64, lane);
-    {
-      T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
-          if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + aBw[i][0][e]);
-        }
-    }
-    // dbeta and dg
-    if (wave == 0) {
-      const int t = lane;
-      float rs = 0.f, cs = 0.f;
-      for (int j = 0; j < 64; ++j) {
-        rs += sR[t * LNX_LDA + j];
-        cs += sBeta[j] * sR[j * LNX_LDA + t];
-      }
-      // sdG[t] holds e^{G_t} <dBw_t, k_t>
-      const float w = sdG[t];
-      if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
-      if (GATE != LNX_GATE_NONE) {
-        float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - cs;
-        // reverse inclusive cumsum over the chunk
-#pragma unroll
-        for (int s_ = 1; s_ < 64; s_ <<= 1) {
-          const float y = __shfl_down(d, s_, LNX_WAVE);
-          if (t + s_ < 64) d += y;
-        }
-        if (t < len) p.dg[tbase + t] = d;
-      }
-    }
   }
 }
 
@@ -802,17 +739,16 @@ __global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
   }
   stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
 
-  TileRegsT<T, 64, 64> rInT;        // dW slab, transposed on the way to LDS
-  TileRegs<T, 64, 64> rIn, rWU, rKs;
+  TileRegs<T, 64, 64> rIn, rWU, rKs;  // dW / dD slab [token][col], W / U slab, K / V slab
   auto fetch = [&](int s_) {
     if (s_ < NKS) {
       const int c0 = 64 * s_;
-      rInT.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
+      rIn.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
       rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
       rKs.load(kg + c0, DK, len, tid);
     } else {
       const int v0 = 64 * (s_ - NKS);
-      rIn.load(wsp<T>(p, p.off.dDT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, 64, tid);
+      rIn.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       rKs.load(vg + v0, p.dv, len, tid);
     }
@@ -828,14 +764,14 @@ __global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ < NKS;
     __syncthreads();
-    if (is_k) rInT.store(sIn, LDC, tid); else rIn.store(sIn, LDC, tid);
+    rIn.store(sIn, LDC, tid);
     rWU.store(sWU, LDC, tid);
     rKs.store(sKs, LDC, tid);
     __syncthreads();
     if (s_ + 1 < nslab) fetch(s_ + 1);
     floatx16 b[1][1];
     frag_zero(b);
-    mma_nt<T, 1, 1>(b, sTmT + 32 * wi * LDC, LDC, sIn + 32 * wj * LDC, LDC, 64, lane);
+    mma_x<T, 1, 1, false, true>(b, sTmT + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
     frag_store<T, 1, 1>(b, sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
     {
       float v[16];
@@ -871,16 +807,15 @@ __global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
       }
     }
   }
-  // K^T slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
+  // K slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
   TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
 #pragma unroll
   for (int u = 0; u < NKS; ++u) {
-    rKT[u].load(wsp<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)(64 * u) * 64, 64, 64, tid);
+    rKT[u].load(kg + 64 * u, DK, len, tid);  // K rows again, for Y K
     rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, DK, len, tid);
   }
   __syncthreads();  // loop tiles dead
-  T* sYa = sIn;   // beta dA E (strictly lower)
-  T* sYb = sWU;   // its transpose
+  T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
     floatx16 y[1][1];
     float v[16], cs = 0.f;
@@ -894,7 +829,6 @@ __global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
       y[0][0][e] = sBeta[i] * da;
     }
     frag_store<T, 1, 1>(y, sYa + 32 * wi * LDC + 32 * wj, LDC, lane);
-    frag_store_t<T, 1, 1>(y, sYb + 32 * wj * LDC + 32 * wi, LDC, lane);
     rows_reduce_add<1>(v, 32 * wi, lane, sRow);
     cs += __shfl_xor(cs, 32, LNX_WAVE);
     if (lane < 32) atomicAdd(&sCol[32 * wj + lane], cs);
@@ -914,8 +848,8 @@ __global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
       const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
       aBw[u][0][0][e] *= sBeta[r] * gm;
     }
-    mma_nt<T, 1, 1>(aBw[u], sYa + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
-    mma_nt<T, 1, 1>(aBw[u], sYb + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
+    mma_x<T, 1, 1, false, true>(aBw[u], sYa + 32 * wi * LDC, LDC, sKT + 32 * wj, LDC, 64, lane);
+    mma_x<T, 1, 1, true, true>(aBw[u], sYa + 32 * wi, LDC, sKT + 32 * wj, LDC, 64, lane);
     if (u > 0) __syncthreads();
     frag_store<T, 1, 1>(aBw[u], sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
     __syncthreads();

@@ -6,19 +6,20 @@
 // reserved and a table built on the device maps slot -> (first token, length, sequence);
 // unused slots have length 0.
 //
-// Per-slot tensors kept in the workspace (element type T = bf16 or fp32 unless noted):
+// Per-slot tensors kept in the workspace (element type T = bf16 or fp32 unless noted), all
+// row-major with the token index first; kernels that contract over tokens read them through
+// the transposing LDS loads of mma_tiles.h, so no transposed copies are stored:
 //   G    fp32 [64] or [64][dk]   cumulative gate inside the chunk
 //   P    [64][64]   scale * <q_i, k_j> * exp(G_i - G_j), i >= j
 //   W    [64][dk]   (I + A)^-1 diag(beta) (K * exp(G))
 //   U    [64][dv]   (I + A)^-1 diag(beta) V
-//   KT   [dk][64]   K^T (scalar / no gate) or (K * exp(G_last - G))^T (vector gate)
-//   WT   [dk][64]   W^T            QgT [dk][64]  (scale * Q * exp(G))^T
 //   TmT  [64][64]   ((I + A)^-1)^T, used by the backward pass
-//   X    [64][64]   <k_i, k_j>_E, i > j, and  Kr [64][dk] = K * exp(G_last - G)   (vector gate only)
-//   D    [64][dv]   U - W S            DT [dv][64] its transpose
+//   D    [64][dv]   U - W S
 //   SnT  [dv][dk]   transpose of the state entering the chunk
-// Backward adds dOT [dv][64], dD [64][dv], dDT [dv][64], dSn [dk][dv] (gradient of the state
-// leaving the chunk), dW [64][dk] and dG (fp32 partial gradient of the cumulative gate).
+//   vector gate only:  X [64][64] = <k_i, k_j>_E (i > j),  Kr [64][dk] = K * exp(G_last - G),
+//                      Qg [64][dk] = scale * Q * exp(G)
+// Backward adds dD [64][dv], dSn [dk][dv] (gradient of the state leaving the chunk), dW [64][dk]
+// and dG (fp32 partial gradient of the cumulative gate).
 #pragma once
 
 #include "mma_tiles.h"
@@ -62,7 +63,7 @@ __device__ __forceinline__ bool xcd_slot_part(int64_t slots, int parts, int64_t&
 inline unsigned lnx_xcd_grid(int64_t slots, int parts) { return (unsigned)(((slots + 7) / 8) * 8 * parts); }
 
 struct ChunkWs {
-  uint64_t tab, G, P, X, W, WT, QgT, U, KT, Kr, TmT, D, DT, SnT, dOT, dD, dDT, dSn, dW, dG, total;
+  uint64_t tab, G, P, X, W, U, Kr, Qg, TmT, D, SnT, dD, dSn, dW, dG, total;
 };
 
 inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
@@ -84,18 +85,13 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.P = take(slots * C * C * es);
   w.X = take(a->gate == LNX_GATE_VECTOR ? slots * C * C * es : 0);
   w.W = take(slots * C * dk * es);
-  w.WT = take(slots * dk * C * es);
-  w.QgT = take(slots * dk * C * es);
   w.U = take(slots * C * dv * es);
-  w.KT = take(slots * dk * C * es);
   w.Kr = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * es : 0);
+  w.Qg = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * es : 0);
   w.TmT = take(slots * C * C * es);
   w.D = take(slots * C * dv * es);
-  w.DT = take(slots * dv * C * es);
   w.SnT = take(slots * dv * dk * es);
-  w.dOT = take(slots * dv * C * es);
   w.dD = take(slots * C * dv * es);
-  w.dDT = take(slots * dv * C * es);
   w.dSn = take(slots * dk * dv * es);
   w.dW = take(slots * C * dk * es);
   w.dG = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);

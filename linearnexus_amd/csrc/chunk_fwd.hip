@@ -6,7 +6,7 @@
 //       P = scale * tril(Q K^T * E);  also K^T and Tm^T for later kernels.
 //   chunk_scan     (one workgroup per (state, 64-column slab of dv), sequential over chunks)
 //       D = U - W S;  S <- e^{G_last} S + (K e^{G_last - G})^T D, with the fp32 state held in
-//       MFMA accumulators across the whole sequence; stores D, D^T and the entering state.
+//       MFMA accumulators across the whole sequence; stores D and the entering state.
 //   chunk_output   (one workgroup per (chunk, 64-column slab), all in parallel)
 //       O = scale (Q e^G) S_n + P D.
 //
@@ -52,14 +52,14 @@ __device__ __forceinline__ float wave_cumsum(float x, int lane) {
 // chunk_prepare2 (no gate / scalar gate): the same computation as chunk_prepare, organised as
 // slab loops with register prefetch so that two workgroups fit a CU: K K^T and Q K^T over
 // 64-channel slabs, the fp32 inverse, then one 64-column slab of [dk | dv] at a time for
-// W / W^T / K^T / Qg^T and U, every result leaving through LDS with 16-byte stores.
+// W and U, every result leaving through LDS with 16-byte stores.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct Prep2Cfg {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kTile = 64 * LDC;
   static constexpr size_t f32_bytes = sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36);
-  static constexpr size_t regionF = (4 * kTile * sizeof(T) > f32_bytes) ? 4 * kTile * sizeof(T) : f32_bytes;
+  static constexpr size_t regionF = (2 * kTile * sizeof(T) > f32_bytes) ? 2 * kTile * sizeof(T) : f32_bytes;
   static constexpr size_t bytes = regionF + 2 * kTile * sizeof(T) + sizeof(float) * 128;
 };
 
@@ -73,8 +73,6 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   float* sX = sT + 64 * LNX_LDA;
   T* sIn = reinterpret_cast<T*>(smem);  // overlays the fp32 matrices once Tw / Tu exist
   T* sOut = sIn + L::kTile;
-  T* sOut2 = sOut + L::kTile;
-  T* sQg = sOut2 + L::kTile;
   T* sKa = reinterpret_cast<T*>(smem + L::regionF);  // K slab, then Tw
   T* sQa = sKa + L::kTile;                           // Q slab, then Tu
   float* sBeta = reinterpret_cast<float*>(sQa + L::kTile);
@@ -124,14 +122,10 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     }
   }
   // first slab of the second loop, in flight during the inverse
-  TileRegsT<T, 64, 64> rInT, rQT;
+  TileRegs<T, 64, 64> rIn;
   auto fetch = [&](int s_) {
-    if (s_ < NKS) {
-      rInT.load(kg + 64 * s_, DK, len, tid);
-      rQT.load(qg + 64 * s_, DK, len, tid);
-    } else {
-      rInT.load(vg + 64 * (s_ - NKS), p.dv, len, tid);
-    }
+    if (s_ < NKS) rIn.load(kg + 64 * s_, DK, len, tid);
+    else rIn.load(vg + 64 * (s_ - NKS), p.dv, len, tid);
   };
   fetch(0);
   __syncthreads();  // slab tiles dead
@@ -168,26 +162,19 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ < NKS;
     __syncthreads();  // fp32 matrices / previous slab's tiles are dead
-    rInT.store(sIn, LDC, tid);
-    if (is_k)
-      rQT.store(sQg, LDC, tid, [&](int r, int) { return (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]); });
+    rIn.store(sIn, LDC, tid);
     __syncthreads();
     if (s_ + 1 < nslab) fetch(s_ + 1);
     floatx16 acc[1][1];
     frag_zero(acc);
-    mma_nt<T, 1, 1>(acc, (is_k ? sKa : sQa) + 32 * wi * LDC, LDC, sIn + 32 * wj * LDC, LDC, 64, lane);
+    // W = Tw K, U = Tu V: the slab is [token][column], contracted along its rows
+    mma_x<T, 1, 1, false, true>(acc, (is_k ? sKa : sQa) + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
     frag_store<T, 1, 1>(acc, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
-    if (is_k) frag_store_t<T, 1, 1>(acc, sOut2 + 32 * wj * LDC + 32 * wi, LDC, lane);
     __syncthreads();
-    if (is_k) {
-      const int c0 = 64 * s_;
-      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + c0, DK, sOut, LDC, 64, tid);
-      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sOut2, LDC, 64, tid);
-      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sIn, LDC, 64, tid);
-      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64 + (int64_t)c0 * 64, 64, sQg, LDC, 64, tid);
-    } else {
+    if (is_k)
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + 64 * s_, DK, sOut, LDC, 64, tid);
+    else
       unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + 64 * (s_ - NKS), p.dv, sOut, LDC, 64, tid);
-    }
   }
 }
 
@@ -253,14 +240,20 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   {
     float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
     T* Krg = ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK;
+    T* Qgg = ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK;
     for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
       const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
       const floatx4 gr = load4(sG + r * LDF + c), gl = load4(sG + 63 * LDF + c), kk = load4(sK + r * LDK + c);
       store4(Gg + r * DK + c, gr);
-      floatx4 kr;
+      const floatx4 qq = load4(sQ + r * LDK + c);
+      floatx4 kr, qgv;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) kr[e] = kk[e] * __expf(fminf(gl[e] - gr[e], 0.f));
+      for (int e = 0; e < 4; ++e) {
+        kr[e] = kk[e] * __expf(fminf(gl[e] - gr[e], 0.f));
+        qgv[e] = qq[e] * p.scale * __expf(gr[e]);
+      }
       store4(Krg + r * DK + c, kr);
+      store4(Qgg + r * DK + c, qgv);
     }
   }
   // pairwise products with the decay inside the channel sum
@@ -289,10 +282,7 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
     }
   }
   __syncthreads();
-  // (scale * Q * e^G)^T through the sQ region
-  stage_tile_t<T, 64, DK>(sQ, LDC, qg, DK, len, tid, [&](int r, int c) { return p.scale * __expf(sG[r * LDF + c]); });
   tri_inverse_64(sA, sT, sX, tid);
-  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.QgT) + slot * DK * 64, 64, sQ, LDC, DK, tid);
 
   T* sTm = sK;                         // T-typed copy of Tm (bf16); fp32 reads sT in place
   T* sTu = reinterpret_cast<T*>(sA);   // Tm * diag(beta)
@@ -320,14 +310,9 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
       frag_zero(acc);
       mma_nt<T, 1, 1>(acc, tm_op + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
       frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
-      frag_store_t<T, 1, 1>(acc, ws_ptr<T>(p, p.off.WT) + slot * DK * 64 + (int64_t)(c0 + 32 * wj) * 64 + 32 * wi, 64, lane);
     }
   }
   __syncthreads();
-  // (K * e^{G_last - G})^T for the scan kernel
-  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid, [&](int r, int c) { return __expf(fminf(sG[63 * LDF + c] - sG[r * LDF + c], 0.f)); });
-  __syncthreads();
-  unstage_tile<T, DK, 64>(ws_ptr<T>(p, p.off.KT) + slot * DK * 64, 64, sKT, LDC, DK, tid);
   // U = Tu V
   {
     T* sVT = sQ;
@@ -352,7 +337,7 @@ template <typename T, int DK> struct ScanSmem {
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int BV = 64;
-  static constexpr int kW = 64 * LDK, kKT = DK * LDC, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
+  static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 128;
 };
 
@@ -367,8 +352,8 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   constexpr int NT = (DK == 128) ? 2 : 1;
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
-  T* sKT = sW + L::kW;
-  T* sU = sKT + L::kKT;
+  T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
+  T* sU = sK + L::kKT;
   T* sST = sU + L::kU;
   T* sDT = sST + L::kST;
   float* sG = reinterpret_cast<float*>(sDT + L::kDT);
@@ -401,12 +386,20 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   auto fetch = [&](int n) {
     const int64_t slot = (int64_t)row * N + n;
     const T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
-    const T* Kg = ws_ptr<T>(p, p.off.KT) + slot * DK * 64;
+    int tok0, len;
+    chunk_span(p.geom, n, tok0, len);
+    const T* Kg = (GATE == LNX_GATE_VECTOR) ? ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK
+                                            : reinterpret_cast<const T*>(p.k) + ((int64_t)row * p.geom.T + tok0) * DK;
+    if (GATE == LNX_GATE_VECTOR) len = 64;
     const T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0;
 #pragma unroll
     for (int i = 0; i < NW; ++i) rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)(tid + 256 * i) * VN);
 #pragma unroll
-    for (int i = 0; i < NK; ++i) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)(tid + 256 * i) * VN);
+    for (int i = 0; i < NK; ++i) {
+      const int idx = tid + 256 * i;
+      rK[i] = vec_zero<T>();
+      if (idx / (DK / VN) < len) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
+    }
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
@@ -423,8 +416,8 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     }
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
-      const int idx = tid + 256 * i, r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
-      *reinterpret_cast<V16*>(sKT + r * LDC + c) = rK[i];
+      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
+      *reinterpret_cast<V16*>(sK + r * LDK + c) = rK[i];
     }
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
@@ -457,8 +450,6 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     }
     frag_store<T, 1, 1>(d, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj,
                         p.dv, lane);
-    frag_store_t<T, 1, 1>(d, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)(v0 + 32 * wj) * 64 + 32 * wi, 64,
-                          lane);
     if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
@@ -480,7 +471,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) S[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
-    mma_nt<T, 1, NT>(S, sKT + srow * LDC, LDC, sDT + scol * LDC, LDC, 64, lane);
+    mma_x<T, 1, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
     __syncthreads();
   }
 
@@ -545,7 +536,7 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   }
   stage_tile<T, BV, DK>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, tid);
   stage_tile<T, 64, 64>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
-  stage_tile<T, BV, 64>(sDT, LDC, ws_ptr<T>(p, p.off.DT) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, BV, tid);
+  stage_tile<T, 64, BV>(sDT, LDC, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);  // D rows [token][v]
   if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
   __syncthreads();
 
@@ -558,7 +549,7 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
     const float gm = (GATE == LNX_GATE_VECTOR) ? 1.f : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
     acc[0][0][e] *= gm;
   }
-  mma_nt<T, 1, 1>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj * LDC, LDC, 64, lane);
+  mma_x<T, 1, 1, false, true>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj, LDC, 64, lane);
   const int64_t obase = (tbase + 32 * wi) * p.dv + v0 + 32 * wj;
   if (p.o_dtype == LNX_BF16)
     frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, p.dv, lane, len - 32 * wi);

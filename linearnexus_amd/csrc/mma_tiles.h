@@ -28,6 +28,21 @@ template <> struct Mma<bf16_t> {
   static __device__ __forceinline__ void mma(floatx16& c, const Frag& a, const Frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // Operand fragment whose contraction index runs along the ROWS of a row-major LDS tile:
+  // lane (r = lane & 31, kg = lane >> 5) gets tile[k0 + 8 kg + 0..7][c0 + r].  Two
+  // ds_read_b64_tr_b16: inside a 16-lane group, result element j of lane L is element (L % 4) of
+  // what lane 4 j + L / 4 addressed, so source lane s = 4 j + q points at row j, columns 4 q .. 4 q + 3.
+  static __device__ __forceinline__ Frag load_t(const bf16_t* tile, int ld, int k0, int c0, int lane) {
+    typedef short short4_ __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) short4_ lds_short4;
+    const int s = lane & 15, grp = lane >> 4;
+    const bf16_t* p = tile + (k0 + 8 * (grp >> 1) + (s >> 2)) * ld + c0 + 16 * (grp & 1) + 4 * (s & 3);
+    const short4_ lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p));
+    const short4_ hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p + 4 * ld));
+    typedef short short8_ __attribute__((ext_vector_type(8)));
+    const short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(Frag, v);
+  }
 };
 
 template <> struct Mma<float> {
@@ -40,6 +55,12 @@ template <> struct Mma<float> {
   static __device__ __forceinline__ void mma(floatx16& c, const Frag& a, const Frag& b) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+  }
+  // fp32: one element per MFMA, so the transposed-source fragment is four conflict-free scalar reads
+  static __device__ __forceinline__ Frag load_t(const float* tile, int ld, int k0, int c0, int lane) {
+    const float* p = tile + (k0 + 4 * (lane >> 5)) * ld + c0 + (lane & 31);
+    Frag v = {p[0], p[ld], p[2 * ld], p[3 * ld]};
+    return v;
   }
 };
 
@@ -67,6 +88,29 @@ __device__ __forceinline__ void mma_nt(floatx16 (&acc)[MT][NT], const T* A, int 
     for (int i = 0; i < MT; ++i) a[i] = M::load(ap + i * 32 * lda + k0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) b[j] = M::load(bp + j * 32 * ldb + k0);
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) M::mma(acc[i][j], a[i], b[j]);
+  }
+}
+
+// General form: TA / TB say that the operand is given as a row-major [K][rows] tile (contraction
+// index along the tile's rows; A / B then point at the tile's first used column) instead of the
+// native [rows][K] layout.
+template <typename T, int MT, int NT, bool TA, bool TB>
+__device__ __forceinline__ void mma_x(floatx16 (&acc)[MT][NT], const T* A, int lda, const T* B, int ldb, int K,
+                                      int lane) {
+  typedef Mma<T> M;
+  const int r = lane & 31, ko = (lane >> 5) * M::VEC;
+  for (int k0 = 0; k0 < K; k0 += M::KS) {
+    typename M::Frag a[MT], b[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      a[i] = TA ? M::load_t(A, lda, k0, 32 * i, lane) : M::load(A + (r + 32 * i) * lda + ko + k0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      b[j] = TB ? M::load_t(B, ldb, k0, 32 * j, lane) : M::load(B + (r + 32 * j) * ldb + ko + k0);
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
