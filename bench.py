@@ -32,7 +32,12 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
-TRAFFIC = {}
+TRAFFIC = {
+    ("gdn_chunk", "chunk_prepare"): 827333560, ("gdn_chunk", "chunk_scan"): 815944299,
+    ("gdn_chunk", "chunk_output"): 740377023, ("gdn_chunk", "bwd_local"): 337702140,
+    ("gdn_chunk", "bwd_scan"): 1084422711, ("gdn_chunk", "bwd_dqk"): 1617126440,
+    ("gdn_chunk", "bwd_wy"): 1394292784, ("decode", "decode_step"): 1083445231,
+}
 
 
 def chunk_flops(dk, dv):
@@ -210,7 +215,8 @@ def bench_decode(args, torch, la, _lib, steps=None):
         "workload": "gated_deltanet_decode_step", "B": B, "H": H, "dk": d, "dv": d, "steps": steps,
         "ms_per_step": dt * 1e3, "tokens_per_s": B / dt, "bytes_per_step": nbytes,
         "roofline": {"bound": "hbm", "kernel": "decode_step", "achieved": nbytes / (kms * 1e-3) / 1e9, "peak": PEAK_HBM,
-                     "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / PEAK_HBM, "traffic": None},
+                     "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / PEAK_HBM,
+                     "traffic": TRAFFIC.get(("decode", "decode_step"))},
     }
 
 
@@ -221,6 +227,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: the scan needs no collective and every figure here is "
@@ -246,6 +254,13 @@ def main():
         print(json.dumps(out))
         return
 
+    if args.calibrate:
+        a = torch.empty(512 * 1024 * 1024 // 4, device="cuda:0").normal_()
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     out, (B, H, T, d) = bench_chunk(args, torch, la, _lib, args.workload)
     if args.workload == "gdn_chunk":
         out["decode_step"] = bench_decode(args, torch, la, _lib)

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int BV = (sizeof(T) == 4 && DK == 128) ? 32 : 64;  // dv slab per workgroup
+  static constexpr int BV = (DK == 128) ? 32 : 64;  // dv slab per workgroup
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
@@ -109,7 +109,7 @@ template <typename T, int DK> struct BScanCfg {
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void bwd_scan_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel(BwdParams p) {
   typedef BScanCfg<T, DK> L;
   typedef typename Vec16<T>::V V16;
   constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV, VN = Vec16<T>::N;
