@@ -295,7 +295,7 @@ template <typename T, int DK, int GATE> struct DqkCfg {
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3 : 1)) void bwd_dqk_kernel(BwdParams p) {
   typedef DqkCfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF;
   extern __shared__ __align__(16) char smem[];
@@ -332,12 +332,16 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
     sMisc[tid] = 0.f;
   }
 
-  TileRegs<T, 64, 64> rdO, rD, rdD, rdSn, rSn;  // S_n slab stays [v][c]: contracted along its rows
+  // dv is consumed in slabs of SV columns; narrow slabs keep the prefetch registers few enough
+  // for three waves per SIMD
+  constexpr int SV = 32, LDS_ = SV + Mma<T>::PAD;
+  TileRegs<T, 64, SV> rdO, rD, rdD, rdSn;
+  TileRegs<T, SV, 64> rSn;  // S_n slab stays [v][c]: contracted along its rows
   auto fetch = [&](int v0) {
     rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
     rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, 64, tid);
+    rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
     rdSn.load(wsp<T>(p, p.off.dSn) + slot * DK * p.dv + (int64_t)ch0 * p.dv + v0, p.dv, 64, tid);
   };
   floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
@@ -347,25 +351,26 @@ __global__ __launch_bounds__(256) void bwd_dqk_kernel(BwdParams p) {
   frag_zero(aK);
   float ss = 0.f;
   fetch(0);
-  for (int v0 = 0; v0 < p.dv; v0 += 64) {
+  for (int v0 = 0; v0 < p.dv; v0 += SV) {
     __syncthreads();
-    rdO.store(sdO, LDC, tid);
-    rD.store(sD, LDC, tid);
-    rdD.store(sdD, LDC, tid);
+    rdO.store(sdO, LDS_, tid);
+    rD.store(sD, LDS_, tid);
+    rdD.store(sdD, LDS_, tid);
     rSn.store(sSn, LDC, tid);
-    rdSn.store(sdSn, LDC, tid);
+    rdSn.store(sdSn, LDS_, tid);
     __syncthreads();
-    if (v0 + 64 < p.dv) fetch(v0 + 64);
-    mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDC, LDC, sD + 32 * wj * LDC, LDC, 64, lane);
-    mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDC, LDC, sSn + 32 * wj, LDC, 64, lane);
-    mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDC, LDC, sSn + 32 * wj, LDC, 64, lane);
-    mma_nt<T, 1, 1>(aK, sD + 32 * wi * LDC, LDC, sdSn + 32 * wj * LDC, LDC, 64, lane);
+    if (v0 + SV < p.dv) fetch(v0 + SV);
+    mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDS_, LDS_, sD + 32 * wj * LDS_, LDS_, SV, lane);
+    mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
+    mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
+    mma_nt<T, 1, 1>(aK, sD + 32 * wi * LDS_, LDS_, sdSn + 32 * wj * LDS_, LDS_, SV, lane);
     if (GATE != LNX_GATE_NONE) {  // thread = (channel row tid / 4, quarter of the slab)
-      const int r = tid >> 2, q4 = (tid & 3) * 16;
+      constexpr int QV = SV / 4;
+      const int r = tid >> 2, q4 = (tid & 3) * QV;
       float t = 0.f;
 #pragma unroll
-      for (int e = 0; e < 16; e += 4) {
-        const floatx4 y = load4(sdSn + r * LDC + q4 + e);
+      for (int e = 0; e < QV; e += 4) {
+        const floatx4 y = load4(sdSn + r * LDS_ + q4 + e);
 #pragma unroll
         for (int u = 0; u < 4; ++u) t += to_f32(sSn[(q4 + e + u) * LDC + r]) * y[u];
       }
@@ -534,7 +539,7 @@ template <typename T, int DK, int GATE> struct WyCfg {
   static constexpr int kR2 = (128 * LDC > 64 * LDK) ? 128 * LDC : 64 * LDK;  // dW^T | dD^T + dBu | dBw | K^T
   static constexpr int kR3 = 64 * LDK;                                       // U slab | W | K
   static constexpr size_t mma_bytes = sizeof(T) * (kR1 + kR2 + kR3);
-  static constexpr size_t vec_bytes = sizeof(float) * 3 * 64 * LDF + sizeof(T) * 64 * LDK;  // alpha, out+, out-, K
+  static constexpr size_t vec_bytes = sizeof(float) * 3 * 64 * LDF + sizeof(T) * 64 * LDK;  // alpha, out+, out-, K (X borrows out-)
   static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > mma_bytes) ? vec_bytes : mma_bytes;
   static constexpr size_t bytes = sizeof(float) * (64 * LNX_LDA + 64 * 4) + big;
 };
@@ -625,20 +630,33 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     float* sOp = sAl + 64 * LDF;                // row-type part of dk (through B_w and the rows of X)
     float* sOm = sOp + 64 * LDF;                // column-type part of dk (columns of X)
     T* sKr = reinterpret_cast<T*>(sOm + 64 * LDF);
+    T* sXp = reinterpret_cast<T*>(sOm);  // X = <k_i, k_j>_E from the forward pass, until out- is needed
     const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
     float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
-    const T* Xg = wsp<T>(p, p.off.X) + slot * 64 * 64;
+    stage_tile<T, 64, 64>(sXp, LDC, wsp<T>(p, p.off.X) + slot * 64 * 64, 64, 64, tid);
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
     }
     stage_tile<T, 64, DK>(sKr, LDK, kg, DK, len, tid);
-    for (int idx = tid; idx < 64 * DK; idx += 256) {
-      const int r = idx / DK, c = idx % DK;
-      const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
-      sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
-      sOm[r * LDF + c] = 0.f;
+    {
+      constexpr int IT = 64 * DK / 4 / 256;
+      floatx4 g1[IT], g0[IT];
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+        g1[it] = load4(Gg + r * DK + c);
+        g0[it] = (r > 0) ? load4(Gg + (r - 1) * DK + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+        floatx4 a4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a4[e] = __expf(fminf(g1[it][e] - g0[it][e], 0.f));
+        store4(sAl + r * LDF + c, a4);
+      }
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -650,7 +668,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     __syncthreads();
     if (tid < 64) {  // dbeta += sum_j dA_ij X_ij
       float rs = 0.f;
-      for (int j = 0; j < tid; ++j) rs += sR[tid * LNX_LDA + j] * to_f32(Xg[tid * 64 + j]);
+      for (int j = 0; j < tid; ++j) rs += sR[tid * LNX_LDA + j] * to_f32(sXp[tid * LDC + j]);
       atomicAdd(&sdB[tid], rs);
     }
     for (int r = wave; r < 64; r += 4) {  // dbeta += <e^G dBw, k>;  out+ = beta e^G dBw
@@ -664,23 +682,39 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     }
     __syncthreads();
     for (int idx = tid; idx < 64 * 64; idx += 256) sR[(idx >> 6) * LNX_LDA + (idx & 63)] *= sBeta[idx >> 6];  // dX
+    for (int idx = tid; idx < 64 * DK; idx += 256) sOm[(idx / DK) * LDF + idx % DK] = 0.f;
     __syncthreads();
     pair_row<T, DK, true>(sOp, sR, sAl, LDF, sKr, LDK, 1.f, tid);
     pair_col<T, DK, true>(sOm, sR, sAl, LDF, sKr, LDK, 1.f, tid);
     __syncthreads();
     T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
-    for (int idx = tid; idx < 64 * DK; idx += 256) {
-      const int r = idx / DK, c = idx % DK;
-      const float up = sOp[r * LDF + c], um = sOm[r * LDF + c];
-      if (r < len) dkg[(int64_t)r * DK + c] = from_f32<T>(to_f32(dkg[(int64_t)r * DK + c]) + up + um);
-      dGg[idx] += to_f32(sKr[r * LDK + c]) * (up - um);
+    {
+      constexpr int IT = 64 * DK / 4 / 256;
+      floatx4 dk0[IT], dg0[IT];
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {  // all global reads first
+        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+        dg0[it] = load4(dGg + r * DK + c);
+      }
+#pragma unroll
+      for (int it = 0; it < IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
+        const floatx4 up = load4(sOp + r * LDF + c), um = load4(sOm + r * LDF + c), kk = load4(sKr + r * LDK + c);
+        if (r < len) store4(dkg + (int64_t)r * DK + c, dk0[it] + up + um);
+        store4(dGg + r * DK + c, dg0[it] + kk * (up - um));
+      }
     }
     __syncthreads();
     if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
     if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
+      float gv[64];
+#pragma unroll
+      for (int r = 0; r < 64; ++r) gv[r] = dGg[r * DK + tid];  // all loads in flight together
       float acc = 0.f;
+#pragma unroll
       for (int r = 63; r >= 0; --r) {
-        acc += dGg[r * DK + tid];
+        acc += gv[r];
         if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
       }
     }
@@ -700,7 +734,7 @@ template <typename T, int DK> struct Wy2Cfg {
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void bwd_wy2_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(BwdParams p) {
   typedef Wy2Cfg<T, DK> L;
   constexpr int LDC = L::LDC, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];

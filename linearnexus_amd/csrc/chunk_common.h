@@ -114,6 +114,8 @@ void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t
 // ---------------------------------------------------------------------------------------
 
 // out[i][c] += mul * sum_{j <= i (j < i if STRICT)} M[i][j] * E_ij[c] * b[j][c]
+// The token loop runs in blocks of 8 whose LDS reads are issued together (the loop is latency
+// bound otherwise); blocks are aligned so that masked tokens multiply by M = 0 / alpha = 1.
 template <typename T, int DK, bool STRICT>
 __device__ __forceinline__ void pair_row(float* out, const float* M, const float* al, int ldf, const T* b, int ldb,
                                          float mul, int tid) {
@@ -121,9 +123,27 @@ __device__ __forceinline__ void pair_row(float* out, const float* M, const float
   for (int i = wave; i < 64; i += 4)
     for (int c = lane; c < DK; c += 64) {
       float e = 1.f, acc = 0.f;
-      for (int j = i; j >= 0; --j) {
-        if (!(STRICT && j == i)) acc += M[i * LNX_LDA + j] * e * to_f32(b[j * ldb + c]);
-        e *= al[j * ldf + c];
+      for (int j0 = i | 7; j0 >= 7; j0 -= 8) {  // tokens j0, j0-1, ..., j0-7
+        float m[8], bv[8], av[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = j0 - u;  // always a valid row: loads are unconditional, masks applied after
+          m[u] = M[i * LNX_LDA + j];
+          bv[u] = to_f32(b[j * ldb + c]);
+          av[u] = al[j * ldf + c];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = j0 - u;
+          const bool on = j <= i;
+          m[u] = (on && !(STRICT && j == i)) ? m[u] : 0.f;
+          av[u] = on ? av[u] : 1.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          acc += m[u] * e * bv[u];
+          e *= av[u];
+        }
       }
       out[i * ldf + c] += mul * acc;
     }
@@ -137,9 +157,26 @@ __device__ __forceinline__ void pair_col(float* out, const float* M, const float
   for (int j = wave; j < 64; j += 4)
     for (int c = lane; c < DK; c += 64) {
       float e = 1.f, acc = 0.f;
-      for (int i = j; i < 64; ++i) {
-        if (i > j) e *= al[i * ldf + c];
-        if (!(STRICT && i == j)) acc += M[i * LNX_LDA + j] * e * to_f32(a[i * lda + c]);
+      for (int i0 = j & ~7; i0 < 64; i0 += 8) {  // tokens i0 .. i0+7
+        float m[8], xv[8], av[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u;
+          m[u] = M[i * LNX_LDA + j];
+          xv[u] = to_f32(a[i * lda + c]);
+          av[u] = al[i * ldf + c];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u;
+          m[u] = (i > j || (!STRICT && i == j)) ? m[u] : 0.f;
+          av[u] = (i > j) ? av[u] : 1.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          e *= av[u];
+          acc += m[u] * e * xv[u];
+        }
       }
       out[j * ldf + c] += mul * acc;
     }

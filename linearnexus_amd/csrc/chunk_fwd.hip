@@ -58,7 +58,7 @@ template <typename T, int DK> struct Prep2Cfg {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kTile = 64 * LDC;
-  static constexpr size_t f32_bytes = sizeof(float) * (2 * 64 * LNX_LDA + 32 * 36);
+  static constexpr size_t f32_bytes = sizeof(float) * (2 * 64 * LNX_LDA);  // A and Tm; the merge scratch overlays the Q slab
   static constexpr size_t regionF = (2 * kTile * sizeof(T) > f32_bytes) ? 2 * kTile * sizeof(T) : f32_bytes;
   static constexpr size_t bytes = regionF + 2 * kTile * sizeof(T) + sizeof(float) * 128;
 };
@@ -70,11 +70,11 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   extern __shared__ __align__(16) char smem[];
   float* sA = reinterpret_cast<float*>(smem);
   float* sT = sA + 64 * LNX_LDA;
-  float* sX = sT + 64 * LNX_LDA;
   T* sIn = reinterpret_cast<T*>(smem);  // overlays the fp32 matrices once Tw / Tu exist
   T* sOut = sIn + L::kTile;
   T* sKa = reinterpret_cast<T*>(smem + L::regionF);  // K slab, then Tw
-  T* sQa = sKa + L::kTile;                           // Q slab, then Tu
+  T* sQa = sKa + L::kTile;                           // Q slab, then the inverse's scratch, then Tu
+  float* sX = reinterpret_cast<float*>(sQa);
   float* sBeta = reinterpret_cast<float*>(sQa + L::kTile);
   float* sG = sBeta + 64;
 
