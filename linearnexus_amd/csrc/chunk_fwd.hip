@@ -336,7 +336,7 @@ template <typename T, int DK> struct ScanSmem {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
-  static constexpr int BV = 64;
+  static constexpr int BV = 64;  // dv slab per workgroup (32 was measured slower for the forward scan)
   static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 128;
 };
@@ -347,9 +347,11 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   typedef typename Vec16<T>::V V16;
   constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD;
   constexpr int VN = Vec16<T>::N;
-  // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and both column tiles,
+  // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and all column tiles,
   // DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
-  constexpr int NT = (DK == 128) ? 2 : 1;
+  constexpr int CT = BV / 32;
+  constexpr int NT = (DK == 128) ? CT : 1;
+  static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
   T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
@@ -380,7 +382,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   }
 
   // register prefetch of the next chunk's tiles
-  constexpr int NW = 64 * DK / VN / 256, NK = DK * 64 / VN / 256, NU = 64 * BV / VN / 256;
+  constexpr int NW = 64 * DK / VN / 256, NK = DK * 64 / VN / 256, NU = (64 * BV / VN + 255) / 256;
   V16 rW[NW], rK[NK], rU[NU];
   float rG = 0.f;
   auto fetch = [&](int n) {
@@ -403,7 +405,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-      rU[i] = *reinterpret_cast<const V16*>(Ug + (int64_t)r * p.dv + c);
+      if (idx < 64 * BV / VN) rU[i] = *reinterpret_cast<const V16*>(Ug + (int64_t)r * p.dv + c);
     }
     if (GATE == LNX_GATE_SCALAR && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
     if (GATE == LNX_GATE_VECTOR && tid < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];  // G_last[c]
@@ -422,7 +424,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-      *reinterpret_cast<V16*>(sU + r * LDU + c) = rU[i];
+      if (idx < 64 * BV / VN) *reinterpret_cast<V16*>(sU + r * LDU + c) = rU[i];
     }
     if (tid < 128) sG[tid] = rG;
   };
@@ -437,24 +439,26 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     __syncthreads();
     if (n + 1 < c1) fetch(n + 1);
 
-    // D = U - W S  (one 32x32 tile per wave)
-    const int wi = wave >> 1, wj = wave & 1;
-    floatx16 d[1][1];
-    frag_zero(d);
-    mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+    // D = U - W S  (one 32x32 tile per wave; with a 32-column slab only waves 0 and 1 have one)
+    const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
+    if (CT == 2 || wave < 2) {
+      floatx16 d[1][1];
+      frag_zero(d);
+      mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-      d[0][0][e] = to_f32(sU[r * LDU + c]) - d[0][0][e];
-    }
-    frag_store<T, 1, 1>(d, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj,
-                        p.dv, lane);
-    if (GATE == LNX_GATE_SCALAR) {
+      for (int e = 0; e < 16; ++e) {
+        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+        d[0][0][e] = to_f32(sU[r * LDU + c]) - d[0][0][e];
+      }
+      frag_store<T, 1, 1>(d, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj,
+                          p.dv, lane);
+      if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
+        for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
+      }
+      frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     __syncthreads();
 
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
@@ -606,7 +610,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("chunk_prepare", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
   lnx_profile_mark("chunk_scan", st);
-  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / 64)), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / ScanSmem<T, DK>::BV)), dim3(256), b2, st, p);
   lnx_profile_mark("chunk_output", st);
   hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
   lnx_profile_mark(nullptr, st);
