@@ -3,7 +3,7 @@
 //   chunk_prepare2 (one workgroup per 64-token chunk, all chunks in parallel; kda_prepare for a vector gate)
 //       A = tril(diag(beta) K K^T * E, -1);  Tm = (I + A)^-1 (fp32, block forward substitution +
 //       MFMA block merges);  W = Tm diag(beta e^G) K;  U = Tm diag(beta) V;
-//       P = scale * tril(Q K^T * E);  also K^T and Tm^T for later kernels.
+//       P = scale * tril(Q K^T * E);  also Tm^T for the backward pass.
 //   chunk_scan     (one workgroup per (state, 64-column slab of dv), sequential over chunks)
 //       D = U - W S;  S <- e^{G_last} S + (K e^{G_last - G})^T D, with the fp32 state held in
 //       MFMA accumulators across the whole sequence; stores D and the entering state.
@@ -49,8 +49,8 @@ __device__ __forceinline__ float wave_cumsum(float x, int lane) {
 }
 
 // ---------------------------------------------------------------------------------------
-// chunk_prepare2 (no gate / scalar gate): the same computation as chunk_prepare, organised as
-// slab loops with register prefetch so that two workgroups fit a CU: K K^T and Q K^T over
+// chunk_prepare2 (no gate / scalar gate), organised as slab loops with register prefetch so
+// that three workgroups fit a CU: K K^T and Q K^T over
 // 64-channel slabs, the fp32 inverse, then one 64-column slab of [dk | dv] at a time for
 // W and U, every result leaving through LDS with 16-byte stores.
 // ---------------------------------------------------------------------------------------
