@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
   rP.store(sP, LDC, tid);
   rdO.store(sdO, LDC, tid);
-  __syncthreads();
+  lds_barrier();
   const int wi = wave >> 1, wj = wave & 1;
   floatx16 acc[1][1];
   frag_zero(acc);
@@ -224,11 +224,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
   for (int n = c1 - 1; n >= c0; --n) {
     const int64_t slot = (int64_t)row * N + n;
     commit();
-    // dS (gradient of the state leaving chunk n) -> LDS transposed, and -> workspace row-major
+    // dS (gradient of the state leaving chunk n) -> LDS, transposed [dv][dk]; the workspace copy
+    // (same layout) leaves from there as whole rows, 16 bytes per lane
     frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
-    frag_store<T, 1, NT>(dS, wsp<T>(p, p.off.dSn) + slot * DK * p.dv + (int64_t)srow * p.dv + v0 + scol, p.dv, lane);
-    __syncthreads();
+    lds_barrier();
     if (n > c0) fetch(n - 1);
+    unstage_tile<T, BV, DK>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, tid);
 
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
     // dD = dD_loc + r_j (K dS)_j
@@ -241,13 +242,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
         const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
         const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[r], 0.f)) : 1.f;
         d[0][0][e] = to_f32(sdDl[r * LDU + c]) + rj * d[0][0][e];
+        sdDl[r * LDU + c] = from_f32<T>(d[0][0][e]);  // complete dD in place, written out from LDS below
+        d[0][0][e] = -d[0][0][e];
       }
-      frag_store<T, 1, 1>(d, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) d[0][0][e] = -d[0][0][e];
       frag_store_t<T, 1, 1>(d, sdDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    __syncthreads();
+    lds_barrier();
+    unstage_tile<T, 64, BV>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, tid);
 
     // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD   (token-contracted: rows of the tiles)
     if (GATE == LNX_GATE_SCALAR) {
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
     }
     mma_x<T, 1, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
     mma_x<T, 1, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
-    __syncthreads();
+    lds_barrier();
   }
   if (p.ds0) {
     float* out = p.ds0 + (int64_t)sidx * DK * p.dv + v0;
@@ -335,14 +336,14 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   // dv is consumed in slabs of SV columns; narrow slabs keep the prefetch registers few enough
   // for three waves per SIMD
   constexpr int SV = 32, LDS_ = SV + Mma<T>::PAD;
-  TileRegs<T, 64, SV> rdO, rD, rdD, rdSn;
-  TileRegs<T, SV, 64> rSn;  // S_n slab stays [v][c]: contracted along its rows
+  TileRegs<T, 64, SV> rdO, rD, rdD;
+  TileRegs<T, SV, 64> rSn, rdSn;  // S_n and dS_n slabs stay [v][c]: contracted along their rows
   auto fetch = [&](int v0) {
     rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
     rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
-    rdSn.load(wsp<T>(p, p.off.dSn) + slot * DK * p.dv + (int64_t)ch0 * p.dv + v0, p.dv, 64, tid);
+    rdSn.load(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
   };
   floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
   frag_zero(aP);
@@ -352,28 +353,24 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   float ss = 0.f;
   fetch(0);
   for (int v0 = 0; v0 < p.dv; v0 += SV) {
-    __syncthreads();
+    lds_barrier();
     rdO.store(sdO, LDS_, tid);
     rD.store(sD, LDS_, tid);
     rdD.store(sdD, LDS_, tid);
     rSn.store(sSn, LDC, tid);
-    rdSn.store(sdSn, LDS_, tid);
-    __syncthreads();
+    rdSn.store(sdSn, LDC, tid);
+    lds_barrier();
     if (v0 + SV < p.dv) fetch(v0 + SV);
     mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDS_, LDS_, sD + 32 * wj * LDS_, LDS_, SV, lane);
     mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
     mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
-    mma_nt<T, 1, 1>(aK, sD + 32 * wi * LDS_, LDS_, sdSn + 32 * wj * LDS_, LDS_, SV, lane);
+    mma_x<T, 1, 1, false, true>(aK, sD + 32 * wi * LDS_, LDS_, sdSn + 32 * wj, LDC, SV, lane);
     if (GATE != LNX_GATE_NONE) {  // thread = (channel row tid / 4, quarter of the slab)
       constexpr int QV = SV / 4;
       const int r = tid >> 2, q4 = (tid & 3) * QV;
       float t = 0.f;
 #pragma unroll
-      for (int e = 0; e < QV; e += 4) {
-        const floatx4 y = load4(sdSn + r * LDS_ + q4 + e);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) t += to_f32(sSn[(q4 + e + u) * LDC + r]) * y[u];
-      }
+      for (int e = 0; e < QV; ++e) t += to_f32(sSn[(q4 + e) * LDC + r]) * to_f32(sdSn[(q4 + e) * LDC + r]);
       ss += t;
     }
   }
@@ -385,7 +382,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     ss = wave_sum(ss);
     if (lane == 0) atomicAdd(&sMisc[1], ss);
   }
-  __syncthreads();  // slab tiles are dead from here on
+  lds_barrier();  // slab tiles are dead from here on
 
   if constexpr (GATE == LNX_GATE_VECTOR) {
     // ---- per-channel gate: element-wise decays, pair terms on the VALU (64 channels) ----
@@ -412,7 +409,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
       sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
     }
-    __syncthreads();
+    lds_barrier();
     {
       T* dWg = wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0;
       for (int idx = tid; idx < 64 * 16; idx += 256) {
@@ -420,16 +417,16 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
         store4(dWg + (int64_t)r * DK + c, load4(sOut + r * LDF + c));
       }
     }
-    __syncthreads();
+    lds_barrier();
     // dq = scale e^G dQg + intra-chunk part
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
       sOut[r * LDF + c] = aQ[0][0][e] * p.scale * __expf(Gg[r * DK + c]);
     }
-    __syncthreads();
+    lds_barrier();
     pair_row<T, 64, false>(sOut, sR, sAl, LDF, sKr, LDC, p.scale, tid);
-    __syncthreads();
+    lds_barrier();
     T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK + ch0;
     for (int idx = tid; idx < 64 * 16; idx += 256) {
       const int r = idx >> 4, c = (idx & 15) * 4;
@@ -437,22 +434,22 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       if (r < len) store4(dqg + (int64_t)r * DK + c, v);
       store4(dGg + r * DK + c, qq * v);
     }
-    __syncthreads();
+    lds_barrier();
     // dk (column-type parts): e^{G_last - G} dKr + P part; chunk-end gate term from the Kr part
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
       sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(Gg[63 * DK + c] - Gg[r * DK + c], 0.f));
     }
-    __syncthreads();
+    lds_barrier();
     float dgc = 0.f;
     if (tid < 64) {
       for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDC + tid]);
       dgc += __expf(Gg[63 * DK + tid]) * sSS[tid];
     }
-    __syncthreads();
+    lds_barrier();
     pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
-    __syncthreads();
+    lds_barrier();
     T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + ch0;
     for (int idx = tid; idx < 64 * 16; idx += 256) {
       const int r = idx >> 4, c = (idx & 15) * 4;
@@ -460,7 +457,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       if (r < len) store4(dkg + (int64_t)r * DK + c, v);
       store4(dGg + r * DK + c, load4(dGg + r * DK + c) - kk * v);
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < 64) dGg[63 * DK + tid] += dgc;
   } else {
     // ---- scalar / no gate ----
@@ -486,7 +483,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     }
     rKT.store(sKr, LDC, tid);
     rQT.store(sQr, LDC, tid);
-    __syncthreads();
+    lds_barrier();
     unstage_tile<T, 64, 64>(wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0, DK, sOut, LDC, 64, tid);
     // inter-chunk parts scaled, then the intra-chunk products on top
     const float gl = sG[63];
@@ -515,10 +512,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       tot = wave_sum(tot);
       if (lane == 0) atomicAdd(&sMisc[0], tot);
     }
-    __syncthreads();  // all reads of sPe / sOut done
+    lds_barrier();  // all reads of sPe / sOut done
     frag_store<T, 1, 1>(aQ, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
     frag_store<T, 1, 1>(aK, sOut2 + 32 * wi * LDC + 32 * wj, LDC, lane);
-    __syncthreads();
+    lds_barrier();
     unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, DK, sPe, LDC, len, tid);
     unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sOut2, LDC, len, tid);
     if (GATE != LNX_GATE_NONE && tid < 64) {
@@ -583,7 +580,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   T* sdWT = R2;
   stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
   stage_tile_t<T, 64, DK>(sdWT, LDC, wsp<T>(p, p.off.dW) + slot * 64 * DK, DK, 64, tid);
-  __syncthreads();
+  lds_barrier();
   floatx16 aBw[MT][1], aM[1][1];
   frag_zero(aBw);
   frag_zero(aM);
@@ -594,10 +591,10 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   T* sdBu = R2 + 64 * LDC;
   T* sU = R3;
   for (int v0 = 0; v0 < p.dv; v0 += 64) {
-    __syncthreads();
+    lds_barrier();
     stage_tile_t<T, 64, 64>(sdDT, LDC, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     stage_tile<T, 64, 64>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    __syncthreads();
+    lds_barrier();
     floatx16 bu[1][1];
     frag_zero(bu);
     mma_nt<T, 1, 1>(bu, sTmT + 32 * wi * LDC, LDC, sdDT + 32 * wj * LDC, LDC, 64, lane);
@@ -609,19 +606,19 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     for (int e = 0; e < 16; ++e) bu[0][0][e] *= sBeta[32 * wi + frag_row(e, lane)];
     frag_store<T, 1, 1>(bu, reinterpret_cast<T*>(p.dv_out) + (tbase + 32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane,
                         len - 32 * wi);
-    __syncthreads();
+    lds_barrier();
     mma_nt<T, 1, 1>(aM, sdBu + 32 * wi * LDC, LDC, sU + 32 * wj * LDC, LDC, 64, lane);
   }
-  __syncthreads();
+  lds_barrier();
 
   // phase 3: dM += dBw W^T
   T* sdBw = R2;
   T* sW = R3;
   frag_store<T, MT, 1>(aBw, sdBw + r0 * LDK + c0, LDK, lane);
   stage_tile<T, 64, DK>(sW, LDK, wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
-  __syncthreads();
+  lds_barrier();
   mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
-  __syncthreads();
+  lds_barrier();
 
   static_assert(GATE == LNX_GATE_VECTOR, "bwd_wy2 handles the other gate kinds");
   {
@@ -665,7 +662,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
         const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
         sOp[r * LDF + c] = aBw[i][0][e] * __expf(Gg[r * DK + c]);  // e^G dBw
       }
-    __syncthreads();
+    lds_barrier();
     if (tid < 64) {  // dbeta += sum_j dA_ij X_ij
       float rs = 0.f;
       for (int j = 0; j < tid; ++j) rs += sR[tid * LNX_LDA + j] * to_f32(sXp[tid * LDC + j]);
@@ -680,13 +677,13 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
       t = wave_sum(t);
       if (lane == 0) atomicAdd(&sdB[r], t);
     }
-    __syncthreads();
+    lds_barrier();
     for (int idx = tid; idx < 64 * 64; idx += 256) sR[(idx >> 6) * LNX_LDA + (idx & 63)] *= sBeta[idx >> 6];  // dX
     for (int idx = tid; idx < 64 * DK; idx += 256) sOm[(idx / DK) * LDF + idx % DK] = 0.f;
-    __syncthreads();
+    lds_barrier();
     pair_row<T, DK, true>(sOp, sR, sAl, LDF, sKr, LDK, 1.f, tid);
     pair_col<T, DK, true>(sOm, sR, sAl, LDF, sKr, LDK, 1.f, tid);
-    __syncthreads();
+    lds_barrier();
     T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
     {
       constexpr int IT = 64 * DK / 4 / 256;
@@ -705,7 +702,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
         store4(dGg + r * DK + c, dg0[it] + kk * (up - um));
       }
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
     if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
       float gv[64];
@@ -797,11 +794,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
 #pragma unroll 1
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ < NKS;
-    __syncthreads();
+    lds_barrier();
     rIn.store(sIn, LDC, tid);
     rWU.store(sWU, LDC, tid);
     rKs.store(sKs, LDC, tid);
-    __syncthreads();
+    lds_barrier();
     if (s_ + 1 < nslab) fetch(s_ + 1);
     floatx16 b[1][1];
     frag_zero(b);
@@ -825,7 +822,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
         }
       if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
     }
-    __syncthreads();
+    lds_barrier();
     mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
     if (!is_k) {  // dv = beta dBu, 16-byte stores
       constexpr int VN = Vec16<T>::N;
@@ -848,7 +845,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
     rKT[u].load(kg + 64 * u, DK, len, tid);  // K rows again, for Y K
     rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, DK, len, tid);
   }
-  __syncthreads();  // loop tiles dead
+  lds_barrier();  // loop tiles dead
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
     floatx16 y[1][1];
@@ -872,7 +869,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
     T* sKT = (u == 0) ? sKs : sTmT;
     rKT[u].store(sKT, LDC, tid);
   }
-  __syncthreads();
+  lds_barrier();
 #pragma unroll
   for (int u = 0; u < NKS; ++u) {
     const T* sKT = (u == 0) ? sKs : sTmT;
@@ -884,9 +881,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
     }
     mma_x<T, 1, 1, false, true>(aBw[u], sYa + 32 * wi * LDC, LDC, sKT + 32 * wj, LDC, 64, lane);
     mma_x<T, 1, 1, true, true>(aBw[u], sYa + 32 * wi, LDC, sKT + 32 * wj, LDC, 64, lane);
-    if (u > 0) __syncthreads();
+    if (u > 0) lds_barrier();
     frag_store<T, 1, 1>(aBw[u], sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
-    __syncthreads();
+    lds_barrier();
     {
       constexpr int VN = Vec16<T>::N, VPR = 64 / VN;
       T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + 64 * u;

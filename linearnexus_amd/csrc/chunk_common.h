@@ -18,7 +18,7 @@
 //   SnT  [dv][dk]   transpose of the state entering the chunk
 //   vector gate only:  X [64][64] = <k_i, k_j>_E (i > j),  Kr [64][dk] = K * exp(G_last - G),
 //                      Qg [64][dk] = scale * Q * exp(G)
-// Backward adds dD [64][dv], dSn [dk][dv] (gradient of the state leaving the chunk), dW [64][dk]
+// Backward adds dD [64][dv], dSn [dv][dk] (gradient of the state leaving the chunk, transposed), dW [64][dk]
 // and dG (fp32 partial gradient of the cumulative gate).
 #pragma once
 

@@ -108,10 +108,10 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   frag_zero(ap);
 #pragma unroll 1
   for (int s_ = 0; s_ < NKS; ++s_) {
-    __syncthreads();
+    lds_barrier();
     rK.store(sKa, LDC, tid);
     rQ.store(sQa, LDC, tid);
-    __syncthreads();
+    lds_barrier();
     if (s_ + 1 < NKS) {
       rK.load(kg + 64 * (s_ + 1), DK, len, tid);
       rQ.load(qg + 64 * (s_ + 1), DK, len, tid);
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     else rIn.load(vg + 64 * (s_ - NKS), p.dv, len, tid);
   };
   fetch(0);
-  __syncthreads();  // slab tiles dead
+  lds_barrier();  // slab tiles dead
   {
     floatx16 pe[1][1];
 #pragma unroll
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     }
     frag_store<T, 1, 1>(pe, sKa + 32 * wi * LDC + 32 * wj, LDC, lane);
   }
-  __syncthreads();
+  lds_barrier();
   unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sKa, LDC, 64, tid);
   tri_inverse_64(sA, sT, sX, tid);
   {
@@ -161,16 +161,16 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
 #pragma unroll 1
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ < NKS;
-    __syncthreads();  // fp32 matrices / previous slab's tiles are dead
+    lds_barrier();  // fp32 matrices / previous slab's tiles are dead
     rIn.store(sIn, LDC, tid);
-    __syncthreads();
+    lds_barrier();
     if (s_ + 1 < nslab) fetch(s_ + 1);
     floatx16 acc[1][1];
     frag_zero(acc);
     // W = Tw K, U = Tu V: the slab is [token][column], contracted along its rows
     mma_x<T, 1, 1, false, true>(acc, (is_k ? sKa : sQa) + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
     frag_store<T, 1, 1>(acc, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
-    __syncthreads();
+    lds_barrier();
     if (is_k)
       unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + 64 * s_, DK, sOut, LDC, 64, tid);
     else
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
     store4(sG + r * LDF + c, x);
   }
   if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
-  __syncthreads();
+  lds_barrier();
   if (tid < DK) {
     float acc = 0.f;
     for (int r = 0; r < 64; ++r) {
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
       sG[r * LDF + tid] = acc;
     }
   }
-  __syncthreads();
+  lds_barrier();
   {
     float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
     T* Krg = ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK;
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
       Pg[idx] = from_f32<T>(p.scale * pp);
     }
   }
-  __syncthreads();
+  lds_barrier();
   tri_inverse_64(sA, sT, sX, tid);
 
   T* sTm = sK;                         // T-typed copy of Tm (bf16); fp32 reads sT in place
@@ -297,11 +297,11 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
     }
   }
   const T* tm_op = (sizeof(T) == 4) ? reinterpret_cast<const T*>(sT) : sTm;
-  __syncthreads();
+  lds_barrier();
   // W = Tm (beta e^G K): transposed, scaled K through the sQ region
   T* sKT = sQ;
   stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid, [&](int r, int c) { return sBeta[r] * __expf(sG[r * LDF + c]); });
-  __syncthreads();
+  lds_barrier();
   const int wi = wave >> 1, wj = wave & 1;
   {
     T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
@@ -312,15 +312,15 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
       frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
     }
   }
-  __syncthreads();
+  lds_barrier();
   // U = Tu V
   {
     T* sVT = sQ;
     T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
     for (int c0 = 0; c0 < p.dv; c0 += 64) {
-      __syncthreads();
+      lds_barrier();
       stage_tile_t<T, 64, 64>(sVT, LDC, vg + c0, p.dv, len, tid);
-      __syncthreads();
+      lds_barrier();
       floatx16 acc[1][1];
       frag_zero(acc);
       mma_nt<T, 1, 1>(acc, sTu + 32 * wi * LDC, LDC, sVT + 32 * wj * LDC, LDC, 64, lane);
@@ -433,11 +433,12 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   for (int n = c0; n < c1; ++n) {
     const int64_t slot = (int64_t)row * N + n;
     commit();
-    // entering state -> LDS (B operand of W S) and -> workspace, both transposed [dv][dk]
+    // entering state -> LDS, transposed [dv][dk] (B operand of W S); the workspace copy leaves
+    // from there as whole rows, 16 bytes per lane
     frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
-    frag_store_t<T, 1, NT>(S, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)(v0 + scol) * DK + srow, DK, lane);
-    __syncthreads();
+    lds_barrier();
     if (n + 1 < c1) fetch(n + 1);
+    unstage_tile<T, BV, DK>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
 
     // D = U - W S  (one 32x32 tile per wave; with a 32-column slab only waves 0 and 1 have one)
     const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
@@ -450,16 +451,16 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       for (int e = 0; e < 16; ++e) {
         const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
         d[0][0][e] = to_f32(sU[r * LDU + c]) - d[0][0][e];
+        sU[r * LDU + c] = from_f32<T>(d[0][0][e]);  // D replaces U in place and is written out from LDS below
       }
-      frag_store<T, 1, 1>(d, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + (int64_t)(32 * wi) * p.dv + v0 + 32 * wj,
-                          p.dv, lane);
       if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
       }
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    __syncthreads();
+    lds_barrier();
+    unstage_tile<T, 64, BV>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, tid);
 
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
     if (GATE == LNX_GATE_SCALAR) {
@@ -476,7 +477,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
         for (int e = 0; e < 16; ++e) S[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
     mma_x<T, 1, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
-    __syncthreads();
+    lds_barrier();
   }
 
   float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0;
@@ -542,7 +543,7 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   stage_tile<T, 64, 64>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
   stage_tile<T, 64, BV>(sDT, LDC, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);  // D rows [token][v]
   if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-  __syncthreads();
+  lds_barrier();
 
   const int wi = wave >> 1, wj = wave & 1;
   floatx16 acc[1][1];

@@ -46,6 +46,17 @@ __device__ __forceinline__ void store4(bf16_t* p, floatx4 x) {
   *reinterpret_cast<bf16x4*>(p) = t;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits until every global
+// load and store of the wave has completed, which puts the full memory latency of a register
+// prefetch (and of streamed-out results) on the critical path of each loop iteration.  Use this
+// one wherever the data exchanged between the waves lives in LDS; global memory written by one
+// wave and read back by another in the same kernel still needs __syncthreads().
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Sum over all 64 lanes; every lane gets the total.
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll

@@ -350,7 +350,7 @@ __device__ __forceinline__ void mm16_store(float* dst, int ld, floatx4 c, int la
 __device__ __forceinline__ void tri_inverse_64(const float* sA, float* sT, float* sX, int tid) {
   const int wave = tid >> 6, lane = tid & 63;
   for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) sT[idx] = 0.f;
-  __syncthreads();
+  lds_barrier();
   if (lane < 16) {
     const int r0 = 16 * wave, c = lane;
     float d[16];
@@ -364,7 +364,7 @@ __device__ __forceinline__ void tri_inverse_64(const float* sA, float* sT, float
 #pragma unroll
     for (int i = 0; i < 16; ++i) sT[(r0 + i) * LNX_LDA + r0 + c] = d[i];
   }
-  __syncthreads();
+  lds_barrier();
   // level 1: blocks (1,0) and (3,2) of the 16x16 grid, one per wave 0/1
   float* sXw = sX + (wave & 1) * 16 * 36;
   const int b = 32 * (wave & 1);  // super-block origin
@@ -372,22 +372,22 @@ __device__ __forceinline__ void tri_inverse_64(const float* sA, float* sT, float
     floatx4 x = mm16_f32(sA + (b + 16) * LNX_LDA + b, LNX_LDA, sT + b * LNX_LDA + b, LNX_LDA, 16, lane);
     mm16_store(sXw, 36, x, lane, 1.f);
   }
-  __syncthreads();
+  lds_barrier();
   if (wave < 2) {
     floatx4 y = mm16_f32(sT + (b + 16) * LNX_LDA + b + 16, LNX_LDA, sXw, 36, 16, lane);
     mm16_store(sT + (b + 16) * LNX_LDA + b, LNX_LDA, y, lane, -1.f);
   }
-  __syncthreads();
+  lds_barrier();
   // level 2: the 32x32 lower-left block, one 16x16 output per wave
   const int bi = 16 * (wave >> 1), bj = 16 * (wave & 1);
   {
     floatx4 x = mm16_f32(sA + (32 + bi) * LNX_LDA, LNX_LDA, sT + bj, LNX_LDA, 32, lane);
     mm16_store(sX + bi * 36 + bj, 36, x, lane, 1.f);
   }
-  __syncthreads();
+  lds_barrier();
   {
     floatx4 y = mm16_f32(sT + (32 + bi) * LNX_LDA + 32, LNX_LDA, sX + bj, 36, 32, lane);
     mm16_store(sT + (32 + bi) * LNX_LDA + bj, LNX_LDA, y, lane, -1.f);
   }
-  __syncthreads();
+  lds_barrier();
 }
