@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
     frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
     lds_barrier();
     if (n > c0) fetch(n - 1);
-    unstage_tile<T, BV, DK>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, tid);
+    unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, tid);
 
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
     // dD = dD_loc + r_j (K dS)_j
@@ -237,18 +237,25 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
       floatx16 d[1][1];
       frag_zero(d);
       mma_nt<T, 1, 1>(d, sK + 32 * wi * LDK, LDK, sdST + 32 * wj * LDK, LDK, DK, lane);
+      // the complete dD replaces the local part in place (all reads first: interleaved with the
+      // writes they would be serialised) and is written out from LDS below
+      float dl[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dl[e] = to_f32(sdDl[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[r], 0.f)) : 1.f;
-        d[0][0][e] = to_f32(sdDl[r * LDU + c]) + rj * d[0][0][e];
-        sdDl[r * LDU + c] = from_f32<T>(d[0][0][e]);  // complete dD in place, written out from LDS below
+        const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f)) : 1.f;
+        d[0][0][e] = dl[e] + rj * d[0][0][e];
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        sdDl[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)] = from_f32<T>(d[0][0][e]);
         d[0][0][e] = -d[0][0][e];
       }
       frag_store_t<T, 1, 1>(d, sdDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
     lds_barrier();
-    unstage_tile<T, 64, BV>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, tid);
+    unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, tid);
 
     // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD   (token-contracted: rows of the tiles)
     if (GATE == LNX_GATE_SCALAR) {

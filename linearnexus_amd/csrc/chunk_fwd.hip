@@ -330,35 +330,44 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
-// chunk_scan
+// chunk_scan: the sequential pass over the chunks of one (state, 64-column slab of dv).
+// Per chunk: D = U - W S, the state update, and -- for 2-byte inputs, where the tiles fit LDS --
+// the outputs o = scale e^G (Q S) + P D of the same slab, so the state and D are not read back
+// by a separate output kernel.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct ScanSmem {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int BV = 64;  // dv slab per workgroup (32 was measured slower for the forward scan)
+  static constexpr bool FUSE_OUT = sizeof(T) == 2;
+  static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
   static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
-  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT) + sizeof(float) * 128;
+  static constexpr int kQ = FUSE_OUT ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
+  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
+                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   typedef ScanSmem<T, DK> L;
-  typedef typename Vec16<T>::V V16;
-  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD;
-  constexpr int VN = Vec16<T>::N;
+  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD, LDO = L::LDO;
+  constexpr bool FUSE = L::FUSE_OUT;
   // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and all column tiles,
   // DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
   constexpr int CT = BV / 32;
   constexpr int NT = (DK == 128) ? CT : 1;
-  static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
+  static_assert(BV == 64, "one 32x32 tile of the [64 x BV] products per wave");
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
   T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
-  T* sU = sK + L::kKT;
+  T* sU = sK + L::kKT; // U rows [token][v], replaced by D
   T* sST = sU + L::kU;
   T* sDT = sST + L::kST;
-  float* sG = reinterpret_cast<float*>(sDT + L::kDT);
+  T* sQ = sDT + L::kDT;  // fused output only: Q rows (vector gate: scale Q e^G), P, output staging
+  T* sP = sQ + L::kQ;
+  bf16_t* sO = reinterpret_cast<bf16_t*>(sP + L::kP);
+  float* sG = reinterpret_cast<float*>(sO + (FUSE ? 64 * LDO : 0));
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
@@ -369,6 +378,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
   const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
   const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
+  const int wi = wave >> 1, wj = wave & 1;  // this wave's tile of the [64 x BV] products
 
   floatx16 S[1][NT];
   frag_zero(S);
@@ -382,77 +392,64 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   }
 
   // register prefetch of the next chunk's tiles
-  constexpr int NW = 64 * DK / VN / 256, NK = DK * 64 / VN / 256, NU = (64 * BV / VN + 255) / 256;
-  V16 rW[NW], rK[NK], rU[NU];
+  TileRegs<T, 64, DK> rW, rK;
+  TileRegs<T, 64, BV> rU;
+  TileRegs<T, 64, FUSE ? DK : 8> rQ;
+  TileRegs<T, 64, FUSE ? 64 : 8> rP;
   float rG = 0.f;
+  int rTok0 = 0, rLen = 0;
   auto fetch = [&](int n) {
     const int64_t slot = (int64_t)row * N + n;
-    const T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
-    int tok0, len;
-    chunk_span(p.geom, n, tok0, len);
-    const T* Kg = (GATE == LNX_GATE_VECTOR) ? ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK
-                                            : reinterpret_cast<const T*>(p.k) + ((int64_t)row * p.geom.T + tok0) * DK;
-    if (GATE == LNX_GATE_VECTOR) len = 64;
-    const T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0;
-#pragma unroll
-    for (int i = 0; i < NW; ++i) rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)(tid + 256 * i) * VN);
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int idx = tid + 256 * i;
-      rK[i] = vec_zero<T>();
-      if (idx / (DK / VN) < len) rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
-    }
-#pragma unroll
-    for (int i = 0; i < NU; ++i) {
-      const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-      if (idx < 64 * BV / VN) rU[i] = *reinterpret_cast<const V16*>(Ug + (int64_t)r * p.dv + c);
+    chunk_span(p.geom, n, rTok0, rLen);
+    const int64_t tbase = (int64_t)row * p.geom.T + rTok0;
+    rW.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
+    if (GATE == LNX_GATE_VECTOR) rK.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, tid);
+    else rK.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, rLen, tid);
+    rU.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+    if (FUSE) {
+      if (GATE == LNX_GATE_VECTOR) rQ.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, tid);
+      else rQ.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, rLen, tid);
+      rP.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
     }
     if (GATE == LNX_GATE_SCALAR && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
     if (GATE == LNX_GATE_VECTOR && tid < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];  // G_last[c]
-  };
-  auto commit = [&]() {
-#pragma unroll
-    for (int i = 0; i < NW; ++i) {
-      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
-      *reinterpret_cast<V16*>(sW + r * LDK + c) = rW[i];
-    }
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
-      *reinterpret_cast<V16*>(sK + r * LDK + c) = rK[i];
-    }
-#pragma unroll
-    for (int i = 0; i < NU; ++i) {
-      const int idx = tid + 256 * i, r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-      if (idx < 64 * BV / VN) *reinterpret_cast<V16*>(sU + r * LDU + c) = rU[i];
-    }
-    if (tid < 128) sG[tid] = rG;
   };
 
   if (c0 < c1) fetch(c0);
   for (int n = c0; n < c1; ++n) {
     const int64_t slot = (int64_t)row * N + n;
-    commit();
-    // entering state -> LDS, transposed [dv][dk] (B operand of W S); the workspace copy leaves
-    // from there as whole rows, 16 bytes per lane
+    const int tok0 = rTok0, len = rLen;
+    rW.store(sW, LDK, tid);
+    rK.store(sK, LDK, tid);
+    rU.store(sU, LDU, tid);
+    if (FUSE) {
+      rQ.store(sQ, LDK, tid);
+      rP.store(sP, LDC, tid);
+    }
+    if (tid < 128) sG[tid] = rG;
+    // entering state -> LDS, transposed [dv][dk] (B operand of W S and Q S); the workspace copy
+    // leaves from there as whole rows, 16 bytes per lane
     frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
     lds_barrier();
     if (n + 1 < c1) fetch(n + 1);
-    unstage_tile<T, BV, DK>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
+    unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
 
-    // D = U - W S  (one 32x32 tile per wave; with a 32-column slab only waves 0 and 1 have one)
-    const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
+    // D = U - W S  (one 32x32 tile per wave)
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
-    if (CT == 2 || wave < 2) {
+    {
       floatx16 d[1][1];
       frag_zero(d);
       mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+      // D replaces U in place (all reads first: interleaved with the writes they would be serialised)
+      // and is written out from LDS below
+      float u[16];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        d[0][0][e] = to_f32(sU[r * LDU + c]) - d[0][0][e];
-        sU[r * LDU + c] = from_f32<T>(d[0][0][e]);  // D replaces U in place and is written out from LDS below
-      }
+      for (int e = 0; e < 16; ++e) u[e] = to_f32(sU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) d[0][0][e] = u[e] - d[0][0][e];
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        sU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)] = from_f32<T>(d[0][0][e]);
       if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
@@ -460,7 +457,25 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
     lds_barrier();
-    unstage_tile<T, 64, BV>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, tid);
+    unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, tid);
+
+    if (FUSE) {
+      // o = scale e^G (Q S) + P D for this slab, staged in LDS in the output type
+      floatx16 o[1][1];
+      frag_zero(o);
+      mma_nt<T, 1, 1>(o, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+      if (GATE != LNX_GATE_VECTOR) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+      }
+      mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
+      if (p.o_dtype == LNX_BF16)
+        frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);
+      else
+        frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + ((int64_t)row * p.geom.T + tok0 + 32 * wi) * p.dv + v0 + 32 * wj,
+                                p.dv, lane, len - 32 * wi);
+    }
 
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
     if (GATE == LNX_GATE_SCALAR) {
@@ -478,6 +493,8 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
     }
     mma_x<T, 1, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
     lds_barrier();
+    if (FUSE && p.o_dtype == LNX_BF16)
+      unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + ((int64_t)row * p.geom.T + tok0) * p.dv + v0, p.dv, sO, LDO, len, tid);
   }
 
   float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0;
@@ -612,8 +629,10 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
   lnx_profile_mark("chunk_scan", st);
   hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / ScanSmem<T, DK>::BV)), dim3(256), b2, st, p);
-  lnx_profile_mark("chunk_output", st);
-  hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
+  if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
+    lnx_profile_mark("chunk_output", st);
+    hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
+  }
   lnx_profile_mark(nullptr, st);
   return LNX_OK;
 }

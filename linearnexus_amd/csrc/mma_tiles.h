@@ -273,15 +273,31 @@ __device__ __forceinline__ void stage_tile_t(T* dst, int ld, const T* src, int64
 }
 
 // LDS tile [ROWS][COLS] (leading dimension ld) -> global, 16-byte vectors, rows < valid only.
-template <typename T, int ROWS, int COLS>
+// FULL: every row is written and the tile is a whole number of 256-thread passes, so the loads
+// and stores are unconditional and issued as two batches.
+template <typename T, int ROWS, int COLS, bool FULL = false>
 __device__ __forceinline__ void unstage_tile(T* dst, int64_t stride, const T* src, int ld, int valid, int tid) {
+  typedef typename Vec16<T>::V V;
   constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = (TOTAL + 255) / 256;
+  if constexpr (FULL) {
+    static_assert(TOTAL % 256 == 0, "whole passes only");
+    V x[IT];
 #pragma unroll
-  for (int it = 0; it < IT; ++it) {
-    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
-    if (idx < TOTAL && r < valid)
-      *reinterpret_cast<typename Vec16<T>::V*>(dst + r * stride + c) =
-          *reinterpret_cast<const typename Vec16<T>::V*>(src + r * ld + c);
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+      x[it] = *reinterpret_cast<const V*>(src + r * ld + c);
+    }
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+      *reinterpret_cast<V*>(dst + r * stride + c) = x[it];
+    }
+  } else {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+      if (idx < TOTAL && r < valid) *reinterpret_cast<V*>(dst + r * stride + c) = *reinterpret_cast<const V*>(src + r * ld + c);
+    }
   }
 }
 
