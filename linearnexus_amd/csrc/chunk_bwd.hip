@@ -393,7 +393,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
 
   if constexpr (GATE == LNX_GATE_VECTOR) {
     // ---- per-channel gate: element-wise decays, pair terms on the VALU (64 channels) ----
-    float* sAl = reinterpret_cast<float*>(sdO);      // [64][LDF] alpha_j[c] = exp(g_j[c])
+    float* sAl = reinterpret_cast<float*>(sdO);      // [64][LDF] cumulative gate G_j[c] of this half's channels
     float* sOut = sAl + 64 * LDF;                    // [64][LDF]
     T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC] (this half's channels)
     T* sQr = sKr + L::kTile;
@@ -411,10 +411,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     }
     rk.store(sKr, LDC, tid);
     rq.store(sQr, LDC, tid);
-    for (int idx = tid; idx < 64 * 64; idx += 256) {
-      const int r = idx >> 6, c = idx & 63;
-      const float prev = (r > 0) ? Gg[(r - 1) * DK + c] : 0.f;
-      sAl[r * LDF + c] = __expf(fminf(Gg[r * DK + c] - prev, 0.f));
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int r = idx >> 4, c = (idx & 15) * 4;
+      store4(sAl + r * LDF + c, load4(Gg + r * DK + c));
     }
     lds_barrier();
     {
@@ -630,7 +629,7 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
   static_assert(GATE == LNX_GATE_VECTOR, "bwd_wy2 handles the other gate kinds");
   {
     // ---- per-channel gate ----
-    float* sAl = reinterpret_cast<float*>(R1);  // [64][LDF]
+    float* sAl = reinterpret_cast<float*>(R1);  // [64][LDF] cumulative gate
     float* sOp = sAl + 64 * LDF;                // row-type part of dk (through B_w and the rows of X)
     float* sOm = sOp + 64 * LDF;                // column-type part of dk (columns of X)
     T* sKr = reinterpret_cast<T*>(sOm + 64 * LDF);
@@ -646,20 +645,16 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
     stage_tile<T, 64, DK>(sKr, LDK, kg, DK, len, tid);
     {
       constexpr int IT = 64 * DK / 4 / 256;
-      floatx4 g1[IT], g0[IT];
+      floatx4 g1[IT];
 #pragma unroll
       for (int it = 0; it < IT; ++it) {
         const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
         g1[it] = load4(Gg + r * DK + c);
-        g0[it] = (r > 0) ? load4(Gg + (r - 1) * DK + c) : floatx4{0.f, 0.f, 0.f, 0.f};
       }
 #pragma unroll
       for (int it = 0; it < IT; ++it) {
         const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-        floatx4 a4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) a4[e] = __expf(fminf(g1[it][e] - g0[it][e], 0.f));
-        store4(sAl + r * LDF + c, a4);
+        store4(sAl + r * LDF + c, g1[it]);
       }
     }
 #pragma unroll

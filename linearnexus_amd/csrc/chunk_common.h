@@ -106,78 +106,146 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward);
 void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st);
 
 // ---------------------------------------------------------------------------------------
-// Vector-gate (KDA) helpers: per-channel decays E_ij[c] = prod_{m=j+1..i} alpha_m[c] are applied
-// with a multiplicative recurrence along the token index, so no exponent of a positive number
-// is ever taken (the property kda.py:426-434 protects with its blocked factorisation).
-// Tiles live in LDS: M [64][LNX_LDA] fp32, al (alpha) and out [64][ldf] fp32, operands [64][ldb].
-// A wavefront owns a token row (or column), its lanes the channels.
+// Vector-gate (KDA) helpers.  The per-channel decays E_ij[c] = exp(G_i[c] - G_j[c]) (i >= j, G the
+// cumulative gate inside the chunk, non-increasing along i) sit inside the token sums.  Wherever a
+// reference token r with j <= r <= i exists for a whole group of rows, the decay factors as
+// E_ij = exp(G_i - G_r) * exp(G_r - G_j), both factors <= 1 (the splitting kda.py:504-523 uses for
+// its forward matrices), and the group's sum over j becomes a small matrix product on
+// v_mfma_f32_16x16x4_f32 with one operand scaled on the fly (fp32 operands: nothing is rounded to
+// bf16 on the way).  Two levels of it: 16-token blocks against everything before (after) them,
+// and the 4-token groups inside a block against the earlier (later) groups of that block -- one
+// accumulator row group of the MFMA is exactly one such group.  Only the 4x4 triangles on the
+// diagonal are left to the VALU (exponents of non-positive numbers).
+// Tiles live in LDS: M [64][LNX_LDA] fp32 (already masked to the lower triangle), G and out
+// [64][ldf] fp32, operands [64][ldb] in T.  All 256 threads must call; each helper contains one
+// workgroup barrier between its two phases (they update `out` with different thread mappings).
 // ---------------------------------------------------------------------------------------
 
 // out[i][c] += mul * sum_{j <= i (j < i if STRICT)} M[i][j] * E_ij[c] * b[j][c]
-// The token loop runs in blocks of 8 whose LDS reads are issued together (the loop is latency
-// bound otherwise); blocks are aligned so that masked tokens multiply by M = 0 / alpha = 1.
-template <typename T, int DK, bool STRICT>
-__device__ __forceinline__ void pair_row(float* out, const float* M, const float* al, int ldf, const T* b, int ldb,
+template <typename T, int CH, bool STRICT>
+__device__ __forceinline__ void pair_row(float* out, const float* M, const float* G, int ldf, const T* b, int ldb,
                                          float mul, int tid) {
-  const int wave = tid >> 6, lane = tid & 63;
-  for (int i = wave; i < 64; i += 4)
-    for (int c = lane; c < DK; c += 64) {
-      float e = 1.f, acc = 0.f;
-      for (int j0 = i | 7; j0 >= 7; j0 -= 8) {  // tokens j0, j0-1, ..., j0-7
-        float m[8], bv[8], av[8];
+  const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, kq = lane >> 4;
+  for (int cb = wave; cb < CH / 16; cb += 4) {
+    const int c = 16 * cb + l16;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int j = j0 - u;  // always a valid row: loads are unconditional, masks applied after
-          m[u] = M[i * LNX_LDA + j];
-          bv[u] = to_f32(b[j * ldb + c]);
-          av[u] = al[j * ldf + c];
-        }
+    for (int I = 0; I < 4; ++I) {
+      floatx4 tot = {0.f, 0.f, 0.f, 0.f};
+      float gi[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int j = j0 - u;
-          const bool on = j <= i;
-          m[u] = (on && !(STRICT && j == i)) ? m[u] : 0.f;
-          av[u] = on ? av[u] : 1.f;
-        }
+      for (int e = 0; e < 4; ++e) gi[e] = G[(16 * I + 4 * kq + e) * ldf + c];
+      // reference 16 I: all tokens before the block; reference 16 I + 4 a: the block's tokens before group a
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          acc += m[u] * e * bv[u];
-          e *= av[u];
+      for (int a = 0; a < 4; ++a) {
+        if (I == 0 && a == 0) continue;
+        const int ref = 16 * I + 4 * a, jlo = (a == 0) ? 0 : 16 * I;
+        const float gref = G[ref * ldf + c];
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j0 = jlo; j0 < ref; j0 += 4) {
+          const int j = j0 + kq;
+          const float av = M[(16 * I + l16) * LNX_LDA + j];
+          const float bv = to_f32(b[j * ldb + c]) * __expf(fminf(gref - G[j * ldf + c], 0.f));
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc, 0, 0, 0);
         }
+        if (a == 0 || kq == a) {  // a > 0: only the rows of group a are meaningful
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tot[e] += acc[e] * __expf(fminf(gi[e] - gref, 0.f));
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) out[(16 * I + 4 * kq + e) * ldf + c] += mul * tot[e];
+    }
+  }
+  lds_barrier();
+  for (int i = wave; i < 64; i += 4) {
+    const int jb = i & ~3;
+    for (int c = lane; c < CH; c += 64) {
+      const float gi = G[i * ldf + c];
+      float m[4], gv[4], bv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {  // unconditional loads, masks applied after
+        m[u] = M[i * LNX_LDA + jb + u];
+        gv[u] = G[(jb + u) * ldf + c];
+        bv[u] = to_f32(b[(jb + u) * ldb + c]);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool on = STRICT ? (jb + u < i) : (jb + u <= i);
+        acc += on ? m[u] * __expf(fminf(gi - gv[u], 0.f)) * bv[u] : 0.f;
       }
       out[i * ldf + c] += mul * acc;
     }
+  }
 }
 
 // out[j][c] += mul * sum_{i >= j (i > j if STRICT)} M[i][j] * E_ij[c] * a[i][c]
-template <typename T, int DK, bool STRICT>
-__device__ __forceinline__ void pair_col(float* out, const float* M, const float* al, int ldf, const T* a, int lda,
+template <typename T, int CH, bool STRICT>
+__device__ __forceinline__ void pair_col(float* out, const float* M, const float* G, int ldf, const T* a, int lda,
                                          float mul, int tid) {
-  const int wave = tid >> 6, lane = tid & 63;
-  for (int j = wave; j < 64; j += 4)
-    for (int c = lane; c < DK; c += 64) {
-      float e = 1.f, acc = 0.f;
-      for (int i0 = j & ~7; i0 < 64; i0 += 8) {  // tokens i0 .. i0+7
-        float m[8], xv[8], av[8];
+  const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, kq = lane >> 4;
+  for (int cb = wave; cb < CH / 16; cb += 4) {
+    const int c = 16 * cb + l16;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u;
-          m[u] = M[i * LNX_LDA + j];
-          xv[u] = to_f32(a[i * lda + c]);
-          av[u] = al[i * ldf + c];
+    for (int J = 0; J < 4; ++J) {
+      floatx4 tot = {0.f, 0.f, 0.f, 0.f};
+      float gj[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gj[e] = G[(16 * J + 4 * kq + e) * ldf + c];
+      // later 16-token blocks (reference: their first token)
+#pragma unroll
+      for (int I = J + 1; I < 4; ++I) {
+        const float gref = G[16 * I * ldf + c];
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i0 = 16 * I; i0 < 16 * I + 16; i0 += 4) {
+          const int i = i0 + kq;
+          const float mv = M[i * LNX_LDA + 16 * J + l16];
+          const float av = to_f32(a[i * lda + c]) * __expf(fminf(G[i * ldf + c] - gref, 0.f));
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(mv, av, acc, 0, 0, 0);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u;
-          m[u] = (i > j || (!STRICT && i == j)) ? m[u] : 0.f;
-          av[u] = (i > j) ? av[u] : 1.f;
-        }
+        for (int e = 0; e < 4; ++e) tot[e] += acc[e] * __expf(fminf(gref - gj[e], 0.f));
+      }
+      // later 4-token groups of the same block (reference: the group's first token); only the
+      // columns of earlier groups are meaningful
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          e *= av[u];
-          acc += m[u] * e * xv[u];
+      for (int g4 = 1; g4 < 4; ++g4) {
+        const int i = 16 * J + 4 * g4 + kq;
+        const float gref = G[(16 * J + 4 * g4) * ldf + c];
+        const float mv = M[i * LNX_LDA + 16 * J + l16];
+        const float av = to_f32(a[i * lda + c]) * __expf(fminf(G[i * ldf + c] - gref, 0.f));
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(mv, av, acc, 0, 0, 0);
+        if (kq < g4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tot[e] += acc[e] * __expf(fminf(gref - gj[e], 0.f));
         }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) out[(16 * J + 4 * kq + e) * ldf + c] += mul * tot[e];
+    }
+  }
+  lds_barrier();
+  for (int j = wave; j < 64; j += 4) {
+    const int ib = j & ~3;
+    for (int c = lane; c < CH; c += 64) {
+      const float gj = G[j * ldf + c];
+      float m[4], gv[4], av[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        m[u] = M[(ib + u) * LNX_LDA + j];
+        gv[u] = G[(ib + u) * ldf + c];
+        av[u] = to_f32(a[(ib + u) * lda + c]);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool on = STRICT ? (ib + u > j) : (ib + u >= j);
+        acc += on ? m[u] * __expf(fminf(gv[u] - gj, 0.f)) * av[u] : 0.f;
       }
       out[j * ldf + c] += mul * acc;
     }
+  }
 }
