@@ -256,29 +256,106 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
       store4(Qgg + r * DK + c, qgv);
     }
   }
-  // pairwise products with the decay inside the channel sum
+  // pairwise products X_ij = <k_i, k_j>_E (i > j) and <q_i, k_j>_E (i >= j) with the decay inside
+  // the channel sum, accumulated in sA and sT.
+  for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) {
+    sA[idx] = 0.f;
+    sT[idx] = 0.f;
+  }
+  lds_barrier();
+  const int l16 = lane & 15, kq = lane >> 4;
   {
-    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
-    T* Xg = ws_ptr<T>(p, p.off.X) + slot * 64 * 64;
-    for (int idx = tid; idx < 64 * 64; idx += 256) {
-      const int i = idx >> 6, j = idx & 63;
-      float x = 0.f, pp = 0.f;
-      if (j <= i) {
-        for (int c = 0; c < DK; c += 4) {
-          const floatx4 gi = load4(sG + i * LDF + c), gj = load4(sG + j * LDF + c);
-          const floatx4 ki = load4(sK + i * LDK + c), kj = load4(sK + j * LDK + c), qi = load4(sQ + i * LDK + c);
+    // 16x16 blocks below the diagonal on the fp32 MFMA: E_ij = exp(G_i - G_ref) exp(G_ref - G_j) with
+    // G_ref the first row of the row block, both factors <= 1 (kda.py:504-523).  Each wave takes a
+    // quarter of the channels; the partial blocks are summed with LDS atomics.
+    constexpr int CW = DK / 4;
+    const int cbase = CW * wave;
+#pragma unroll
+    for (int I = 1; I < 4; ++I) {
+      const int i = 16 * I + l16;
+#pragma unroll
+      for (int J = 0; J < I; ++J) {
+        const int j = 16 * J + l16;
+        floatx4 ax = {0.f, 0.f, 0.f, 0.f}, ap = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < CW / 4; ++ks) {
+          const int c = cbase + 4 * ks + kq;
+          const float gref = sG[16 * I * LDF + c];
+          const float fa = __expf(fminf(sG[i * LDF + c] - gref, 0.f));
+          const float fb = __expf(fminf(gref - sG[j * LDF + c], 0.f));
+          const float kb = to_f32(sK[j * LDK + c]) * fb;
+          ax = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sK[i * LDK + c]) * fa, kb, ax, 0, 0, 0);
+          ap = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sQ[i * LDK + c]) * fa, kb, ap, 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          atomicAdd(&sA[(16 * I + 4 * kq + e) * LNX_LDA + j], ax[e]);
+          atomicAdd(&sT[(16 * I + 4 * kq + e) * LNX_LDA + j], ap[e]);
+        }
+      }
+    }
+  }
+  {
+    // 16x16 blocks on the diagonal on the VALU, exponents of non-positive numbers only
+    // (kda.py:483-502): wave = block, lane = (row, quarter of the channels)
+    constexpr int CQ = DK / 4;
+    const int i = 16 * wave + l16;
+    float xs[16], ps[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) xs[j] = ps[j] = 0.f;
+#pragma unroll 1
+    for (int c0 = kq * CQ; c0 < (kq + 1) * CQ; c0 += 8) {
+      float ki[8], qi[8], gi[8];
+#pragma unroll
+      for (int u = 0; u < 8; u += 4) {
+        const floatx4 a4 = load4(sK + i * LDK + c0 + u), b4 = load4(sQ + i * LDK + c0 + u), g4 = load4(sG + i * LDF + c0 + u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ki[u + e] = a4[e], qi[u + e] = b4[e], gi[u + e] = g4[e];
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int r = 16 * wave + j;
+#pragma unroll
+        for (int u = 0; u < 8; u += 4) {
+          const floatx4 kj = load4(sK + r * LDK + c0 + u), gj = load4(sG + r * LDF + c0 + u);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float ee = __expf(fminf(gi[e] - gj[e], 0.f)) * kj[e];
-            x += ki[e] * ee;
-            pp += qi[e] * ee;
+            const float ee = __expf(fminf(gi[u + e] - gj[e], 0.f)) * kj[e];
+            xs[j] += ki[u + e] * ee;
+            ps[j] += qi[u + e] * ee;
           }
         }
       }
-      x = (j < i) ? x : 0.f;
-      sA[i * LNX_LDA + j] = sBeta[i] * x;
-      Xg[idx] = from_f32<T>(x);
-      Pg[idx] = from_f32<T>(p.scale * pp);
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      xs[j] += __shfl_xor(xs[j], 16, LNX_WAVE);
+      xs[j] += __shfl_xor(xs[j], 32, LNX_WAVE);
+      ps[j] += __shfl_xor(ps[j], 16, LNX_WAVE);
+      ps[j] += __shfl_xor(ps[j], 32, LNX_WAVE);
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if ((j >> 2) == kq) {  // every channel quarter's lanes write four of the columns
+        sA[i * LNX_LDA + 16 * wave + j] = xs[j];
+        sT[i * LNX_LDA + 16 * wave + j] = ps[j];
+      }
+  }
+  lds_barrier();
+  {
+    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
+    T* Xg = ws_ptr<T>(p, p.off.X) + slot * 64 * 64;
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int i = idx >> 4, j0 = (idx & 15) * 4;
+      floatx4 x = load4(sA + i * LNX_LDA + j0), pp = load4(sT + i * LNX_LDA + j0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[e] = (j0 + e < i) ? x[e] : 0.f;
+        pp[e] = (j0 + e <= i) ? p.scale * pp[e] : 0.f;
+      }
+      store4(Xg + i * 64 + j0, x);
+      store4(Pg + i * 64 + j0, pp);
+      store4(sA + i * LNX_LDA + j0, x * sBeta[i]);
     }
   }
   lds_barrier();
