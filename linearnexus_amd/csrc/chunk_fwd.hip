@@ -257,89 +257,62 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
     }
   }
   // pairwise products X_ij = <k_i, k_j>_E (i > j) and <q_i, k_j>_E (i >= j) with the decay inside
-  // the channel sum, accumulated in sA and sT.
-  for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) {
-    sA[idx] = 0.f;
-    sT[idx] = 0.f;
-  }
-  lds_barrier();
+  // the channel sum, formed in sA and sT.
   const int l16 = lane & 15, kq = lane >> 4;
   {
     // 16x16 blocks below the diagonal on the fp32 MFMA: E_ij = exp(G_i - G_ref) exp(G_ref - G_j) with
-    // G_ref the first row of the row block, both factors <= 1 (kda.py:504-523).  Each wave takes a
-    // quarter of the channels; the partial blocks are summed with LDS atomics.
-    constexpr int CW = DK / 4;
-    const int cbase = CW * wave;
-#pragma unroll
-    for (int I = 1; I < 4; ++I) {
-      const int i = 16 * I + l16;
-#pragma unroll
-      for (int J = 0; J < I; ++J) {
-        const int j = 16 * J + l16;
-        floatx4 ax = {0.f, 0.f, 0.f, 0.f}, ap = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < CW / 4; ++ks) {
-          const int c = cbase + 4 * ks + kq;
-          const float gref = sG[16 * I * LDF + c];
-          const float fa = __expf(fminf(sG[i * LDF + c] - gref, 0.f));
-          const float fb = __expf(fminf(gref - sG[j * LDF + c], 0.f));
-          const float kb = to_f32(sK[j * LDK + c]) * fb;
-          ax = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sK[i * LDK + c]) * fa, kb, ax, 0, 0, 0);
-          ap = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sQ[i * LDK + c]) * fa, kb, ap, 0, 0, 0);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          atomicAdd(&sA[(16 * I + 4 * kq + e) * LNX_LDA + j], ax[e]);
-          atomicAdd(&sT[(16 * I + 4 * kq + e) * LNX_LDA + j], ap[e]);
-        }
+    // G_ref the first row of the row block, both factors <= 1 (kda.py:504-523).  Twelve tasks
+    // (six blocks, two products), three per wave.
+    for (int t = wave; t < 12; t += 4) {
+      const int pr = t % 6, I = (pr < 1) ? 1 : (pr < 3) ? 2 : 3, J = pr - ((I == 1) ? 0 : (I == 2) ? 1 : 3);
+      const T* sRow = (t < 6) ? sK : sQ;
+      float* dst = (t < 6) ? sA : sT;
+      const int i = 16 * I + l16, j = 16 * J + l16;
+      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+      for (int ks = 0; ks < DK / 4; ++ks) {
+        const int c = 4 * ks + kq;
+        const float gref = sG[16 * I * LDF + c];
+        const float fa = __expf(fminf(sG[i * LDF + c] - gref, 0.f));
+        const float fb = __expf(fminf(gref - sG[j * LDF + c], 0.f));
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sRow[i * LDK + c]) * fa, to_f32(sK[j * LDK + c]) * fb, acc, 0, 0, 0);
       }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[(16 * I + 4 * kq + e) * LNX_LDA + j] = acc[e];
     }
   }
   {
     // 16x16 blocks on the diagonal on the VALU, exponents of non-positive numbers only
-    // (kda.py:483-502): wave = block, lane = (row, quarter of the channels)
-    constexpr int CQ = DK / 4;
-    const int i = 16 * wave + l16;
-    float xs[16], ps[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j) xs[j] = ps[j] = 0.f;
+    // (kda.py:483-502): wave = block; lane = (pair of rows rp and 15 - rp, eighth of the channels).
+    // The two rows together have 17 columns j <= i, walked in one loop of 17 steps.
+    constexpr int CE = DK / 8;
+    const int rp = lane & 7, ce = lane >> 3, r0 = 16 * wave;
 #pragma unroll 1
-    for (int c0 = kq * CQ; c0 < (kq + 1) * CQ; c0 += 8) {
-      float ki[8], qi[8], gi[8];
+    for (int t = 0; t < 17; ++t) {
+      const bool first = t <= rp;
+      const int i = r0 + (first ? rp : 15 - rp), j = r0 + (first ? t : t - rp - 1);
+      float x = 0.f, pp = 0.f;
 #pragma unroll
-      for (int u = 0; u < 8; u += 4) {
-        const floatx4 a4 = load4(sK + i * LDK + c0 + u), b4 = load4(sQ + i * LDK + c0 + u), g4 = load4(sG + i * LDF + c0 + u);
+      for (int c = ce * CE; c < (ce + 1) * CE; c += 4) {
+        const floatx4 ki = load4(sK + i * LDK + c), qi = load4(sQ + i * LDK + c), gi = load4(sG + i * LDF + c);
+        const floatx4 kj = load4(sK + j * LDK + c), gj = load4(sG + j * LDF + c);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) ki[u + e] = a4[e], qi[u + e] = b4[e], gi[u + e] = g4[e];
-      }
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int r = 16 * wave + j;
-#pragma unroll
-        for (int u = 0; u < 8; u += 4) {
-          const floatx4 kj = load4(sK + r * LDK + c0 + u), gj = load4(sG + r * LDF + c0 + u);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float ee = __expf(fminf(gi[u + e] - gj[e], 0.f)) * kj[e];
-            xs[j] += ki[u + e] * ee;
-            ps[j] += qi[u + e] * ee;
-          }
+        for (int e = 0; e < 4; ++e) {
+          const float ee = __expf(fminf(gi[e] - gj[e], 0.f)) * kj[e];
+          x += ki[e] * ee;
+          pp += qi[e] * ee;
         }
       }
-    }
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      xs[j] += __shfl_xor(xs[j], 16, LNX_WAVE);
-      xs[j] += __shfl_xor(xs[j], 32, LNX_WAVE);
-      ps[j] += __shfl_xor(ps[j], 16, LNX_WAVE);
-      ps[j] += __shfl_xor(ps[j], 32, LNX_WAVE);
-    }
-#pragma unroll
-    for (int j = 0; j < 16; ++j)
-      if ((j >> 2) == kq) {  // every channel quarter's lanes write four of the columns
-        sA[i * LNX_LDA + 16 * wave + j] = xs[j];
-        sT[i * LNX_LDA + 16 * wave + j] = ps[j];
+      for (int m = 8; m < 64; m <<= 1) {
+        x += __shfl_xor(x, m, LNX_WAVE);
+        pp += __shfl_xor(pp, m, LNX_WAVE);
       }
+      if (ce == 0) {
+        sA[i * LNX_LDA + j] = x;
+        sT[i * LNX_LDA + j] = pp;
+      }
+    }
   }
   lds_barrier();
   {
