@@ -452,6 +452,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     if (tid < 64) {
       for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDC + tid]);
       dgc += __expf(Gg[63 * DK + tid]) * sSS[tid];
+      sSS[tid] = dgc;  // chunk-end gate term, added to row 63 below
     }
     lds_barrier();
     pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
@@ -461,10 +462,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       const int r = idx >> 4, c = (idx & 15) * 4;
       const floatx4 v = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
       if (r < len) store4(dkg + (int64_t)r * DK + c, v);
-      store4(dGg + r * DK + c, load4(dGg + r * DK + c) - kk * v);
+      floatx4 dgv = load4(dGg + r * DK + c) - kk * v;  // written above by this same thread
+      if (r == 63) dgv += load4(sSS + c);
+      store4(dGg + r * DK + c, dgv);
     }
-    lds_barrier();
-    if (tid < 64) dGg[63 * DK + tid] += dgc;
   } else {
     // ---- scalar / no gate ----
     T* sPe = sdO;     // scale E dP   [i][j]
@@ -537,18 +538,18 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK, int GATE> struct WyCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
+  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = 64 + 4;
   static constexpr int kR1 = 64 * LDC;                                       // Tm^T, later Y
   static constexpr int kR2 = (128 * LDC > 64 * LDK) ? 128 * LDC : 64 * LDK;  // dW^T | dD^T + dBu | dBw | K^T
   static constexpr int kR3 = 64 * LDK;                                       // U slab | W | K
   static constexpr size_t mma_bytes = sizeof(T) * (kR1 + kR2 + kR3);
-  static constexpr size_t vec_bytes = sizeof(float) * 3 * 64 * LDF + sizeof(T) * 64 * LDK;  // alpha, out+, out-, K (X borrows out-)
+  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 64 * LDC;  // vector gate, per 64-channel half: G, out, K
   static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > mma_bytes) ? vec_bytes : mma_bytes;
   static constexpr size_t bytes = sizeof(float) * (64 * LNX_LDA + 64 * 4) + big;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_wy_kernel(BwdParams p) {
   typedef WyCfg<T, DK, GATE> L;
   typedef RowTiles<DK> RTl;
   constexpr int LDK = L::LDK, LDC = L::LDC, LDF = L::LDF, MT = RTl::MT;
@@ -628,83 +629,98 @@ __global__ __launch_bounds__(256) void bwd_wy_kernel(BwdParams p) {
 
   static_assert(GATE == LNX_GATE_VECTOR, "bwd_wy2 handles the other gate kinds");
   {
-    // ---- per-channel gate ----
-    float* sAl = reinterpret_cast<float*>(R1);  // [64][LDF] cumulative gate
-    float* sOp = sAl + 64 * LDF;                // row-type part of dk (through B_w and the rows of X)
-    float* sOm = sOp + 64 * LDF;                // column-type part of dk (columns of X)
-    T* sKr = reinterpret_cast<T*>(sOm + 64 * LDF);
-    T* sXp = reinterpret_cast<T*>(sOm);  // X = <k_i, k_j>_E from the forward pass, until out- is needed
+    // ---- per-channel gate: the pair terms of dk and dG, one 64-channel half at a time ----
+    float* sGc = reinterpret_cast<float*>(R1);       // [64][LDF] cumulative gate of the half
+    float* sOut = sGc + 64 * LDF;                    // [64][LDF] row-type part of dk, then the column-type part
+    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC]
+    T* sXp = reinterpret_cast<T*>(sOut);             // X = <k_i, k_j>_E from the forward pass, until out is needed
     const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
     float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
     stage_tile<T, 64, 64>(sXp, LDC, wsp<T>(p, p.off.X) + slot * 64 * 64, 64, 64, tid);
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
     }
-    stage_tile<T, 64, DK>(sKr, LDK, kg, DK, len, tid);
-    {
-      constexpr int IT = 64 * DK / 4 / 256;
-      floatx4 g1[IT];
-#pragma unroll
-      for (int it = 0; it < IT; ++it) {
-        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-        g1[it] = load4(Gg + r * DK + c);
-      }
-#pragma unroll
-      for (int it = 0; it < IT; ++it) {
-        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-        store4(sAl + r * LDF + c, g1[it]);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = r0 + 32 * i + frag_row(e, lane), c = c0 + frag_col(lane);
-        sOp[r * LDF + c] = aBw[i][0][e] * __expf(Gg[r * DK + c]);  // e^G dBw
-      }
     lds_barrier();
-    if (tid < 64) {  // dbeta += sum_j dA_ij X_ij
+    {  // dbeta += sum_j dA_ij X_ij, then dX = beta_i dA_ij in place; thread = (row, quarter of the columns)
+      const int r = tid >> 2, j0 = (tid & 3) * 16;
       float rs = 0.f;
-      for (int j = 0; j < tid; ++j) rs += sR[tid * LNX_LDA + j] * to_f32(sXp[tid * LDC + j]);
-      atomicAdd(&sdB[tid], rs);
-    }
-    for (int r = wave; r < 64; r += 4) {  // dbeta += <e^G dBw, k>;  out+ = beta e^G dBw
-      float t = 0.f;
-      for (int c = lane; c < DK; c += 64) {
-        t += sOp[r * LDF + c] * to_f32(sKr[r * LDK + c]);
-        sOp[r * LDF + c] *= sBeta[r];
-      }
-      t = wave_sum(t);
-      if (lane == 0) atomicAdd(&sdB[r], t);
-    }
-    lds_barrier();
-    for (int idx = tid; idx < 64 * 64; idx += 256) sR[(idx >> 6) * LNX_LDA + (idx & 63)] *= sBeta[idx >> 6];  // dX
-    for (int idx = tid; idx < 64 * DK; idx += 256) sOm[(idx / DK) * LDF + idx % DK] = 0.f;
-    lds_barrier();
-    pair_row<T, DK, true>(sOp, sR, sAl, LDF, sKr, LDK, 1.f, tid);
-    pair_col<T, DK, true>(sOm, sR, sAl, LDF, sKr, LDK, 1.f, tid);
-    lds_barrier();
-    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
-    {
-      constexpr int IT = 64 * DK / 4 / 256;
-      floatx4 dk0[IT], dg0[IT];
 #pragma unroll
-      for (int it = 0; it < IT; ++it) {  // all global reads first
-        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + c) : floatx4{0.f, 0.f, 0.f, 0.f};
-        dg0[it] = load4(dGg + r * DK + c);
-      }
+      for (int u = 0; u < 16; u += 4) {
+        const floatx4 a4 = load4(sR + r * LNX_LDA + j0 + u), x4 = load4(sXp + r * LDC + j0 + u);
 #pragma unroll
-      for (int it = 0; it < IT; ++it) {
-        const int idx = tid + 256 * it, r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-        const floatx4 up = load4(sOp + r * LDF + c), um = load4(sOm + r * LDF + c), kk = load4(sKr + r * LDK + c);
-        if (r < len) store4(dkg + (int64_t)r * DK + c, dk0[it] + up + um);
-        store4(dGg + r * DK + c, dg0[it] + kk * (up - um));
+        for (int e = 0; e < 4; ++e) rs += a4[e] * x4[e];
+        store4(sR + r * LNX_LDA + j0 + u, a4 * sBeta[r]);
+      }
+      rs += __shfl_xor(rs, 1, LNX_WAVE);
+      rs += __shfl_xor(rs, 2, LNX_WAVE);
+      if ((tid & 3) == 0) atomicAdd(&sdB[r], rs);
+    }
+    for (int h = 0; h < DK / 64; ++h) {
+      const int ch0 = 64 * h;
+      floatx4 dk0[4], dg0[4], up[4];
+      lds_barrier();  // X tile / the previous half's tiles are dead
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {  // all global reads of the half first
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        up[it] = load4(Gg + r * DK + ch0 + c);
+        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+        dg0[it] = load4(dGg + r * DK + ch0 + c);
+      }
+      stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, DK, len, tid);
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        store4(sGc + r * LDF + c, up[it]);
+      }
+      lds_barrier();
+      if (DK == 64 || (wave >> 1) == h) {  // the waves whose dBw columns lie in this half: out = e^G dBw
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int r = r0 + 32 * i + frag_row(e, lane), c = c0 - ch0 + frag_col(lane);
+            sOut[r * LDF + c] = aBw[i][0][e] * __expf(sGc[r * LDF + c]);
+          }
+      }
+      lds_barrier();
+      {  // dbeta += <e^G dBw, k>;  out = beta e^G dBw; thread = (row, quarter of the channels)
+        const int r = tid >> 2, q0 = (tid & 3) * 16;
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < 16; u += 4) {
+          const floatx4 o4 = load4(sOut + r * LDF + q0 + u), k4 = load4(sKr + r * LDC + q0 + u);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) t += o4[e] * k4[e];
+          store4(sOut + r * LDF + q0 + u, o4 * sBeta[r]);
+        }
+        t += __shfl_xor(t, 1, LNX_WAVE);
+        t += __shfl_xor(t, 2, LNX_WAVE);
+        if ((tid & 3) == 0) atomicAdd(&sdB[r], t);
+      }
+      lds_barrier();
+      pair_row<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      lds_barrier();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {  // row-type part to registers, out restarts from zero
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        up[it] = load4(sOut + r * LDF + c);
+        store4(sOut + r * LDF + c, floatx4{0.f, 0.f, 0.f, 0.f});
+      }
+      lds_barrier();
+      pair_col<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      lds_barrier();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        const floatx4 um = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
+        if (r < len) store4(dkg + (int64_t)r * DK + ch0 + c, dk0[it] + up[it] + um);
+        store4(dGg + r * DK + ch0 + c, dg0[it] + kk * (up[it] - um));
       }
     }
-    lds_barrier();
+    __syncthreads();  // dG is read back below by other threads than wrote it: global memory must be ordered too
     if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
     if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
       float gv[64];
