@@ -39,28 +39,6 @@ template <typename T> __device__ __forceinline__ T* wsp(const BwdParams& p, uint
   return reinterpret_cast<T*>(p.ws + off);
 }
 
-// Tiling of a [64 x DK] product over four waves: DK=128 -> both row tiles, column tile = wave;
-// DK=64 -> one 32x32 tile per wave.
-template <int DK> struct RowTiles {
-  static constexpr int MT = (DK == 128) ? 2 : 1;
-  static __device__ __forceinline__ int row0(int wave) { return (DK == 128) ? 0 : 32 * (wave >> 1); }
-  static __device__ __forceinline__ int col0(int wave) { return (DK == 128) ? 32 * wave : 32 * (wave & 1); }
-};
-
-// acc_rows[row0 + r] += sum over this wave's columns of acc[r][c] * partner(r, c); the caller
-// zeroes `rows` and synchronises.  partner(row, col) gives the element to multiply with.
-template <int MT, typename F>
-__device__ __forceinline__ void frag_rowdot(const floatx16 (&acc)[MT][1], int row0, int col0, int lane, float* rows,
-                                            F partner) {
-  float v[16 * MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e)
-      v[16 * i + e] = acc[i][0][e] * partner(row0 + 32 * i + frag_row(e, lane), col0 + frag_col(lane));
-  rows_reduce_add<MT>(v, row0, lane, rows);
-}
-
 // ---------------------------------------------------------------------------------------
 // bwd_local: dD_loc[j][v] = sum_i P[i][j] dO[i][v]; dO^T slab to the workspace
 // ---------------------------------------------------------------------------------------
@@ -534,224 +512,28 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
 }
 
 // ---------------------------------------------------------------------------------------
-// bwd_wy
+// bwd_wy2: gradients through the WY transform (dBw = Tm^T dW, dBu = Tm^T dD, dv, dbeta,
+// dA = -tril(dBw W^T + dBu U^T, -1) and its contributions to dk and dg) as one loop over 64-column
+// slabs of [dk | dv] with the next slab's tiles prefetched into registers, every product one
+// 32x32 tile per wave, row and column sums taken from the fragments, results stored through LDS
+// with 16-byte vectors.  The per-channel (vector) gate replaces the dense dA products of the
+// epilogue by the pair-term helpers, one 64-channel half at a time.
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK, int GATE> struct WyCfg {
+template <typename T, int DK, int GATE> struct Wy2Cfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = 64 + 4;
-  static constexpr int kR1 = 64 * LDC;                                       // Tm^T, later Y
-  static constexpr int kR2 = (128 * LDC > 64 * LDK) ? 128 * LDC : 64 * LDK;  // dW^T | dD^T + dBu | dBw | K^T
-  static constexpr int kR3 = 64 * LDK;                                       // U slab | W | K
-  static constexpr size_t mma_bytes = sizeof(T) * (kR1 + kR2 + kR3);
-  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 64 * LDC;  // vector gate, per 64-channel half: G, out, K
-  static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > mma_bytes) ? vec_bytes : mma_bytes;
-  static constexpr size_t bytes = sizeof(float) * (64 * LNX_LDA + 64 * 4) + big;
-};
-
-template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_wy_kernel(BwdParams p) {
-  typedef WyCfg<T, DK, GATE> L;
-  typedef RowTiles<DK> RTl;
-  constexpr int LDK = L::LDK, LDC = L::LDC, LDF = L::LDF, MT = RTl::MT;
-  extern __shared__ __align__(16) char smem[];
-  float* sR = reinterpret_cast<float*>(smem);  // [64][LNX_LDA]: dA * X (scalar) or dA, then beta dA (vector)
-  float* sG = sR + 64 * LNX_LDA;
-  float* sBeta = sG + 64;
-  float* sdB = sBeta + 64;  // dbeta accumulator
-  float* sdG = sdB + 64;    // gate-gradient accumulator (wrt cumulative G)
-  T* R1 = reinterpret_cast<T*>(sdG + 64);
-  T* R2 = R1 + L::kR1;
-  T* R3 = R2 + L::kR2;
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int N = p.geom.N;
-  const int64_t slot = blockIdx.x;
-  const int row = (int)(slot / N), n = (int)(slot % N);
-  int tok0, len;
-  chunk_span(p.geom, n, tok0, len);
-  if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
-  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
-  const int wi = wave >> 1, wj = wave & 1;
-  const int r0 = RTl::row0(wave), c0 = RTl::col0(wave);
-
-  if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
-    sdB[tid] = 0.f;
-    sdG[tid] = 0.f;
-  }
-  // phase 1: dBw = Tm^T dW
-  T* sTmT = R1;
-  T* sdWT = R2;
-  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
-  stage_tile_t<T, 64, DK>(sdWT, LDC, wsp<T>(p, p.off.dW) + slot * 64 * DK, DK, 64, tid);
-  lds_barrier();
-  floatx16 aBw[MT][1], aM[1][1];
-  frag_zero(aBw);
-  frag_zero(aM);
-  mma_nt<T, MT, 1>(aBw, sTmT + r0 * LDC, LDC, sdWT + c0 * LDC, LDC, 64, lane);
-
-  // phase 2: per dv slab, dBu = Tm^T dD;  dv = beta dBu;  dbeta += <dBu, v>;  dM += dBu U^T
-  T* sdDT = R2;
-  T* sdBu = R2 + 64 * LDC;
-  T* sU = R3;
-  for (int v0 = 0; v0 < p.dv; v0 += 64) {
-    lds_barrier();
-    stage_tile_t<T, 64, 64>(sdDT, LDC, wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    stage_tile<T, 64, 64>(sU, LDC, wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    lds_barrier();
-    floatx16 bu[1][1];
-    frag_zero(bu);
-    mma_nt<T, 1, 1>(bu, sTmT + 32 * wi * LDC, LDC, sdDT + 32 * wj * LDC, LDC, 64, lane);
-    frag_store<T, 1, 1>(bu, sdBu + 32 * wi * LDC + 32 * wj, LDC, lane);
-    frag_rowdot<1>(bu, 32 * wi, 32 * wj, lane, sdB, [&](int r, int c) {
-      return (r < len) ? to_f32(vg[(int64_t)r * p.dv + v0 + c]) : 0.f;
-    });
-#pragma unroll
-    for (int e = 0; e < 16; ++e) bu[0][0][e] *= sBeta[32 * wi + frag_row(e, lane)];
-    frag_store<T, 1, 1>(bu, reinterpret_cast<T*>(p.dv_out) + (tbase + 32 * wi) * p.dv + v0 + 32 * wj, p.dv, lane,
-                        len - 32 * wi);
-    lds_barrier();
-    mma_nt<T, 1, 1>(aM, sdBu + 32 * wi * LDC, LDC, sU + 32 * wj * LDC, LDC, 64, lane);
-  }
-  lds_barrier();
-
-  // phase 3: dM += dBw W^T
-  T* sdBw = R2;
-  T* sW = R3;
-  frag_store<T, MT, 1>(aBw, sdBw + r0 * LDK + c0, LDK, lane);
-  stage_tile<T, 64, DK>(sW, LDK, wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
-  lds_barrier();
-  mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDK, LDK, sW + 32 * wj * LDK, LDK, DK, lane);
-  lds_barrier();
-
-  static_assert(GATE == LNX_GATE_VECTOR, "bwd_wy2 handles the other gate kinds");
-  {
-    // ---- per-channel gate: the pair terms of dk and dG, one 64-channel half at a time ----
-    float* sGc = reinterpret_cast<float*>(R1);       // [64][LDF] cumulative gate of the half
-    float* sOut = sGc + 64 * LDF;                    // [64][LDF] row-type part of dk, then the column-type part
-    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC]
-    T* sXp = reinterpret_cast<T*>(sOut);             // X = <k_i, k_j>_E from the forward pass, until out is needed
-    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
-    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
-    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
-    stage_tile<T, 64, 64>(sXp, LDC, wsp<T>(p, p.off.X) + slot * 64 * 64, 64, 64, tid);
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
-    }
-    lds_barrier();
-    {  // dbeta += sum_j dA_ij X_ij, then dX = beta_i dA_ij in place; thread = (row, quarter of the columns)
-      const int r = tid >> 2, j0 = (tid & 3) * 16;
-      float rs = 0.f;
-#pragma unroll
-      for (int u = 0; u < 16; u += 4) {
-        const floatx4 a4 = load4(sR + r * LNX_LDA + j0 + u), x4 = load4(sXp + r * LDC + j0 + u);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) rs += a4[e] * x4[e];
-        store4(sR + r * LNX_LDA + j0 + u, a4 * sBeta[r]);
-      }
-      rs += __shfl_xor(rs, 1, LNX_WAVE);
-      rs += __shfl_xor(rs, 2, LNX_WAVE);
-      if ((tid & 3) == 0) atomicAdd(&sdB[r], rs);
-    }
-    for (int h = 0; h < DK / 64; ++h) {
-      const int ch0 = 64 * h;
-      floatx4 dk0[4], dg0[4], up[4];
-      lds_barrier();  // X tile / the previous half's tiles are dead
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {  // all global reads of the half first
-        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
-        up[it] = load4(Gg + r * DK + ch0 + c);
-        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
-        dg0[it] = load4(dGg + r * DK + ch0 + c);
-      }
-      stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, DK, len, tid);
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
-        store4(sGc + r * LDF + c, up[it]);
-      }
-      lds_barrier();
-      if (DK == 64 || (wave >> 1) == h) {  // the waves whose dBw columns lie in this half: out = e^G dBw
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int r = r0 + 32 * i + frag_row(e, lane), c = c0 - ch0 + frag_col(lane);
-            sOut[r * LDF + c] = aBw[i][0][e] * __expf(sGc[r * LDF + c]);
-          }
-      }
-      lds_barrier();
-      {  // dbeta += <e^G dBw, k>;  out = beta e^G dBw; thread = (row, quarter of the channels)
-        const int r = tid >> 2, q0 = (tid & 3) * 16;
-        float t = 0.f;
-#pragma unroll
-        for (int u = 0; u < 16; u += 4) {
-          const floatx4 o4 = load4(sOut + r * LDF + q0 + u), k4 = load4(sKr + r * LDC + q0 + u);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) t += o4[e] * k4[e];
-          store4(sOut + r * LDF + q0 + u, o4 * sBeta[r]);
-        }
-        t += __shfl_xor(t, 1, LNX_WAVE);
-        t += __shfl_xor(t, 2, LNX_WAVE);
-        if ((tid & 3) == 0) atomicAdd(&sdB[r], t);
-      }
-      lds_barrier();
-      pair_row<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
-      lds_barrier();
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {  // row-type part to registers, out restarts from zero
-        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
-        up[it] = load4(sOut + r * LDF + c);
-        store4(sOut + r * LDF + c, floatx4{0.f, 0.f, 0.f, 0.f});
-      }
-      lds_barrier();
-      pair_col<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
-      lds_barrier();
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
-        const floatx4 um = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
-        if (r < len) store4(dkg + (int64_t)r * DK + ch0 + c, dk0[it] + up[it] + um);
-        store4(dGg + r * DK + ch0 + c, dg0[it] + kk * (up[it] - um));
-      }
-    }
-    __syncthreads();  // dG is read back below by other threads than wrote it: global memory must be ordered too
-    if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
-    if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
-      float gv[64];
-#pragma unroll
-      for (int r = 0; r < 64; ++r) gv[r] = dGg[r * DK + tid];  // all loads in flight together
-      float acc = 0.f;
-#pragma unroll
-      for (int r = 63; r >= 0; --r) {
-        acc += gv[r];
-        if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// bwd_wy2 (no gate / scalar gate): bwd_wy as one loop over 64-column slabs of [dk | dv] with the
-// next slab's tiles prefetched into registers, every product one 32x32 tile per wave, row and
-// column sums taken from the fragments, results stored through LDS with 16-byte vectors.
-// ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct Wy2Cfg {
-  static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDC = LNX_C + PAD;
+  static constexpr int LDC = LNX_C + PAD, LDF = 64 + 4;
   static constexpr int kTile = 64 * LDC;
-  static constexpr size_t bytes = sizeof(T) * 5 * kTile + sizeof(float) * 64 * 6;
+  static constexpr size_t nfloat = 64 * 6 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0);  // + dA (vector gate)
+  // vector-gate epilogue inside the tile region: G and out [64][LDF] fp32, K rows [64][LDC]
+  static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * kTile;
+  static_assert(GATE != LNX_GATE_VECTOR || vec_bytes <= sizeof(T) * 5 * kTile, "epilogue tiles overlay the loop tiles");
+  static constexpr size_t bytes = sizeof(T) * 5 * kTile + sizeof(float) * nfloat;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(BwdParams p) {
-  typedef Wy2Cfg<T, DK> L;
-  constexpr int LDC = L::LDC, NKS = DK / 64;
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2 : 3) : 1)) void bwd_wy2_kernel(BwdParams p) {
+  typedef Wy2Cfg<T, DK, GATE> L;
+  constexpr int LDC = L::LDC, LDF = L::LDF, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
   float* sG = reinterpret_cast<float*>(smem);
   float* sBeta = sG + 64;
@@ -759,7 +541,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
   float* sdGk = sdB + 64;    // e^{G} <dBw, k>
   float* sRow = sdGk + 64;   // sum_j dA_ij E_ij X_ij
   float* sCol = sRow + 64;   // sum_i beta_i dA_ij E_ij X_ij
-  T* sTmT = reinterpret_cast<T*>(sCol + 64);
+  float* sR = sCol + 64;     // vector gate only: dA, then beta dA  [64][LNX_LDA]
+  T* sTmT = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
   T* sIn = sTmT + L::kTile;   // dW^T / dD^T slab  [col][token]
   T* sWU = sIn + L::kTile;    // W / U slab        [token][col]
   T* sdBt = sWU + L::kTile;   // dB slab           [token][col]
@@ -829,7 +612,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
         const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
         v[e] = b[0][0][e] * to_f32(sKs[r * LDC + c]);
       }
-      rows_reduce_add<1>(v, 32 * wi, lane, is_k ? sdGk : sdB);
+      if (GATE != LNX_GATE_VECTOR || !is_k) rows_reduce_add<1>(v, 32 * wi, lane, is_k ? sdGk : sdB);
     }
     if (is_k) {
 #pragma unroll
@@ -838,7 +621,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
 #pragma unroll
           for (int e = 0; e < 16; ++e) aBw[u][0][0][e] = b[0][0][e];
         }
-      if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
+      if (GATE != LNX_GATE_VECTOR && !(wi == 0 && wj == 1))
+        mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
     }
     lds_barrier();
     mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
@@ -855,6 +639,114 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
         }
       }
     }
+  }
+  if constexpr (GATE == LNX_GATE_VECTOR) {
+    lds_barrier();  // loop tiles dead
+    // ---- per-channel gate: the pair terms of dk and dG, one 64-channel half at a time ----
+    float* sGc = reinterpret_cast<float*>(sTmT);     // [64][LDF] cumulative gate of the half
+    float* sOut = sGc + 64 * LDF;                    // [64][LDF] row-type part of dk, then the column-type part
+    T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC]
+    T* sXp = reinterpret_cast<T*>(sOut);             // X = <k_i, k_j>_E from the forward pass, until out is needed
+    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK;
+    float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK;
+    T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK;
+    stage_tile<T, 64, 64>(sXp, LDC, wsp<T>(p, p.off.X) + slot * 64 * 64, 64, 64, tid);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
+    }
+    lds_barrier();
+    {  // dbeta += sum_j dA_ij X_ij, then dX = beta_i dA_ij in place; thread = (row, quarter of the columns)
+      const int r = tid >> 2, j0 = (tid & 3) * 16;
+      float rs = 0.f;
+#pragma unroll
+      for (int u = 0; u < 16; u += 4) {
+        const floatx4 a4 = load4(sR + r * LNX_LDA + j0 + u), x4 = load4(sXp + r * LDC + j0 + u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) rs += a4[e] * x4[e];
+        store4(sR + r * LNX_LDA + j0 + u, a4 * sBeta[r]);
+      }
+      rs += __shfl_xor(rs, 1, LNX_WAVE);
+      rs += __shfl_xor(rs, 2, LNX_WAVE);
+      if ((tid & 3) == 0) atomicAdd(&sdB[r], rs);
+    }
+    for (int h = 0; h < DK / 64; ++h) {
+      const int ch0 = 64 * h;
+      floatx4 dk0[4], dg0[4], up[4];
+      lds_barrier();  // X tile / the previous half's tiles are dead
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {  // all global reads of the half first
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        up[it] = load4(Gg + r * DK + ch0 + c);
+        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+        dg0[it] = load4(dGg + r * DK + ch0 + c);
+      }
+      stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, DK, len, tid);
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        store4(sGc + r * LDF + c, up[it]);
+      }
+      lds_barrier();
+#pragma unroll
+      for (int u = 0; u < NKS; ++u)
+        if (u == h) {  // out = e^G dBw
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+            sOut[r * LDF + c] = aBw[u][0][0][e] * __expf(sGc[r * LDF + c]);
+          }
+        }
+      lds_barrier();
+      {  // dbeta += <e^G dBw, k>;  out = beta e^G dBw; thread = (row, quarter of the channels)
+        const int r = tid >> 2, q0 = (tid & 3) * 16;
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < 16; u += 4) {
+          const floatx4 o4 = load4(sOut + r * LDF + q0 + u), k4 = load4(sKr + r * LDC + q0 + u);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) t += o4[e] * k4[e];
+          store4(sOut + r * LDF + q0 + u, o4 * sBeta[r]);
+        }
+        t += __shfl_xor(t, 1, LNX_WAVE);
+        t += __shfl_xor(t, 2, LNX_WAVE);
+        if ((tid & 3) == 0) atomicAdd(&sdB[r], t);
+      }
+      lds_barrier();
+      pair_row<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      lds_barrier();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {  // row-type part to registers, out restarts from zero
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        up[it] = load4(sOut + r * LDF + c);
+        store4(sOut + r * LDF + c, floatx4{0.f, 0.f, 0.f, 0.f});
+      }
+      lds_barrier();
+      pair_col<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      lds_barrier();
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        const floatx4 um = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
+        if (r < len) store4(dkg + (int64_t)r * DK + ch0 + c, dk0[it] + up[it] + um);
+        store4(dGg + r * DK + ch0 + c, dg0[it] + kk * (up[it] - um));
+      }
+    }
+    __syncthreads();  // dG is read back below by other threads than wrote it: global memory must be ordered too
+    if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
+    if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
+      float gv[64];
+#pragma unroll
+      for (int r = 0; r < 64; ++r) gv[r] = dGg[r * DK + tid];  // all loads in flight together
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 63; r >= 0; --r) {
+        acc += gv[r];
+        if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
+      }
+    }
+    return;
   }
   // K slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
   TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
@@ -935,22 +827,14 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 3 : 1)) void bwd_wy2_kernel(
   }
 }
 
-template <typename T, int DK, int GATE> struct WySelect {
-  static constexpr size_t bytes = Wy2Cfg<T, DK>::bytes;
-  static auto kernel() { return bwd_wy2_kernel<T, DK, GATE>; }
-};
-template <typename T, int DK> struct WySelect<T, DK, LNX_GATE_VECTOR> {
-  static constexpr size_t bytes = WyCfg<T, DK, LNX_GATE_VECTOR>::bytes;
-  static auto kernel() { return bwd_wy_kernel<T, DK, LNX_GATE_VECTOR>; }
-};
 
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   auto k1 = bwd_scan_kernel<T, DK, GATE>;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
-  auto k3 = WySelect<T, DK, GATE>::kernel();
-  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = WySelect<T, DK, GATE>::bytes;
+  auto k3 = bwd_wy2_kernel<T, DK, GATE>;
+  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = Wy2Cfg<T, DK, GATE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
