@@ -384,22 +384,35 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
 // Per chunk: D = U - W S, the state update, and -- for 2-byte inputs, where the tiles fit LDS --
 // the outputs o = scale e^G (Q S) + P D of the same slab, so the state and D are not read back
 // by a separate output kernel.
+//
+// The pass is one dependent chain per workgroup and only (states x slabs) workgroups exist, so
+// nothing hides memory instructions behind another workgroup.  The 512 threads therefore split
+// into two roles, one wave of each per SIMD: waves 0-3 do the matrix work on the tiles in LDS,
+// waves 4-7 ("movers") only move data -- global loads two chunks ahead into registers, tile
+// writes into LDS as soon as the previous chunk's reader is done with a tile, and the
+// LDS -> global copies of the state, D and the outputs.  Three barriers per chunk:
+//   B1  tiles of chunk n and the entering state S_n (transposed, LDS) are complete
+//         compute: D                         movers: loads of chunk n+2, S_n -> workspace
+//   B2  D is in LDS (plain in place of U, decay-scaled and transposed for the update)
+//         compute: outputs, state update     movers: W of chunk n+1 -> LDS, D -> workspace
+//   B3  all reads of chunk n's tiles are done
+//         compute: S_{n+1} -> LDS            movers: remaining tiles of chunk n+1 -> LDS, outputs -> global
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct ScanSmem {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
-  static constexpr int BV = 64;  // dv slab per workgroup (32 was measured slower for the forward scan)
+  static constexpr int BV = 64;  // dv slab per workgroup
   static constexpr bool FUSE_OUT = sizeof(T) == 2;
   static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
   static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr int kQ = FUSE_OUT ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
-                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * 128;
+                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (128 + 4);
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
+__global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   typedef ScanSmem<T, DK> L;
   constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD, LDO = L::LDO;
   constexpr bool FUSE = L::FUSE_OUT;
@@ -418,6 +431,7 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   T* sP = sQ + L::kQ;
   bf16_t* sO = reinterpret_cast<bf16_t*>(sP + L::kP);
   float* sG = reinterpret_cast<float*>(sO + (FUSE ? 64 * LDO : 0));
+  int* sMeta = reinterpret_cast<int*>(sG + 128);  // first token and length of the chunk whose tiles are in LDS
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
@@ -426,6 +440,87 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
   const int v0 = blockIdx.y * BV;
   int c0, c1;
   seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+
+  if (wave >= 4) {
+    // ---------------- movers ----------------
+    const int mt = tid - 256;
+    struct Tiles {
+      TileRegs<T, 64, DK> W, K;
+      TileRegs<T, 64, BV> U;
+      TileRegs<T, 64, FUSE ? DK : 8> Q;
+      TileRegs<T, 64, FUSE ? 64 : 8> P;
+      float G;
+      int tok0, len;
+    };
+    // register sets: 2-byte inputs are fetched two chunks ahead (two sets used alternately), 4-byte
+    // inputs one chunk ahead (a second set would not fit the register file)
+    constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;
+    Tiles ta, tb;
+    ta.G = tb.G = 0.f;
+    ta.tok0 = ta.len = tb.tok0 = tb.len = 0;
+    auto fetch = [&](Tiles& R, int n) {
+      const int64_t slot = (int64_t)row * N + n;
+      chunk_span(p.geom, n, R.tok0, R.len);
+      const int64_t tbase = (int64_t)row * p.geom.T + R.tok0;
+      R.W.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+      if (GATE == LNX_GATE_VECTOR) R.K.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+      else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, R.len, mt);
+      R.U.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+      if (FUSE) {
+        if (GATE == LNX_GATE_VECTOR) R.Q.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+        else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, R.len, mt);
+        R.P.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      }
+      if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = ws_ptr<float>(p, p.off.G)[slot * 64 + mt];
+      if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];  // G_last[c]
+    };
+    auto commit_rest = [&](const Tiles& R) {
+      R.K.store(sK, LDK, mt);
+      R.U.store(sU, LDU, mt);
+      if (FUSE) {
+        R.Q.store(sQ, LDK, mt);
+        R.P.store(sP, LDC, mt);
+      }
+      if (mt < 128) sG[mt] = R.G;
+      if (mt == 0) {
+        sMeta[0] = R.tok0;
+        sMeta[1] = R.len;
+      }
+    };
+    auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n + 1
+      const int64_t slot = (int64_t)row * N + n;
+      const int tok0 = cur.tok0, len = cur.len;
+      if (n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
+      unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
+      lds_barrier();  // B2
+      if (n + 1 < c1) nxt.W.store(sW, LDK, mt);
+      unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
+      lds_barrier();  // B3
+      if (n + 1 < c1) commit_rest(nxt);
+      if (FUSE && p.o_dtype == LNX_BF16)
+        unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + ((int64_t)row * p.geom.T + tok0) * p.dv + v0, p.dv, sO, LDO, len, mt);
+      lds_barrier();  // B1 of the next chunk
+    };
+    if (c0 < c1) {
+      fetch(ta, c0);
+      ta.W.store(sW, LDK, mt);
+      commit_rest(ta);
+    }
+    if (AHEAD == 2 && c0 + 1 < c1) fetch(tb, c0 + 1);
+    lds_barrier();  // B1 of the first chunk
+    if (AHEAD == 2) {
+      // chunk c0 is in LDS, so set a is free: it takes chunk c0 + 2 in the first step
+      for (int n = c0; n < c1; n += 2) {
+        step(ta, tb, n);
+        if (n + 1 < c1) step(tb, ta, n + 1);
+      }
+    } else {
+      for (int n = c0; n < c1; ++n) step(ta, ta, n);
+    }
+    return;
+  }
+
+  // ---------------- compute waves ----------------
   const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
   const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
   const int wi = wave >> 1, wj = wave & 1;  // this wave's tile of the [64 x BV] products
@@ -440,50 +535,10 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       for (int e = 0; e < 16; ++e)
         S[0][j][e] = s0[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
   }
-
-  // register prefetch of the next chunk's tiles
-  TileRegs<T, 64, DK> rW, rK;
-  TileRegs<T, 64, BV> rU;
-  TileRegs<T, 64, FUSE ? DK : 8> rQ;
-  TileRegs<T, 64, FUSE ? 64 : 8> rP;
-  float rG = 0.f;
-  int rTok0 = 0, rLen = 0;
-  auto fetch = [&](int n) {
-    const int64_t slot = (int64_t)row * N + n;
-    chunk_span(p.geom, n, rTok0, rLen);
-    const int64_t tbase = (int64_t)row * p.geom.T + rTok0;
-    rW.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
-    if (GATE == LNX_GATE_VECTOR) rK.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, tid);
-    else rK.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, rLen, tid);
-    rU.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    if (FUSE) {
-      if (GATE == LNX_GATE_VECTOR) rQ.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, tid);
-      else rQ.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, rLen, tid);
-      rP.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
-    }
-    if (GATE == LNX_GATE_SCALAR && tid < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + tid];
-    if (GATE == LNX_GATE_VECTOR && tid < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];  // G_last[c]
-  };
-
-  if (c0 < c1) fetch(c0);
+  // entering state -> LDS, transposed [dv][dk] (B operand of W S and Q S; the movers copy it to the workspace)
+  if (c0 < c1) frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
+  lds_barrier();  // B1 of the first chunk
   for (int n = c0; n < c1; ++n) {
-    const int64_t slot = (int64_t)row * N + n;
-    const int tok0 = rTok0, len = rLen;
-    rW.store(sW, LDK, tid);
-    rK.store(sK, LDK, tid);
-    rU.store(sU, LDU, tid);
-    if (FUSE) {
-      rQ.store(sQ, LDK, tid);
-      rP.store(sP, LDC, tid);
-    }
-    if (tid < 128) sG[tid] = rG;
-    // entering state -> LDS, transposed [dv][dk] (B operand of W S and Q S); the workspace copy
-    // leaves from there as whole rows, 16 bytes per lane
-    frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
-    lds_barrier();
-    if (n + 1 < c1) fetch(n + 1);
-    unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
-
     // D = U - W S  (one 32x32 tile per wave)
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
     {
@@ -491,7 +546,6 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       frag_zero(d);
       mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
       // D replaces U in place (all reads first: interleaved with the writes they would be serialised)
-      // and is written out from LDS below
       float u[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) u[e] = to_f32(sU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
@@ -506,11 +560,10 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
       }
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    lds_barrier();
-    unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, tid);
+    lds_barrier();  // B2
 
     if (FUSE) {
-      // o = scale e^G (Q S) + P D for this slab, staged in LDS in the output type
+      // o = scale e^G (Q S) + P D for this slab
       floatx16 o[1][1];
       frag_zero(o);
       mma_nt<T, 1, 1>(o, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
@@ -520,13 +573,14 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
           o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
       }
       mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
-      if (p.o_dtype == LNX_BF16)
-        frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);
-      else
+      if (p.o_dtype == LNX_BF16) {
+        frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
+      } else {
+        const int tok0 = sMeta[0], len = sMeta[1];
         frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + ((int64_t)row * p.geom.T + tok0 + 32 * wi) * p.dv + v0 + 32 * wj,
                                 p.dv, lane, len - 32 * wi);
+      }
     }
-
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
     if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
@@ -542,9 +596,9 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(FwdParams p) {
         for (int e = 0; e < 16; ++e) S[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
     }
     mma_x<T, 1, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
-    lds_barrier();
-    if (FUSE && p.o_dtype == LNX_BF16)
-      unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + ((int64_t)row * p.geom.T + tok0) * p.dv + v0, p.dv, sO, LDO, len, tid);
+    lds_barrier();  // B3
+    if (n + 1 < c1) frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
+    lds_barrier();  // B1 of the next chunk
   }
 
   float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0;
@@ -678,7 +732,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("chunk_prepare", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
   lnx_profile_mark("chunk_scan", st);
-  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / ScanSmem<T, DK>::BV)), dim3(256), b2, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / ScanSmem<T, DK>::BV)), dim3(512), b2, st, p);
   if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
     hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
