@@ -74,11 +74,20 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
-// bwd_scan
+// bwd_scan: the reverse sequential pass over the chunks of one (state, slab of dv).  Per chunk:
+//   dD = dD_loc + r_j (K dS)_j   (the complete gradient of D, back to the workspace),
+//   dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD,
+// with dS the gradient of the state leaving the chunk (stored transposed for bwd_dqk).
+// Same organisation as the forward scan: waves 0-3 compute on the tiles in LDS, waves 4-7 move
+// data (global loads two chunks ahead, tile writes as soon as a tile's reader is done, LDS ->
+// global copies of dS and dD), three barriers per chunk:
+//   B1  tiles of chunk n and dS^T are in LDS      compute: dD          movers: loads of chunk n-2, dS -> workspace
+//   B2  dD is in LDS (plain and negated-transposed)  compute: dS update   movers: K of chunk n-1 -> LDS, dD -> workspace
+//   B3  all reads of chunk n's tiles are done     compute: dS^T -> LDS  movers: remaining tiles of chunk n-1 -> LDS
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int BV = (DK == 128) ? 32 : 64;  // dv slab per workgroup
+  static constexpr int BV = (DK == 128 && sizeof(T) == 4) ? 32 : 64;  // dv slab per workgroup (LDS capacity)
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
@@ -87,10 +96,9 @@ template <typename T, int DK> struct BScanCfg {
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel(BwdParams p) {
+__global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   typedef BScanCfg<T, DK> L;
-  typedef typename Vec16<T>::V V16;
-  constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV, VN = Vec16<T>::N;
+  constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV;
   constexpr int CT = BV / 32;                      // column tiles of the slab
   constexpr int NT = (DK == 128) ? CT : 1;         // state tiles per wave (row tile = wave or wave & 1)
   static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
@@ -111,6 +119,92 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
   const int v0 = blockIdx.y * BV;
   int c0, c1;
   seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+
+  if (wave >= 4) {
+    // ---------------- movers ----------------
+    const int mt = tid - 256;
+    typedef TileRegs<T, 64, BV> Slab;
+    struct Tiles {
+      TileRegs<T, 64, DK> K, Q, W;
+      Slab dO, dD;
+      float os[Slab::IT];  // scale * e^{G_i} of the dO row each vector belongs to
+      float G;
+    };
+    constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;  // chunks fetched ahead (register sets in use)
+    Tiles ta, tb;
+    ta.G = tb.G = 0.f;
+    auto fetch = [&](Tiles& R, int n) {
+      const int64_t slot = (int64_t)row * N + n;
+      int tok0, len;
+      chunk_span(p.geom, n, tok0, len);
+      const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+      // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)
+      if (GATE == LNX_GATE_VECTOR) {
+        R.K.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        R.Q.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+      } else {
+        R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, len, mt);
+        R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, len, mt);
+      }
+      R.W.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+      R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, mt);
+      R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+#pragma unroll
+      for (int it = 0; it < Slab::IT; ++it) {
+        const int r = min((mt + 256 * it) / Slab::VPR, 63);
+        R.os[it] = (GATE == LNX_GATE_VECTOR) ? 1.f
+                   : (GATE == LNX_GATE_NONE) ? p.scale
+                                             : p.scale * __expf(wsp<float>(p, p.off.G)[slot * 64 + r]);
+      }
+      if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = wsp<float>(p, p.off.G)[slot * 64 + mt];
+      if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+    };
+    auto commit_rest = [&](const Tiles& R) {
+      R.Q.store(sQ, LDK, mt);
+      R.W.store(sW, LDK, mt);
+      R.dD.store(sdDl, LDU, mt);
+#pragma unroll
+      for (int it = 0; it < Slab::IT; ++it) {
+        const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
+        typename Vec16<T>::V o = R.dO.x[it];
+        if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}: (scale Q e^G)^T dO = Q^T (that)
+#pragma unroll
+          for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * R.os[it]);
+        }
+        if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
+      }
+      if (mt < 128) sG[mt] = R.G;
+    };
+    auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n - 1
+      const int64_t slot = (int64_t)row * N + n;
+      if (n - AHEAD >= c0) fetch(cur, n - AHEAD);  // chunk n's registers are free again
+      unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
+      lds_barrier();  // B2
+      if (n - 1 >= c0) nxt.K.store(sK, LDK, mt);
+      unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+      lds_barrier();  // B3
+      if (n - 1 >= c0) commit_rest(nxt);
+      lds_barrier();  // B1 of the next chunk
+    };
+    if (c0 < c1) {
+      fetch(ta, c1 - 1);
+      ta.K.store(sK, LDK, mt);
+      commit_rest(ta);
+    }
+    if (AHEAD == 2 && c1 - 2 >= c0) fetch(tb, c1 - 2);
+    lds_barrier();  // B1 of the first chunk
+    if (AHEAD == 2) {
+      for (int n = c1 - 1; n >= c0; n -= 2) {
+        step(ta, tb, n);
+        if (n - 1 >= c0) step(tb, ta, n - 1);
+      }
+    } else {
+      for (int n = c1 - 1; n >= c0; --n) step(ta, ta, n);
+    }
+    return;
+  }
+
+  // ---------------- compute waves ----------------
   const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
   const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
   // tile of the [64 x BV] token-by-value products owned by this wave (none for CT == 1, wave >= 2)
@@ -127,88 +221,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
       for (int e = 0; e < 16; ++e)
         dS[0][j][e] = src[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
   }
-
-  constexpr int NK = 64 * DK / VN / 256, NO = (BV * 64 / VN + 255) / 256;
-  V16 rK[NK], rQ[NK], rW[NK], rO[NO], rD[NO];
-  float rOs[NO];  // scale * e^{G_i} of the dO row each vector belongs to
-  float rG = 0.f;
-  auto fetch = [&](int n) {
-    const int64_t slot = (int64_t)row * N + n;
-    int tok0, len;
-    chunk_span(p.geom, n, tok0, len);
-    const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-    // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)
-    const T* Kg = (GATE == LNX_GATE_VECTOR) ? wsp<T>(p, p.off.Kr) + slot * 64 * DK
-                                            : reinterpret_cast<const T*>(p.k) + tbase * DK;
-    const T* Qg = (GATE == LNX_GATE_VECTOR) ? wsp<T>(p, p.off.Qg) + slot * 64 * DK
-                                            : reinterpret_cast<const T*>(p.q) + tbase * DK;
-    const T* Wg = wsp<T>(p, p.off.W) + slot * 64 * DK;
-    const int klen = (GATE == LNX_GATE_VECTOR) ? 64 : len;
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int idx = tid + 256 * i, r = idx / (DK / VN);
-      rK[i] = vec_zero<T>();
-      rQ[i] = vec_zero<T>();
-      if (r < klen) {
-        rK[i] = *reinterpret_cast<const V16*>(Kg + (int64_t)idx * VN);
-        rQ[i] = *reinterpret_cast<const V16*>(Qg + (int64_t)idx * VN);
-      }
-      rW[i] = *reinterpret_cast<const V16*>(Wg + (int64_t)idx * VN);
-    }
-    const T* Og = reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0;
-    const T* Dg = wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0;
-#pragma unroll
-    for (int i = 0; i < NO; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < BV * 64 / VN) {
-        const int r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-        rO[i] = vec_zero<T>();
-        if (r < len) rO[i] = *reinterpret_cast<const V16*>(Og + (int64_t)r * p.dv + c);
-        rD[i] = *reinterpret_cast<const V16*>(Dg + (int64_t)r * p.dv + c);
-        rOs[i] = (GATE == LNX_GATE_VECTOR) ? 1.f
-                 : (GATE == LNX_GATE_NONE) ? p.scale
-                                           : p.scale * __expf(wsp<float>(p, p.off.G)[slot * 64 + r]);
-      }
-    }
-    if (GATE == LNX_GATE_SCALAR && tid < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + tid];
-    if (GATE == LNX_GATE_VECTOR && tid < DK) rG = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + tid];
-  };
-  auto commit = [&]() {
-    if (tid < 128) sG[tid] = rG;
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int idx = tid + 256 * i, r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
-      *reinterpret_cast<V16*>(sK + r * LDK + c) = rK[i];
-      *reinterpret_cast<V16*>(sQ + r * LDK + c) = rQ[i];
-      *reinterpret_cast<V16*>(sW + r * LDK + c) = rW[i];
-    }
-#pragma unroll
-    for (int i = 0; i < NO; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < BV * 64 / VN) {
-        const int r = idx / (BV / VN), c = (idx % (BV / VN)) * VN;
-        V16 o = rO[i];
-        if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}: (scale Q e^G)^T dO = Q^T (that)
-#pragma unroll
-          for (int e = 0; e < VN; ++e) o[e] = from_f32<T>(to_f32(o[e]) * rOs[i]);
-        }
-        *reinterpret_cast<V16*>(sdO + r * LDU + c) = o;
-        *reinterpret_cast<V16*>(sdDl + r * LDU + c) = rD[i];
-      }
-    }
-  };
-
-  if (c0 < c1) fetch(c1 - 1);
+  // dS (gradient of the state leaving the chunk) -> LDS, transposed [dv][dk]; the movers copy it to the workspace
+  if (c0 < c1) frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
+  lds_barrier();  // B1 of the first chunk
   for (int n = c1 - 1; n >= c0; --n) {
-    const int64_t slot = (int64_t)row * N + n;
-    commit();
-    // dS (gradient of the state leaving chunk n) -> LDS, transposed [dv][dk]; the workspace copy
-    // (same layout) leaves from there as whole rows, 16 bytes per lane
-    frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
-    lds_barrier();
-    if (n > c0) fetch(n - 1);
-    unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, tid);
-
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
     // dD = dD_loc + r_j (K dS)_j
     if (has_tile) {
@@ -216,7 +232,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
       frag_zero(d);
       mma_nt<T, 1, 1>(d, sK + 32 * wi * LDK, LDK, sdST + 32 * wj * LDK, LDK, DK, lane);
       // the complete dD replaces the local part in place (all reads first: interleaved with the
-      // writes they would be serialised) and is written out from LDS below
+      // writes they would be serialised); the movers write it out
       float dl[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) dl[e] = to_f32(sdDl[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
@@ -232,8 +248,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
       }
       frag_store_t<T, 1, 1>(d, sdDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    lds_barrier();
-    unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, tid);
+    lds_barrier();  // B2
 
     // dS <- e^{G_last} dS + (scale Q e^G)^T dO - W^T dD   (token-contracted: rows of the tiles)
     if (GATE == LNX_GATE_SCALAR) {
@@ -251,7 +266,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_scan_kernel
     }
     mma_x<T, 1, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
     mma_x<T, 1, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
-    lds_barrier();
+    lds_barrier();  // B3
+    if (n > c0) frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
+    lds_barrier();  // B1 of the next chunk
   }
   if (p.ds0) {
     float* out = p.ds0 + (int64_t)sidx * DK * p.dv + v0;
@@ -843,7 +860,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("bwd_local", st);
   hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
   lnx_profile_mark("bwd_scan", st);
-  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(256), b1, st, p);
+  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(512), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("bwd_wy", st);
