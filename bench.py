@@ -33,10 +33,10 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
 TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 827333560, ("gdn_chunk", "chunk_scan"): 815944299,
-    ("gdn_chunk", "chunk_output"): 740377023, ("gdn_chunk", "bwd_local"): 337702140,
-    ("gdn_chunk", "bwd_scan"): 1084422711, ("gdn_chunk", "bwd_dqk"): 1617126440,
-    ("gdn_chunk", "bwd_wy"): 1394292784, ("decode", "decode_step"): 1083445231,
+    ("gdn_chunk", "chunk_prepare"): 865266704, ("gdn_chunk", "chunk_scan"): 1151563238,
+    ("gdn_chunk", "bwd_local"): 337689355, ("gdn_chunk", "bwd_scan"): 1084420419,
+    ("gdn_chunk", "bwd_dqk"): 1617062844, ("gdn_chunk", "bwd_wy"): 1485695358,
+    ("decode", "decode_step"): 1083425683,
 }
 
 
