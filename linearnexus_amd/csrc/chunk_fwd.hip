@@ -491,7 +491,6 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       const int64_t slot = (int64_t)row * N + n;
       const int tok0 = cur.tok0, len = cur.len;
       if (n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
-      unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
       lds_barrier();  // B2
       if (n + 1 < c1) nxt.W.store(sW, LDK, mt);
       unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
@@ -560,6 +559,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       }
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
+    // S_n -> workspace (the movers are busy issuing loads in this phase)
+    unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
     lds_barrier();  // B2
 
     if (FUSE) {
