@@ -159,6 +159,8 @@ def bench_chunk(args, torch, la, _lib, name):
     avg = {n: sum(v_) / len(v_) for n, v_ in per_kernel.items()}
     if "chunk_output" not in avg:  # 2-byte inputs: the scan kernel also forms the outputs
         fl["chunk_scan"] += fl.pop("chunk_output")
+    if "bwd_local" not in avg:     # ... and the backward scan the chunk-local part of dD
+        fl["bwd_scan"] += fl.pop("bwd_local")
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
     peak = PEAK_FP32_MFMA if variant == "delta32" else PEAK_BF16

@@ -91,14 +91,19 @@ template <typename T, int DK> struct BScanCfg {
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
-  // K, Q, W rows [token][dk];  dO, dD_loc slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk]
-  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST) + sizeof(float) * 128;
+  // 2-byte inputs: the chunk-local part dD_loc = P^T dO is formed here as well (P and the unscaled dO
+  // tile fit LDS), so bwd_local does not run
+  static constexpr bool FUSE_LOCAL = sizeof(T) == 2;
+  static constexpr int kP = FUSE_LOCAL ? 64 * LDC : 0, kRaw = FUSE_LOCAL ? kSlab : 0;
+  // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
+  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * 128;
 };
 
 template <typename T, int DK, int GATE>
 __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   typedef BScanCfg<T, DK> L;
   constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV;
+  constexpr bool FUSE = L::FUSE_LOCAL;
   constexpr int CT = BV / 32;                      // column tiles of the slab
   constexpr int NT = (DK == 128) ? CT : 1;         // state tiles per wave (row tile = wave or wave & 1)
   static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
@@ -110,7 +115,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   T* sdDl = sdO + L::kSlab;
   T* sdDT = sdDl + L::kSlab;
   T* sdST = sdDT + L::kdDT;
-  float* sG = reinterpret_cast<float*>(sdST + L::kdST);
+  T* sP = sdST + L::kdST;   // fused local part only: P [i][j] and the unscaled dO slab
+  T* sdOr = sP + L::kP;
+  float* sG = reinterpret_cast<float*>(sdOr + L::kRaw);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
@@ -126,7 +133,8 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     typedef TileRegs<T, 64, BV> Slab;
     struct Tiles {
       TileRegs<T, 64, DK> K, Q, W;
-      Slab dO, dD;
+      Slab dO, dD;                       // dD: the chunk-local part from bwd_local (not fused only)
+      TileRegs<T, 64, FUSE ? 64 : 8> P;  // fused only
       float os[Slab::IT];  // scale * e^{G_i} of the dO row each vector belongs to
       float G;
     };
@@ -148,7 +156,8 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       }
       R.W.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
       R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, mt);
-      R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+      if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
 #pragma unroll
       for (int it = 0; it < Slab::IT; ++it) {
         const int r = min((mt + 256 * it) / Slab::VPR, 63);
@@ -162,7 +171,12 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     auto commit_rest = [&](const Tiles& R) {
       R.Q.store(sQ, LDK, mt);
       R.W.store(sW, LDK, mt);
-      R.dD.store(sdDl, LDU, mt);
+      if (FUSE) {
+        R.P.store(sP, LDC, mt);
+        R.dO.store(sdOr, LDU, mt);
+      } else {
+        R.dD.store(sdDl, LDU, mt);
+      }
 #pragma unroll
       for (int it = 0; it < Slab::IT; ++it) {
         const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
@@ -178,6 +192,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n - 1
       const int64_t slot = (int64_t)row * N + n;
       if (n - AHEAD >= c0) fetch(cur, n - AHEAD);  // chunk n's registers are free again
+      if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       lds_barrier();  // B2
       if (n - 1 >= c0) nxt.K.store(sK, LDK, mt);
@@ -234,8 +249,16 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       // the complete dD replaces the local part in place (all reads first: interleaved with the
       // writes they would be serialised); the movers write it out
       float dl[16];
+      if (FUSE) {  // dD_loc[j][v] = sum_i P[i][j] dO[i][v]: both operands contract along the rows of their tiles
+        floatx16 l[1][1];
+        frag_zero(l);
+        mma_x<T, 1, 1, true, true>(l, sP + 32 * wi, LDC, sdOr + 32 * wj, LDU, 64, lane);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) dl[e] = to_f32(sdDl[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
+        for (int e = 0; e < 16; ++e) dl[e] = l[0][0][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dl[e] = to_f32(sdDl[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f)) : 1.f;
@@ -857,8 +880,10 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b3)) != hipSuccess)
     return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  lnx_profile_mark("bwd_local", st);
-  hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
+  if (!BScanCfg<T, DK>::FUSE_LOCAL) {  // otherwise bwd_scan forms the chunk-local part itself
+    lnx_profile_mark("bwd_local", st);
+    hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
+  }
   lnx_profile_mark("bwd_scan", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(512), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
