@@ -179,6 +179,10 @@ def bench_chunk(args, torch, la, _lib, name):
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": TRAFFIC.get((name, dom))},
     }
+    tr = TRAFFIC.get((name, dom))
+    if tr:  # the same kernel against the HBM roof, from its measured traffic
+        out["roofline_hbm_measured"] = {"kernel": dom, "achieved": tr / (avg[dom] * 1e-3) / 1e9, "peak": PEAK_HBM,
+                                        "unit": "GB/s", "frac": tr / (avg[dom] * 1e-3) / 1e9 / PEAK_HBM}
     return out, (B, H, T, d)
 
 

@@ -180,28 +180,32 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
 
 // ---------------------------------------------------------------------------------------
 // kda_prepare: chunk_prepare for a per-channel (vector) gate.  The pairwise products carry the
-// decay inside the dk sum, X_ij = sum_c k_i[c] k_j[c] exp(G_i[c] - G_j[c]); they are evaluated
-// on the VALU with exponents of non-positive numbers only (i >= j), as the reference does for
-// its diagonal blocks (kda.py:483-502).  Everything after A is the same MFMA pipeline, with the
-// decays folded element-wise into the staged operands.
+// decay inside the dk sum, X_ij = sum_c k_i[c] k_j[c] exp(G_i[c] - G_j[c]).  The channels are
+// taken in 64-wide halves (K, Q and the fp32 gate tile of one half fit LDS twice per CU): per half
+// the cumulative gate, K e^{G_last - G} and scale Q e^G go to the workspace and the half's share of
+// the pair products is accumulated -- 16x16 blocks below the diagonal on the fp32 MFMA with the
+// decay factored through the first row of the row block (kda.py:504-523), diagonal blocks on the
+// VALU with exponents of non-positive numbers only (kda.py:483-502).  After the inverse, W and U
+// are formed by one loop over 64-column slabs of [K | V] with register prefetch, results leaving
+// through LDS with 16-byte stores.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK> struct KdaPrepSmem {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int LDK = DK + PAD, LDC = LNX_C + PAD, LDF = DK + 4;
-  static constexpr int kK = 64 * LDK;                                     // sK, later the T-typed copy of Tm
-  static constexpr int kQ = (64 * LDK > DK * LDC) ? 64 * LDK : DK * LDC;  // sQ, later transposed staging
-  static constexpr size_t bytes =
-      sizeof(T) * (kK + kQ) + sizeof(float) * (64 * LDF + 2 * 64 * LNX_LDA + 32 * 36 + 64);
+  static constexpr int LDC = LNX_C + PAD, LDF = 64 + 4;
+  static constexpr int kTile = 64 * LDC;
+  // K half (later Tm), Q half (later Tm diag(beta)); gate half (later the staged slab); A (later the
+  // output staging); the P accumulator / inverse; inverse scratch; beta
+  static constexpr size_t bytes = sizeof(T) * 2 * kTile + sizeof(float) * (64 * LDF + 2 * 64 * LNX_LDA + 32 * 36 + 64);
 };
 
 template <typename T, int DK>
-__global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_kernel(FwdParams p) {
   typedef KdaPrepSmem<T, DK> L;
-  constexpr int LDK = L::LDK, LDC = L::LDC, LDF = L::LDF;
+  constexpr int LDC = L::LDC, LDF = L::LDF, NH = DK / 64;
   extern __shared__ __align__(16) char smem[];
   T* sK = reinterpret_cast<T*>(smem);
-  T* sQ = sK + L::kK;
-  float* sG = reinterpret_cast<float*>(sQ + L::kQ);  // [64][LDF] cumulative gate
+  T* sQ = sK + L::kTile;
+  float* sG = reinterpret_cast<float*>(sQ + L::kTile);  // [64][LDF] cumulative gate of the half
   float* sA = sG + 64 * LDF;
   float* sT = sA + 64 * LNX_LDA;
   float* sX = sT + 64 * LNX_LDA;
@@ -218,111 +222,136 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
-
-  stage_tile<T, 64, DK>(sK, LDK, kg, DK, len, tid);
-  stage_tile<T, 64, DK>(sQ, LDK, qg, DK, len, tid);
-  for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
-    const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-    floatx4 x = {0.f, 0.f, 0.f, 0.f};
-    if (r < len) x = load4(p.g + (tbase + r) * DK + c);
-    store4(sG + r * LDF + c, x);
-  }
-  if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
-  lds_barrier();
-  if (tid < DK) {
-    float acc = 0.f;
-    for (int r = 0; r < 64; ++r) {
-      acc += sG[r * LDF + tid];
-      sG[r * LDF + tid] = acc;
-    }
-  }
-  lds_barrier();
-  {
-    float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
-    T* Krg = ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK;
-    T* Qgg = ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK;
-    for (int idx = tid; idx < 64 * DK / 4; idx += 256) {
-      const int r = idx / (DK / 4), c = (idx % (DK / 4)) * 4;
-      const floatx4 gr = load4(sG + r * LDF + c), gl = load4(sG + 63 * LDF + c), kk = load4(sK + r * LDK + c);
-      store4(Gg + r * DK + c, gr);
-      const floatx4 qq = load4(sQ + r * LDK + c);
-      floatx4 kr, qgv;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        kr[e] = kk[e] * __expf(fminf(gl[e] - gr[e], 0.f));
-        qgv[e] = qq[e] * p.scale * __expf(gr[e]);
-      }
-      store4(Krg + r * DK + c, kr);
-      store4(Qgg + r * DK + c, qgv);
-    }
-  }
-  // pairwise products X_ij = <k_i, k_j>_E (i > j) and <q_i, k_j>_E (i >= j) with the decay inside
-  // the channel sum, formed in sA and sT.
+  float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
   const int l16 = lane & 15, kq = lane >> 4;
-  {
-    // 16x16 blocks below the diagonal on the fp32 MFMA: E_ij = exp(G_i - G_ref) exp(G_ref - G_j) with
-    // G_ref the first row of the row block, both factors <= 1 (kda.py:504-523).  Twelve tasks
-    // (six blocks, two products), three per wave.
-    for (int t = wave; t < 12; t += 4) {
+
+  // ---- phase A: per 64-channel half ----
+  TileRegs<T, 64, 64> rK, rQ;
+  TileRegs<float, 64, 64> rG;
+  auto fetch_half = [&](int h) {
+    rK.load(kg + 64 * h, DK, len, tid);
+    rQ.load(qg + 64 * h, DK, len, tid);
+    rG.load(p.g + tbase * DK + 64 * h, DK, len, tid);
+  };
+  fetch_half(0);
+  if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+  floatx4 acc[3];  // this wave's three below-diagonal tasks (block, product), summed over the halves
+#pragma unroll
+  for (int u = 0; u < 3; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) {  // the diagonal blocks accumulate here over the halves
+    sA[idx] = 0.f;
+    sT[idx] = 0.f;
+  }
+
+#pragma unroll 1
+  for (int h = 0; h < NH; ++h) {
+    lds_barrier();  // the previous half's tiles are dead
+    rK.store(sK, LDC, tid);
+    rQ.store(sQ, LDC, tid);
+    rG.store(sG, LDF, tid);
+    lds_barrier();
+    if (h + 1 < NH) fetch_half(h + 1);
+    {  // cumulative gate along the tokens, per channel: 16-row segments in parallel, then their offsets
+      const int c = tid & 63, seg = tid >> 6;
+      float run = 0.f;
+#pragma unroll
+      for (int r = 16 * seg; r < 16 * seg + 16; ++r) {
+        run += sG[r * LDF + c];
+        sG[r * LDF + c] = run;
+      }
+      lds_barrier();
+      float off = 0.f;
+      for (int s_ = 0; s_ < seg; ++s_) off += sG[(16 * s_ + 15) * LDF + c];
+      lds_barrier();
+#pragma unroll
+      for (int r = 16 * seg; r < 16 * seg + 16; ++r) sG[r * LDF + c] += off;
+    }
+    lds_barrier();
+    {  // G, K e^{G_last - G}, scale Q e^G of this half -> workspace
+      T* Krg = ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK + 64 * h;
+      T* Qgg = ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK + 64 * h;
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+        const floatx4 gr = load4(sG + r * LDF + c), gl = load4(sG + 63 * LDF + c);
+        const floatx4 kk = load4(sK + r * LDC + c), qq = load4(sQ + r * LDC + c);
+        floatx4 kr, qgv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          kr[e] = kk[e] * __expf(fminf(gl[e] - gr[e], 0.f));
+          qgv[e] = qq[e] * p.scale * __expf(gr[e]);
+        }
+        store4(Gg + r * DK + 64 * h + c, gr);
+        store4(Krg + r * DK + c, kr);
+        store4(Qgg + r * DK + c, qgv);
+      }
+    }
+    // blocks below the diagonal: six blocks x two products = twelve tasks, three per wave
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      const int t = wave + 4 * u;
       const int pr = t % 6, I = (pr < 1) ? 1 : (pr < 3) ? 2 : 3, J = pr - ((I == 1) ? 0 : (I == 2) ? 1 : 3);
       const T* sRow = (t < 6) ? sK : sQ;
-      float* dst = (t < 6) ? sA : sT;
       const int i = 16 * I + l16, j = 16 * J + l16;
-      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
-      for (int ks = 0; ks < DK / 4; ++ks) {
+      for (int ks = 0; ks < 16; ++ks) {
         const int c = 4 * ks + kq;
         const float gref = sG[16 * I * LDF + c];
         const float fa = __expf(fminf(sG[i * LDF + c] - gref, 0.f));
         const float fb = __expf(fminf(gref - sG[j * LDF + c], 0.f));
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sRow[i * LDK + c]) * fa, to_f32(sK[j * LDK + c]) * fb, acc, 0, 0, 0);
+        acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sRow[i * LDC + c]) * fa, to_f32(sK[j * LDC + c]) * fb, acc[u], 0, 0, 0);
       }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) dst[(16 * I + 4 * kq + e) * LNX_LDA + j] = acc[e];
     }
-  }
-  {
-    // 16x16 blocks on the diagonal on the VALU, exponents of non-positive numbers only
-    // (kda.py:483-502): wave = block; lane = (pair of rows rp and 15 - rp, eighth of the channels).
-    // The two rows together have 17 columns j <= i, walked in one loop of 17 steps.
-    constexpr int CE = DK / 8;
-    const int rp = lane & 7, ce = lane >> 3, r0 = 16 * wave;
+    {  // diagonal blocks: wave = block; lane = (pair of rows rp and 15 - rp, eighth of the half's channels);
+       // the two rows together have 17 columns j <= i
+      const int rp = lane & 7, ce = lane >> 3, r0 = 16 * wave;
 #pragma unroll 1
-    for (int t = 0; t < 17; ++t) {
-      const bool first = t <= rp;
-      const int i = r0 + (first ? rp : 15 - rp), j = r0 + (first ? t : t - rp - 1);
-      float x = 0.f, pp = 0.f;
+      for (int t = 0; t < 17; ++t) {
+        const bool first = t <= rp;
+        const int i = r0 + (first ? rp : 15 - rp), j = r0 + (first ? t : t - rp - 1);
+        float x = 0.f, pp = 0.f;
 #pragma unroll
-      for (int c = ce * CE; c < (ce + 1) * CE; c += 4) {
-        const floatx4 ki = load4(sK + i * LDK + c), qi = load4(sQ + i * LDK + c), gi = load4(sG + i * LDF + c);
-        const floatx4 kj = load4(sK + j * LDK + c), gj = load4(sG + j * LDF + c);
+        for (int c = 8 * ce; c < 8 * ce + 8; c += 4) {
+          const floatx4 ki = load4(sK + i * LDC + c), qi = load4(sQ + i * LDC + c), gi = load4(sG + i * LDF + c);
+          const floatx4 kj = load4(sK + j * LDC + c), gj = load4(sG + j * LDF + c);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float ee = __expf(fminf(gi[e] - gj[e], 0.f)) * kj[e];
-          x += ki[e] * ee;
-          pp += qi[e] * ee;
+          for (int e = 0; e < 4; ++e) {
+            const float ee = __expf(fminf(gi[e] - gj[e], 0.f)) * kj[e];
+            x += ki[e] * ee;
+            pp += qi[e] * ee;
+          }
+        }
+#pragma unroll
+        for (int m = 8; m < 64; m <<= 1) {
+          x += __shfl_xor(x, m, LNX_WAVE);
+          pp += __shfl_xor(pp, m, LNX_WAVE);
+        }
+        if (ce == 0) {  // the same lane owns (i, j) in every half
+          sA[i * LNX_LDA + j] += x;
+          sT[i * LNX_LDA + j] += pp;
         }
       }
-#pragma unroll
-      for (int m = 8; m < 64; m <<= 1) {
-        x += __shfl_xor(x, m, LNX_WAVE);
-        pp += __shfl_xor(pp, m, LNX_WAVE);
-      }
-      if (ce == 0) {
-        sA[i * LNX_LDA + j] = x;
-        sT[i * LNX_LDA + j] = pp;
-      }
     }
+  }
+  // ---- phase B: assemble X and <q, k>_E in sA / sT, write X and P, A = beta X, inverse ----
+#pragma unroll
+  for (int u = 0; u < 3; ++u) {
+    const int t = wave + 4 * u;
+    const int pr = t % 6, I = (pr < 1) ? 1 : (pr < 3) ? 2 : 3, J = pr - ((I == 1) ? 0 : (I == 2) ? 1 : 3);
+    float* dst = (t < 6) ? sA : sT;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[(16 * I + 4 * kq + e) * LNX_LDA + 16 * J + l16] = acc[u][e];
   }
   lds_barrier();
   {
     T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
     T* Xg = ws_ptr<T>(p, p.off.X) + slot * 64 * 64;
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int i = idx >> 4, j0 = (idx & 15) * 4;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = tid + 256 * it, i = idx >> 4, j0 = (idx & 15) * 4;
       floatx4 x = load4(sA + i * LNX_LDA + j0), pp = load4(sT + i * LNX_LDA + j0);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < 4; ++e) {  // entries above the diagonal of the diagonal blocks were never written
         x[e] = (j0 + e < i) ? x[e] : 0.f;
         pp[e] = (j0 + e <= i) ? p.scale * pp[e] : 0.f;
       }
@@ -334,48 +363,70 @@ __global__ __launch_bounds__(256) void kda_prepare_kernel(FwdParams p) {
   lds_barrier();
   tri_inverse_64(sA, sT, sX, tid);
 
-  T* sTm = sK;                         // T-typed copy of Tm (bf16); fp32 reads sT in place
-  T* sTu = reinterpret_cast<T*>(sA);   // Tm * diag(beta)
+  // ---- phase C: Tm^T to the workspace; Tm and Tm diag(beta) as MFMA operands ----
+  T* sTm = sK;
+  T* sTu = sQ;
   {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
     for (int idx = tid; idx < 64 * 64; idx += 256) {
       const int r = idx >> 6, c = idx & 63;
       TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
       const float t = sT[r * LNX_LDA + c];
+      sTm[r * LDC + c] = from_f32<T>(t);
       sTu[r * LDC + c] = from_f32<T>(t * sBeta[c]);
-      if (sizeof(T) == 2) sTm[r * LDC + c] = from_f32<T>(t);
     }
   }
-  const T* tm_op = (sizeof(T) == 4) ? reinterpret_cast<const T*>(sT) : sTm;
-  lds_barrier();
-  // W = Tm (beta e^G K): transposed, scaled K through the sQ region
-  T* sKT = sQ;
-  stage_tile_t<T, 64, DK>(sKT, LDC, kg, DK, len, tid, [&](int r, int c) { return sBeta[r] * __expf(sG[r * LDF + c]); });
-  lds_barrier();
+  // ---- phase D: W = Tm (beta e^G K), U = Tu V, one 64-column slab at a time ----
+  T* sIn = reinterpret_cast<T*>(sG);    // staged slab [token][col]
+  T* sOut = reinterpret_cast<T*>(sA);   // result slab on its way to the workspace
   const int wi = wave >> 1, wj = wave & 1;
-  {
-    T* Wg = ws_ptr<T>(p, p.off.W) + slot * 64 * DK;
-    for (int c0 = 0; c0 < DK; c0 += 64) {
-      floatx16 acc[1][1];
-      frag_zero(acc);
-      mma_nt<T, 1, 1>(acc, tm_op + 32 * wi * LDC, LDC, sKT + (c0 + 32 * wj) * LDC, LDC, 64, lane);
-      frag_store<T, 1, 1>(acc, Wg + 32 * wi * DK + c0 + 32 * wj, DK, lane);
+  const int nslab = NH + p.dv / 64;
+  typedef TileRegs<T, 64, 64> Slab;
+  constexpr int VN = Slab::N;
+  Slab rIn;
+  floatx4 rGs[Slab::IT][VN / 4];  // K slabs: the gate values of exactly the elements this thread holds
+  auto fetch_slab = [&](int s_) {
+    if (s_ < NH) {
+      rIn.load(kg + 64 * s_, DK, len, tid);
+#pragma unroll
+      for (int it = 0; it < Slab::IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * VN;
+#pragma unroll
+        for (int j = 0; j < VN / 4; ++j) rGs[it][j] = load4(Gg + r * DK + 64 * s_ + c + 4 * j);
+      }
+    } else {
+      rIn.load(vg + 64 * (s_ - NH), p.dv, len, tid);
     }
-  }
-  lds_barrier();
-  // U = Tu V
-  {
-    T* sVT = sQ;
-    T* Ug = ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv;
-    for (int c0 = 0; c0 < p.dv; c0 += 64) {
-      lds_barrier();
-      stage_tile_t<T, 64, 64>(sVT, LDC, vg + c0, p.dv, len, tid);
-      lds_barrier();
-      floatx16 acc[1][1];
-      frag_zero(acc);
-      mma_nt<T, 1, 1>(acc, sTu + 32 * wi * LDC, LDC, sVT + 32 * wj * LDC, LDC, 64, lane);
-      frag_store<T, 1, 1>(acc, Ug + 32 * wi * p.dv + c0 + 32 * wj, p.dv, lane);
+  };
+  __syncthreads();  // G is read back from the workspace by other threads than wrote it: global memory must be ordered too
+  fetch_slab(0);
+#pragma unroll 1
+  for (int s_ = 0; s_ < nslab; ++s_) {
+    const bool is_k = s_ < NH;
+    lds_barrier();  // the previous slab's tiles (first pass: the inverse, the gate tile) are dead
+    if (is_k) {     // K slab scaled by beta_t e^{G_t[c]} on its way into LDS
+#pragma unroll
+      for (int it = 0; it < Slab::IT; ++it) {
+        const int idx = tid + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * VN;
+        typename Vec16<T>::V x = rIn.x[it];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * sBeta[r] * __expf(rGs[it][e / 4][e % 4]));
+        *reinterpret_cast<typename Vec16<T>::V*>(sIn + r * LDC + c) = x;
+      }
+    } else {
+      rIn.store(sIn, LDC, tid);
     }
+    lds_barrier();
+    if (s_ + 1 < nslab) fetch_slab(s_ + 1);
+    floatx16 o[1][1];
+    frag_zero(o);
+    mma_x<T, 1, 1, false, true>(o, (is_k ? sTm : sTu) + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
+    frag_store<T, 1, 1>(o, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
+    lds_barrier();
+    if (is_k)
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + 64 * s_, DK, sOut, LDC, 64, tid);
+    else
+      unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + 64 * (s_ - NH), p.dv, sOut, LDC, 64, tid);
   }
 }
 

@@ -1,6 +1,6 @@
 """Benchmark-shaped parity checks on the GPU.
 
-The fp64 oracle finishes in seconds only on slices, so at the full BASELINE shapes the checks
+The fp64 oracle finishes in seconds only on slices, so at the full benchmark shapes the checks
 are (a) the oracle on a slice of the (batch, head) rows of the very same launch and
 (b) size-independent properties: MFMA chunk path == fp32 token-by-token kernel, the adjoint
 identity <dO, o(v)> = <dv, v>, and var-len == per-sequence launches."""
