@@ -161,8 +161,6 @@ def bench_chunk(args, torch, la, _lib, name):
         fl["chunk_scan"] += fl.pop("chunk_output")
     if "bwd_local" not in avg:     # ... and the backward scan the chunk-local part of dD
         fl["bwd_scan"] += fl.pop("bwd_local")
-    if "bwd_chunk" in avg:         # no gate / scalar gate: one kernel for the chunk-local gradients
-        fl["bwd_chunk"] = fl.pop("bwd_dqk") + fl.pop("bwd_wy")
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
     peak = PEAK_FP32_MFMA if variant == "delta32" else PEAK_BF16

@@ -868,312 +868,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 }
 
 
-// ---------------------------------------------------------------------------------------
-// bwd_chunk (no gate / scalar gate): everything of the backward pass that is local to a chunk once
-// the reverse scan has left dD and dS_n in the workspace -- the work of bwd_dqk and bwd_wy2 in one
-// kernel, so that dW, the partial dk and the second reads of dD, D and K never touch memory.
-// One workgroup per chunk.
-//   phase 1, loop over 32-column slabs of dv (next slab prefetched into registers):
-//     dP += dO D^T,  dQg += dO S_n,  dW -= dD S_n,  dKr += D dS_n^T,  <dS_n, S_n>;
-//     dB_u = Tm^T dD (slab),  dv = beta dB_u,  dbeta += <dB_u, v>,  dM += dB_u U^T
-//   phase 2, loop over 64-channel halves of dk:
-//     dB_w = Tm^T dW,  dM += dB_w W^T,  X += K K^T,  <dB_w, k>;
-//     dq = scale e^G dQg + dPe K,  column part of dk = e^{G_last - G} dKr + dPe^T Q,  gate terms
-//   phase 3: dA = -tril(dM) E,  Y = beta dA;  dk = column part + beta e^G dB_w + (Y + Y^T) K;  dbeta, dg
-// ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct FusedCfg {
-  static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int SV = 32;  // dv slab of phase 1
-  static constexpr int LDC = LNX_C + PAD, LDS_ = SV + PAD, LDK = DK + PAD, NH = DK / 64;
-  static constexpr int kTile = 64 * LDC, kSlab = 64 * LDS_, kState = SV * LDK;
-  // phase 1: Tm^T | dO D dD U V slabs | dB_u slab | S_n and dS_n slabs
-  static constexpr int p1 = kTile + 6 * kSlab + 2 * kState;
-  // phase 2/3: Tm^T | dPe | K halves | Q half | dW half (then staging) | W half (then Y) | dB_w
-  static constexpr int p2 = kTile * (6 + NH);
-  static constexpr size_t bytes = sizeof(T) * (p1 > p2 ? p1 : p2) + sizeof(float) * 64 * 8;
-};
-
-template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void bwd_chunk_kernel(BwdParams p) {
-  static_assert(GATE != LNX_GATE_VECTOR, "the per-channel gate keeps bwd_dqk / bwd_wy2");
-  typedef FusedCfg<T, DK> L;
-  constexpr int LDC = L::LDC, LDS_ = L::LDS_, LDK = L::LDK, SV = L::SV, NH = L::NH;
-  extern __shared__ __align__(16) char smem[];
-  float* sG = reinterpret_cast<float*>(smem);
-  float* sBeta = sG + 64;
-  float* sdB = sBeta + 64;   // dbeta: <dB_u, v>
-  float* sdGk = sdB + 64;    // <dB_w, k> (before the factor e^G)
-  float* sRow = sdGk + 64;   // sum_j dA_ij E_ij X_ij
-  float* sCol = sRow + 64;   // sum_i beta_i dA_ij E_ij X_ij
-  float* sdG = sCol + 64;    // <q, dq> - <k, column part of dk>
-  float* sMisc = sdG + 64;   // [0] = sum_j r_j <dKr_j, k_j>, [1] = <dS_n, S_n>
-  T* sTmT = reinterpret_cast<T*>(sMisc + 64);
-  // phase 1
-  T* sdO = sTmT + L::kTile;
-  T* sD = sdO + L::kSlab;
-  T* sdD = sD + L::kSlab;
-  T* sU = sdD + L::kSlab;
-  T* sV = sU + L::kSlab;
-  T* sdBu = sV + L::kSlab;
-  T* sSn = sdBu + L::kSlab;   // [v][c]
-  T* sdSn = sSn + L::kState;  // [v][c]
-  // phase 2 / 3
-  T* sPe = sTmT + L::kTile;
-  T* sKh = sPe + L::kTile;    // NH tiles
-  T* sQh = sKh + NH * L::kTile;
-  T* sdWh = sQh + L::kTile;   // dW half, then staging of dq / dk
-  T* sWh = sdWh + L::kTile;   // W half, then Y
-  T* sdBw = sWh + L::kTile;
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int N = p.geom.N;
-  const int64_t slot = blockIdx.x;
-  const int row = (int)(slot / N), n = (int)(slot % N);
-  int tok0, len;
-  chunk_span(p.geom, n, tok0, len);
-  if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
-  const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
-  const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
-  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
-  const int wi = wave >> 1, wj = wave & 1;
-
-  if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
-    sdB[tid] = 0.f;
-    sdGk[tid] = 0.f;
-    sRow[tid] = 0.f;
-    sCol[tid] = 0.f;
-    sdG[tid] = 0.f;
-    sMisc[tid] = 0.f;
-  }
-  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
-
-  // ---------------- phase 1 ----------------
-  TileRegs<T, 64, SV> rdO, rD, rdD, rU, rV;
-  TileRegs<T, SV, DK> rSn, rdSn;
-  auto fetch1 = [&](int v0) {
-    rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
-    rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    rU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-    rV.load(vg + v0, p.dv, len, tid);
-    rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
-    rdSn.load(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
-  };
-  floatx16 aP[1][1], aM[1][1], aQ[NH][1][1], aW[NH][1][1], aK[NH][1][1];
-  frag_zero(aP);
-  frag_zero(aM);
-#pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    frag_zero(aQ[h]);
-    frag_zero(aW[h]);
-    frag_zero(aK[h]);
-  }
-  float ss = 0.f;
-  fetch1(0);
-#pragma unroll 1
-  for (int v0 = 0; v0 < p.dv; v0 += SV) {
-    lds_barrier();  // Tm^T staged / the previous slab's readers are done
-    rdO.store(sdO, LDS_, tid);
-    rD.store(sD, LDS_, tid);
-    rdD.store(sdD, LDS_, tid);
-    rU.store(sU, LDS_, tid);
-    rV.store(sV, LDS_, tid);
-    rSn.store(sSn, LDK, tid);
-    rdSn.store(sdSn, LDK, tid);
-    lds_barrier();
-    if (v0 + SV < p.dv) fetch1(v0 + SV);
-    if (wj == 0) {  // dB_u slab = Tm^T dD: two 32x32 tiles, waves 0 and 2
-      floatx16 b[1][1];
-      frag_zero(b);
-      mma_x<T, 1, 1, false, true>(b, sTmT + 32 * wi * LDC, LDC, sdD, LDS_, 64, lane);
-      frag_store<T, 1, 1>(b, sdBu + 32 * wi * LDS_, LDS_, lane);
-      float v[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) v[e] = b[0][0][e] * to_f32(sV[(32 * wi + frag_row(e, lane)) * LDS_ + frag_col(lane)]);
-      rows_reduce_add<1>(v, 32 * wi, lane, sdB);
-    }
-    mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDS_, LDS_, sD + 32 * wj * LDS_, LDS_, SV, lane);
-#pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      mma_x<T, 1, 1, false, true>(aQ[h], sdO + 32 * wi * LDS_, LDS_, sSn + 64 * h + 32 * wj, LDK, SV, lane);
-      mma_x<T, 1, 1, false, true>(aW[h], sdD + 32 * wi * LDS_, LDS_, sSn + 64 * h + 32 * wj, LDK, SV, lane);
-      mma_x<T, 1, 1, false, true>(aK[h], sD + 32 * wi * LDS_, LDS_, sdSn + 64 * h + 32 * wj, LDK, SV, lane);
-    }
-    if (GATE != LNX_GATE_NONE) {  // <dS_n, S_n>: thread = (state column c = tid % DK ..., quarter of the slab rows)
-      for (int idx = tid; idx < DK * 4; idx += 256) {
-        const int c = idx >> 2, q4 = (idx & 3) * (SV / 4);
-        float t = 0.f;
-#pragma unroll
-        for (int e = 0; e < SV / 4; ++e) t += to_f32(sSn[(q4 + e) * LDK + c]) * to_f32(sdSn[(q4 + e) * LDK + c]);
-        ss += t;
-      }
-    }
-    lds_barrier();  // dB_u slab complete
-    mma_nt<T, 1, 1>(aM, sdBu + 32 * wi * LDS_, LDS_, sU + 32 * wj * LDS_, LDS_, SV, lane);
-    {  // dv = beta dB_u, 16-byte stores
-      constexpr int VN = Vec16<T>::N, VPR = SV / VN;
-      T* dvg = reinterpret_cast<T*>(p.dv_out) + tbase * p.dv + v0;
-      for (int idx = tid; idx < 64 * VPR; idx += 256) {
-        const int r = idx / VPR, c = (idx % VPR) * VN;
-        if (r < len) {
-          typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBu + r * LDS_ + c);
-#pragma unroll
-          for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * sBeta[r]);
-          *reinterpret_cast<typename Vec16<T>::V*>(dvg + (int64_t)r * p.dv + c) = x;
-        }
-      }
-    }
-  }
-  if (GATE == LNX_GATE_SCALAR) {
-    ss = wave_sum(ss);
-    if (lane == 0) atomicAdd(&sMisc[1], ss);
-  }
-
-  // ---------------- phase 2 ----------------
-  TileRegs<T, 64, 64> rK[NH], rQ, rW;
-#pragma unroll
-  for (int h = 0; h < NH; ++h) rK[h].load(kg + 64 * h, DK, len, tid);
-  rQ.load(qg, DK, len, tid);
-  rW.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, tid);
-  lds_barrier();  // phase-1 tiles dead
-  {
-    floatx16 pe[1][1];
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      pe[0][0][e] = (i >= j) ? p.scale * dec * aP[0][0][e] : 0.f;
-    }
-    frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
-  }
-#pragma unroll
-  for (int h = 0; h < NH; ++h) rK[h].store(sKh + h * L::kTile, LDC, tid);
-  const float gl = sG[63];
-  floatx16 aBw[NH][1][1], aX[1][1];
-  frag_zero(aX);
-  float tot = 0.f;
-#pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    const T* sK_ = sKh + h * L::kTile;
-    if (h > 0) lds_barrier();  // the previous half's tiles are dead
-    rQ.store(sQh, LDC, tid);
-    rW.store(sWh, LDC, tid);
-    {
-      floatx16 nw[1][1];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) nw[0][0][e] = -aW[h][0][0][e];
-      frag_store<T, 1, 1>(nw, sdWh + 32 * wi * LDC + 32 * wj, LDC, lane);
-    }
-    lds_barrier();
-    if (h + 1 < NH) {
-      rQ.load(qg + 64 * (h + 1), DK, len, tid);
-      rW.load(wsp<T>(p, p.off.W) + slot * 64 * DK + 64 * (h + 1), DK, 64, tid);
-    }
-    // dB_w = Tm^T dW (this half's columns)
-    frag_zero(aBw[h]);
-    mma_x<T, 1, 1, false, true>(aBw[h], sTmT + 32 * wi * LDC, LDC, sdWh + 32 * wj, LDC, 64, lane);
-    frag_store<T, 1, 1>(aBw[h], sdBw + 32 * wi * LDC + 32 * wj, LDC, lane);
-    {
-      float v[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e)
-        v[e] = aBw[h][0][0][e] * to_f32(sK_[(32 * wi + frag_row(e, lane)) * LDC + 32 * wj + frag_col(lane)]);
-      rows_reduce_add<1>(v, 32 * wi, lane, sdGk);
-    }
-    if (!(wi == 0 && wj == 1)) mma_nt<T, 1, 1>(aX, sK_ + 32 * wi * LDC, LDC, sK_ + 32 * wj * LDC, LDC, 64, lane);
-    // inter-chunk parts scaled, then the intra-chunk products on top
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-      const float gq = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[r]);
-      const float gk = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gl - sG[r], 0.f));
-      aQ[h][0][0][e] *= gq;
-      aK[h][0][0][e] *= gk;
-      tot += aK[h][0][0][e] * to_f32(sK_[r * LDC + c]);
-    }
-    // dq += dPe K,  dk += dPe^T Q: K, Q (and dPe for the second product) contracted along tile rows
-    mma_x<T, 1, 1, false, true>(aQ[h], sPe + 32 * wi * LDC, LDC, sK_ + 32 * wj, LDC, 64, lane);
-    mma_x<T, 1, 1, true, true>(aK[h], sPe + 32 * wi, LDC, sQh + 32 * wj, LDC, 64, lane);
-    if (GATE != LNX_GATE_NONE) {
-      // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts)
-      float v[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        v[e] = aQ[h][0][0][e] * to_f32(sQh[r * LDC + c]) - aK[h][0][0][e] * to_f32(sK_[r * LDC + c]);
-      }
-      rows_reduce_add<1>(v, 32 * wi, lane, sdG);
-    }
-    lds_barrier();  // dB_w complete; all reads of dW done
-    mma_nt<T, 1, 1>(aM, sdBw + 32 * wi * LDC, LDC, sWh + 32 * wj * LDC, LDC, 64, lane);
-    frag_store<T, 1, 1>(aQ[h], sdWh + 32 * wi * LDC + 32 * wj, LDC, lane);
-    lds_barrier();
-    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + 64 * h, DK, sdWh, LDC, len, tid);
-  }
-  if (GATE != LNX_GATE_NONE) {
-    tot = wave_sum(tot);
-    if (lane == 0) atomicAdd(&sMisc[0], tot);
-  }
-
-  // ---------------- phase 3 ----------------
-  lds_barrier();  // W half and the staging tile are dead
-  T* sYa = sWh;   // beta dA E (strictly lower); its transpose is read through the same tile
-  {
-    floatx16 y[1][1];
-    float v[16], cs = 0.f;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      const float da = (i > j) ? -aM[0][0][e] * dec : 0.f;
-      v[e] = da * aX[0][0][e];
-      cs += sBeta[i] * v[e];
-      y[0][0][e] = sBeta[i] * da;
-    }
-    frag_store<T, 1, 1>(y, sYa + 32 * wi * LDC + 32 * wj, LDC, lane);
-    rows_reduce_add<1>(v, 32 * wi, lane, sRow);
-    cs += __shfl_xor(cs, 32, LNX_WAVE);
-    if (lane < 32) atomicAdd(&sCol[32 * wj + lane], cs);
-  }
-  lds_barrier();
-#pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    const T* sK_ = sKh + h * L::kTile;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int r = 32 * wi + frag_row(e, lane);
-      const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[r]);
-      aBw[h][0][0][e] = aBw[h][0][0][e] * sBeta[r] * gm + aK[h][0][0][e];
-    }
-    mma_x<T, 1, 1, false, true>(aBw[h], sYa + 32 * wi * LDC, LDC, sK_ + 32 * wj, LDC, 64, lane);
-    mma_x<T, 1, 1, true, true>(aBw[h], sYa + 32 * wi, LDC, sK_ + 32 * wj, LDC, 64, lane);
-    if (h > 0) lds_barrier();  // the staging tile has been written out
-    frag_store<T, 1, 1>(aBw[h], sdWh + 32 * wi * LDC + 32 * wj, LDC, lane);
-    lds_barrier();
-    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + 64 * h, DK, sdWh, LDC, len, tid);
-  }
-  // dbeta and dg (all row / column sums are complete: the last atomics precede the barrier above)
-  if (wave == 0) {
-    const int t = lane;
-    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[t]);
-    const float w = gm * sdGk[t], rs = sRow[t];
-    if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
-    if (GATE != LNX_GATE_NONE) {
-      float d = sdG[t] + sBeta[t] * (w + rs) - sCol[t];
-      if (t == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
-#pragma unroll
-      for (int s_ = 1; s_ < 64; s_ <<= 1) {
-        const float y = __shfl_down(d, s_, LNX_WAVE);
-        if (t + s_ < 64) d += y;
-      }
-      if (t < len) p.dg[tbase + t] = d;
-    }
-  }
-}
-
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
@@ -1192,19 +886,10 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   }
   lnx_profile_mark("bwd_scan", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(512), b1, st, p);
-  if constexpr (GATE == LNX_GATE_VECTOR) {
-    lnx_profile_mark("bwd_dqk", st);
-    hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
-    lnx_profile_mark("bwd_wy", st);
-    hipLaunchKernelGGL(k3, dim3((unsigned)slots), dim3(256), b3, st, p);
-  } else {
-    auto k4 = bwd_chunk_kernel<T, DK, GATE>;
-    const size_t b4 = FusedCfg<T, DK>::bytes;
-    if ((e = hipFuncSetAttribute((const void*)k4, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b4)) != hipSuccess)
-      return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    lnx_profile_mark("bwd_chunk", st);
-    hipLaunchKernelGGL(k4, dim3((unsigned)slots), dim3(256), b4, st, p);
-  }
+  lnx_profile_mark("bwd_dqk", st);
+  hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
+  lnx_profile_mark("bwd_wy", st);
+  hipLaunchKernelGGL(k3, dim3((unsigned)slots), dim3(256), b3, st, p);
   lnx_profile_mark(nullptr, st);
   return LNX_OK;
 }
