@@ -110,8 +110,8 @@ __global__ __launch_bounds__(256) void l2norm_bwd_kernel(const T* x, const T* dy
 }
 
 int check_norm_args(const void* a, const void* b, int64_t rows, int d, int dtype) {
-  if (!a || !b) return lnx_set_error(LNX_ERR_NULL, "l2norm: NULL tensor");
   if (rows < 0 || d <= 0) return lnx_set_error(LNX_ERR_SHAPE, "l2norm: rows=%lld d=%d", (long long)rows, d);
+  if (rows > 0 && (!a || !b)) return lnx_set_error(LNX_ERR_NULL, "l2norm: NULL tensor");  // empty tensors may be null
   if (dtype != LNX_F32 && dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "l2norm: dtype %d", dtype);
   return LNX_OK;
 }

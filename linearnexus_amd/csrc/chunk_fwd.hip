@@ -807,14 +807,17 @@ int launch_fwd_gate(int gate, const FwdParams& p, int nstate, hipStream_t st) {
 
 int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (!a) return lnx_set_error(LNX_ERR_NULL, "args is NULL");
-  if (!a->q || !a->k || !a->v || !a->beta) return lnx_set_error(LNX_ERR_NULL, "q, k, v and beta are required");
-  if (!backward && (!a->o || !a->final_state)) return lnx_set_error(LNX_ERR_NULL, "o and final_state are required");
-  if (backward && (!a->d_o || !a->d_q || !a->d_k || !a->d_v || !a->d_beta))
-    return lnx_set_error(LNX_ERR_NULL, "d_o, d_q, d_k, d_v and d_beta are required");
-  if (a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
-  if (backward && a->gate != LNX_GATE_NONE && !a->d_g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs d_g", a->gate);
-  if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
   if (a->B < 0 || a->H <= 0 || a->T < 0) return lnx_set_error(LNX_ERR_SHAPE, "bad dimensions B=%d H=%d T=%d", a->B, a->H, a->T);
+  // tensors without elements (no batch rows, or no tokens) may come with null pointers
+  const bool tokens = a->B > 0 && a->T > 0;
+  if (tokens && (!a->q || !a->k || !a->v || !a->beta)) return lnx_set_error(LNX_ERR_NULL, "q, k, v and beta are required");
+  if (!backward && ((tokens && !a->o) || (a->B > 0 && !a->final_state)))
+    return lnx_set_error(LNX_ERR_NULL, "o and final_state are required");
+  if (backward && tokens && (!a->d_o || !a->d_q || !a->d_k || !a->d_v || !a->d_beta))
+    return lnx_set_error(LNX_ERR_NULL, "d_o, d_q, d_k, d_v and d_beta are required");
+  if (tokens && a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
+  if (backward && tokens && a->gate != LNX_GATE_NONE && !a->d_g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs d_g", a->gate);
+  if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
   if (a->dk != 64 && a->dk != 128) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128}, got %d", a->dk);
   if (a->dv <= 0 || a->dv % 64 != 0) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dv %% 64 == 0, got %d", a->dv);
   if (a->chunk != LNX_C) return lnx_set_error(LNX_ERR_SHAPE, "chunk length must be %d, got %d", LNX_C, a->chunk);

@@ -228,12 +228,14 @@ int launch_dk(bool decode, int dk, int gate, const TokenParams& p, dim3 grid, hi
 
 int token_entry(bool decode, const lnx_scan_args* a, void* stream) {
   if (!a) return lnx_set_error(LNX_ERR_NULL, "args is NULL");
-  if (!a->q || !a->k || !a->v || !a->beta || !a->o || !a->final_state)
-    return lnx_set_error(LNX_ERR_NULL, "q, k, v, beta, o and final_state are required");
-  if (a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
-  if (decode && !a->initial_state) return lnx_set_error(LNX_ERR_NULL, "decode step needs the current state");
   if (a->B < 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0 || (!decode && a->T < 0))
     return lnx_set_error(LNX_ERR_SHAPE, "bad dimensions B=%d H=%d T=%d dk=%d dv=%d", a->B, a->H, a->T, a->dk, a->dv);
+  // tensors without elements (no batch rows, or no tokens in a scan) may come with null pointers
+  const bool tokens = a->B > 0 && (decode || a->T > 0);
+  if ((tokens && (!a->q || !a->k || !a->v || !a->beta || !a->o)) || (a->B > 0 && !a->final_state))
+    return lnx_set_error(LNX_ERR_NULL, "q, k, v, beta, o and final_state are required");
+  if (tokens && a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
+  if (decode && a->B > 0 && !a->initial_state) return lnx_set_error(LNX_ERR_NULL, "decode step needs the current state");
   if (a->dv % 4 != 0) return lnx_set_error(LNX_ERR_SHAPE, "dv must be a multiple of 4, got %d", a->dv);
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
   if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);

@@ -38,9 +38,14 @@ def test_struct_layout_matches_header():
 def test_argument_validation_without_gpu():
     lib = _lib.load()
     a = _lib.ScanArgs()
-    assert lib.lnx_decode_step(a, None) == -1 and b"required" in lib.lnx_last_error()
-    assert lib.lnx_chunk_fwd(a, None) < 0
-    assert lib.lnx_chunk_bwd(a, None) < 0
+    for fn in (lib.lnx_decode_step, lib.lnx_recurrent_fwd, lib.lnx_chunk_fwd, lib.lnx_chunk_bwd):
+        assert fn(a, None) == -2 and b"dimensions" in lib.lnx_last_error()  # all-zero struct: H = 0
+    a.B, a.H, a.T, a.dk, a.dv, a.chunk = 1, 1, 1, 64, 64, 64
+    for fn in (lib.lnx_decode_step, lib.lnx_recurrent_fwd, lib.lnx_chunk_fwd, lib.lnx_chunk_bwd):
+        assert fn(a, None) == -1 and b"required" in lib.lnx_last_error()    # null tensors with elements
+    a.B = 0  # an empty batch has no elements behind any pointer: accepted, nothing is launched
+    for fn in (lib.lnx_decode_step, lib.lnx_recurrent_fwd, lib.lnx_chunk_fwd, lib.lnx_chunk_bwd):
+        assert fn(a, None) == 0
     assert lib.lnx_l2norm_fwd(None, None, 4, 8, 0, None) == -1
 
 

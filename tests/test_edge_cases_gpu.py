@@ -1,0 +1,133 @@
+"""GPU parity on the edges of the input space: empty and one-token inputs, packed batches with
+empty and one-token sequences, wide value heads, hand-over of the state between two calls, and
+the closed forms the reference's tests use (beta = 0, test_deltanet.py:281-297).  Tolerances as
+everywhere: max|x - ref| / max|ref| below 1e-4 for fp32 inputs and 2e-2 for bf16 inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import recurrent as rc
+from oracle.adjoint import delta_rule_adjoint
+from oracle.inputs import make_inputs
+from conftest import max_rel
+from test_chunk_bwd_gpu import gpu_grads, check, _prep as _prep_bwd
+from test_chunk_fwd_gpu import gpu_chunk_fwd, oracle_fwd, _prep
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+GATES = ["none", "scalar", "vector"]
+
+
+@pytest.mark.parametrize("gate", GATES)
+def test_empty_sequence_returns_initial_state(gate):
+    import linearnexus_amd as la
+    B, H, d = 2, 3, 64
+    z = lambda *s: torch.zeros(*s, device=DEV)
+    S0 = torch.randn(B, H, d, d, device=DEV)
+    q = k = v = z(B, H, 0, d)
+    beta = z(B, H, 0)
+    if gate == "none":
+        o, S = la.delta_rule_chunkwise(q, k, v, beta, S0)
+        o2, S2 = la.delta_rule_recurrent(q, k, v, beta, S0)
+    else:
+        g = z(B, H, 0) if gate == "scalar" else z(B, H, 0, d)
+        fn = (la.gated_delta_rule_chunkwise, la.gated_delta_rule_recurrent) if gate == "scalar" else (la.kda_chunkwise, la.kda_recurrent)
+        o, S = fn[0](q, k, v, g, beta, None, S0)
+        o2, S2 = fn[1](q, k, v, g, beta, None, S0)
+    assert o.shape == (B, H, 0, d) and o2.shape == (B, H, 0, d)
+    assert torch.equal(S, S0) and torch.equal(S2, S0)
+
+
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("T", [1, 63, 64, 65])
+def test_lengths_around_one_chunk(gate, T):
+    x = make_inputs(61, 1, 2, T, 64, 64, gate=gate, with_state=True, with_grad=True)
+    o_ref, S_ref = oracle_fwd(x, gate)
+    o, S = gpu_chunk_fwd(x, gate, torch.float32)
+    assert max_rel(o.float().cpu().numpy(), o_ref) < 1e-4 and max_rel(S.cpu().numpy(), S_ref) < 1e-4
+    ref = delta_rule_adjoint(x["q"], x["k"], x["v"], x["beta"], x["dO"], x.get("g"), x["dS"], None, x["S0"], False)
+    check(gpu_grads(x, gate, torch.float32), ref, 1e-4)
+
+
+@pytest.mark.parametrize("gate", GATES)
+def test_packed_batch_with_empty_and_one_token_sequences(gate):
+    H, d = 2, 64
+    cu = np.array([0, 0, 1, 66, 66, 130, 131], np.int32)  # lengths 0, 1, 65, 0, 64, 1
+    T, nseq = int(cu[-1]), len(cu) - 1
+    x = make_inputs(62, 1, H, T, d, d, gate=gate, with_grad=True)
+    rng = np.random.default_rng(62)
+    x["S0"] = (rng.standard_normal((nseq, H, d, d)) * 0.02).astype(np.float32)
+    x["dS"] = (rng.standard_normal((nseq, H, d, d)) * 0.1).astype(np.float32)
+
+    def one(q, k, v, *rest, initial_state=None):
+        y = {"q": q, "k": k, "v": v, "beta": rest[-1], "S0": initial_state}
+        if gate != "none":
+            y["g"] = rest[0]
+        return oracle_fwd(y, gate)
+
+    args = [x["q"], x["k"], x["v"]] + ([x["g"]] if gate != "none" else []) + [x["beta"]]
+    o_ref, S_ref = rc.varlen(one, cu, *args, initial_state=x["S0"])
+    o, S = gpu_chunk_fwd(x, gate, torch.float32, cu=cu)
+    assert max_rel(o.cpu().numpy(), o_ref) < 1e-4 and max_rel(S.cpu().numpy(), S_ref) < 1e-4
+    assert np.array_equal(S[0].cpu().numpy(), x["S0"][0]) and np.array_equal(S[3].cpu().numpy(), x["S0"][3])
+    parts = []
+    for s in range(nseq):
+        a, b = cu[s], cu[s + 1]
+        sl = lambda n: x[n][:, :, a:b]
+        parts.append(delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), sl("g") if gate != "none" else None,
+                                        x["dS"][s:s + 1], None, x["S0"][s:s + 1], False))
+    names = ("dq", "dk", "dv", "dbeta") + (("dg",) if gate != "none" else ())
+    ref = {n: np.concatenate([p[n] for p in parts], 2) for n in names}
+    ref["dS0"] = np.concatenate([p["dS0"] for p in parts], 0)
+    check(gpu_grads(x, gate, torch.float32, cu=cu), ref, 1e-4)
+
+
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("bf16", [False, True])
+def test_wide_value_head(gate, bf16):
+    """dv = 256 with dk = 64: four value slabs per state."""
+    x = make_inputs(63, 1, 2, 150, 64, 256, gate=gate, with_state=True, with_grad=True)
+    xf, dt = _prep(x, bf16)
+    o_ref, S_ref = oracle_fwd(xf, gate)
+    o, S = gpu_chunk_fwd(xf, gate, dt)
+    tol = 2e-2 if bf16 else 1e-4
+    assert max_rel(o.float().cpu().numpy(), o_ref) < tol and max_rel(S.cpu().numpy(), S_ref) < tol
+    xb, dt = _prep_bwd(x, bf16)
+    ref = delta_rule_adjoint(xb["q"], xb["k"], xb["v"], xb["beta"], xb["dO"], xb.get("g"), xb["dS"], None, xb["S0"], False)
+    check(gpu_grads(xb, gate, dt), ref, tol)
+
+
+@pytest.mark.parametrize("gate", GATES)
+def test_state_hand_over_between_calls(gate):
+    """[0, T1) followed by [T1, T) with the first call's final state == one call over [0, T)."""
+    T, T1 = 200, 77
+    x = make_inputs(64, 2, 2, T, 128, 128, gate=gate, with_state=True)
+    o_full, S_full = gpu_chunk_fwd(x, gate, torch.float32)
+    cut = lambda a, b: {n: (t[:, :, a:b] if n not in ("S0",) else t) for n, t in x.items()}
+    x1 = cut(0, T1)
+    o1, S1 = gpu_chunk_fwd(x1, gate, torch.float32)
+    x2 = cut(T1, T)
+    x2["S0"] = S1.cpu().numpy()
+    o2, S2 = gpu_chunk_fwd(x2, gate, torch.float32)
+    o12 = torch.cat([o1, o2], 2)
+    assert max_rel(o12.cpu().numpy(), o_full.cpu().numpy()) < 1e-4
+    assert max_rel(S2.cpu().numpy(), S_full.cpu().numpy()) < 1e-4
+
+
+@pytest.mark.parametrize("gate", GATES)
+def test_beta_zero_closed_form(gate):
+    """beta = 0: S_T = (prod alpha) S0 and o_t = scale * (e^{G_t} S0)^T q_t."""
+    B, H, T, d = 1, 2, 100, 64
+    x = make_inputs(65, B, H, T, d, d, gate=gate, with_state=True)
+    x["beta"] = np.zeros_like(x["beta"])
+    o, S = gpu_chunk_fwd(x, gate, torch.float32)
+    if gate == "none":
+        G = np.zeros((B, H, T, d))
+    elif gate == "scalar":
+        G = np.cumsum(x["g"].astype(np.float64), 2)[..., None] * np.ones(d)
+    else:
+        G = np.cumsum(x["g"].astype(np.float64), 2)
+    S0 = x["S0"].astype(np.float64)
+    S_ref = np.exp(G[:, :, -1])[..., None] * S0
+    o_ref = d ** -0.5 * np.einsum("bhtk,bhkv->bhtv", x["q"].astype(np.float64) * np.exp(G), S0)
+    assert max_rel(S.cpu().numpy(), S_ref) < 1e-4 and max_rel(o.cpu().numpy(), o_ref) < 1e-4
