@@ -645,15 +645,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     frag_zero(b);
     mma_x<T, 1, 1, false, true>(b, sTmT + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
     frag_store<T, 1, 1>(b, sdBt + 32 * wi * LDC + 32 * wj, LDC, lane);
-    {
-      float v[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        v[e] = b[0][0][e] * to_f32(sKs[r * LDC + c]);
-      }
-      if (GATE != LNX_GATE_VECTOR || !is_k) rows_reduce_add<1>(v, 32 * wi, lane, is_k ? sdGk : sdB);
-    }
     if (is_k) {
 #pragma unroll
       for (int u = 0; u < NKS; ++u)
@@ -666,6 +657,19 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     }
     lds_barrier();
     mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
+    if (GATE != LNX_GATE_VECTOR || !is_k) {  // <dB row, k row> / <dB row, v row>; thread = (row, quarter of the slab)
+      const int r = tid >> 2, q0 = (tid & 3) * 16;
+      float t = 0.f;
+#pragma unroll
+      for (int u = 0; u < 16; u += 4) {
+        const floatx4 b4 = load4(sdBt + r * LDC + q0 + u), k4 = load4(sKs + r * LDC + q0 + u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t += b4[e] * k4[e];
+      }
+      t += __shfl_xor(t, 1, LNX_WAVE);
+      t += __shfl_xor(t, 2, LNX_WAVE);
+      if ((tid & 3) == 0) atomicAdd(&(is_k ? sdGk : sdB)[r], t);
+    }
     if (!is_k) {  // dv = beta dBu, 16-byte stores
       constexpr int VN = Vec16<T>::N;
       T* dvg = reinterpret_cast<T*>(p.dv_out) + tbase * p.dv + 64 * (s_ - NKS);
