@@ -526,14 +526,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     mma_x<T, 1, 1, false, true>(aQ, sPe + 32 * wi * LDC, LDC, sKr + 32 * wj, LDC, 64, lane);
     mma_x<T, 1, 1, true, true>(aK, sPe + 32 * wi, LDC, sQr + 32 * wj, LDC, 64, lane);
     if (GATE != LNX_GATE_NONE) {
-      // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts)
-      float v[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-        v[e] = aQ[0][0][e] * to_f32(sQr[r * LDC + c]) - aK[0][0][e] * to_f32(sKr[r * LDC + c]);
-      }
-      rows_reduce_add<1>(v, 32 * wi, lane, sdG);
       tot = wave_sum(tot);
       if (lane == 0) atomicAdd(&sMisc[0], tot);
     }
@@ -543,10 +535,24 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     lds_barrier();
     unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, DK, sPe, LDC, len, tid);
     unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sOut2, LDC, len, tid);
-    if (GATE != LNX_GATE_NONE && tid < 64) {
-      float d = sdG[tid];
-      if (tid == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
-      atomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + tid], d);
+    if (GATE != LNX_GATE_NONE) {
+      // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts), from the
+      // staged tiles; thread = (row, quarter of the channels)
+      const int r = tid >> 2, q0 = (tid & 3) * 16;
+      float d = 0.f;
+#pragma unroll
+      for (int u = 0; u < 16; u += 4) {
+        const floatx4 dq4 = load4(sPe + r * LDC + q0 + u), q4 = load4(sQr + r * LDC + q0 + u);
+        const floatx4 dk4 = load4(sOut2 + r * LDC + q0 + u), k4 = load4(sKr + r * LDC + q0 + u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) d += dq4[e] * q4[e] - dk4[e] * k4[e];
+      }
+      d += __shfl_xor(d, 1, LNX_WAVE);
+      d += __shfl_xor(d, 2, LNX_WAVE);
+      if ((tid & 3) == 0) {
+        if (r == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
+        atomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + r], d);
+      }
     }
   }
 }
