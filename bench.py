@@ -151,6 +151,17 @@ def bench_chunk(args, torch, la, _lib, name):
         per_kernel.setdefault(kn, []).append(ms)
     _lib.profile_enable(False)
 
+    # the same forward without gradients (prefill / inference): forward_only is set, nothing is saved
+    with torch.no_grad():
+        for _ in range(2):
+            forward()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            forward()
+        torch.cuda.synchronize()
+        fwd_only_ms = (time.perf_counter() - t1) / args.steps * 1e3
+
     if nseq:
         nchunks = H * int(sum(-(-int(l) // C) for l in (cu_np[1:] - cu_np[:-1])))
     else:
@@ -176,6 +187,7 @@ def bench_chunk(args, torch, la, _lib, name):
         "tflops_algorithmic": total_fl / dtm / 1e12,
         "mfma_peak_frac": total_fl / dtm / 1e12 / peak,
         "kernel_ms": {n: round(t, 4) for n, t in avg.items()},
+        "forward_only_ms": round(fwd_only_ms, 4),
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": TRAFFIC.get((name, dom))},
     }

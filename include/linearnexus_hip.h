@@ -49,6 +49,9 @@ typedef struct lnx_scan_args {
   int32_t use_qk_l2norm;    /* normalise q, k rows as x / (|x|_2 + 1e-6) inside the op */
   int32_t nseq;             /* number of packed sequences; 0 for a dense batch */
   float scale;              /* multiplies q (after normalisation) */
+  int32_t forward_only;     /* lnx_chunk_fwd: no backward pass will follow, do not write the per-chunk tensors
+                               only lnx_chunk_bwd reads (inference / prefill); the workspace is still needed */
+  int32_t reserved;         /* must be 0 */
 
   const void* q;
   const void* k;
@@ -98,7 +101,7 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  * Chunked (WY) forward on MFMA.  Replaces delta_rule_chunkwise (delta_net.py:216-354),
  * gated_delta_rule_chunkwise (gated_deltanet.py:232-534), kda_chunkwise (kda.py:350-655).
  * The workspace keeps the per-chunk tensors the backward pass re-uses; pass the same
- * workspace, unchanged, to lnx_chunk_bwd.
+ * workspace, unchanged, to lnx_chunk_bwd (unless forward_only was set).
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);

@@ -29,6 +29,7 @@ struct FwdParams {
   float* sT_out;
   void* o;
   int dv, o_dtype;
+  int save;  // write the per-chunk tensors the backward pass (or the separate output kernel) reads
   float scale;
   char* ws;
   ChunkWs off;
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     T* sTu = sQa;
     for (int idx = tid; idx < 64 * 64; idx += 256) {
       const int r = idx >> 6, c = idx & 63;
-      TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
+      if (p.save) TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
       const float t = sT[r * LNX_LDA + c];
       const float bu = sBeta[c];
       const float bw = (GATE == LNX_GATE_NONE) ? bu : bu * __expf(sG[c]);
@@ -355,7 +356,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         x[e] = (j0 + e < i) ? x[e] : 0.f;
         pp[e] = (j0 + e <= i) ? p.scale * pp[e] : 0.f;
       }
-      store4(Xg + i * 64 + j0, x);
+      if (p.save) store4(Xg + i * 64 + j0, x);
       store4(Pg + i * 64 + j0, pp);
       store4(sA + i * LNX_LDA + j0, x * sBeta[i]);
     }
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
     for (int idx = tid; idx < 64 * 64; idx += 256) {
       const int r = idx >> 6, c = idx & 63;
-      TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
+      if (p.save) TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
       const float t = sT[r * LNX_LDA + c];
       sTm[r * LDC + c] = from_f32<T>(t);
       sTu[r * LDC + c] = from_f32<T>(t * sBeta[c]);
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       if (n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
       lds_barrier();  // B2
       if (n + 1 < c1) nxt.W.store(sW, LDK, mt);
-      unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
+      if (p.save) unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
       lds_barrier();  // B3
       if (n + 1 < c1) commit_rest(nxt);
       if (FUSE && p.o_dtype == LNX_BF16)
@@ -611,7 +612,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
     // S_n -> workspace (the movers are busy issuing loads in this phase)
-    unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
+    if (p.save)
+      unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
     lds_barrier();  // B2
 
     if (FUSE) {
@@ -824,6 +826,8 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
   if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);
   if (a->use_qk_l2norm) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take pre-normalised q, k (use lnx_l2norm_fwd)");
+  if (a->reserved != 0) return lnx_set_error(LNX_ERR_SHAPE, "reserved field must be 0");
+  if (backward && a->forward_only) return lnx_set_error(LNX_ERR_SHAPE, "forward_only is set: the workspace holds nothing for a backward pass");
   if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
     return lnx_set_error(LNX_ERR_SHAPE, "packed batches need B == 1 and nseq > 0 (B=%d nseq=%d)", a->B, a->nseq);
   return LNX_OK;
@@ -868,6 +872,8 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.g = a->g; p.s0 = a->initial_state;
   p.sT_out = a->final_state; p.o = a->o; p.dv = a->dv; p.o_dtype = a->o_dtype; p.scale = a->scale;
+  // 4-byte inputs form the outputs in a separate kernel that reads the state and D back
+  p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);

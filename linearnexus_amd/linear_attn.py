@@ -266,6 +266,8 @@ class _ChunkScan(torch.autograd.Function):
         sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
         a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
         a.nseq = nseq
+        # nothing to differentiate (inference, torch.no_grad()): the kernels skip what only the backward reads
+        a.forward_only = int(not any(ctx.needs_input_grad))
         a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
         a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
         lib = _lib.load()

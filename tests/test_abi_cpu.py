@@ -26,13 +26,13 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() >= 1
+    assert lib.lnx_abi_version() == 2
 
 
 def test_struct_layout_matches_header():
-    # 12 four-byte scalars, then 17 pointers, then the workspace size
-    assert ctypes.sizeof(_lib.ScanArgs) == 48 + 18 * 8 + 8
-    assert _lib.ScanArgs.q.offset == 48
+    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size
+    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8
+    assert _lib.ScanArgs.q.offset == 56
 
 
 def test_argument_validation_without_gpu():

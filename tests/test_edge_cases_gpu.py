@@ -131,3 +131,24 @@ def test_beta_zero_closed_form(gate):
     S_ref = np.exp(G[:, :, -1])[..., None] * S0
     o_ref = d ** -0.5 * np.einsum("bhtk,bhkv->bhtv", x["q"].astype(np.float64) * np.exp(G), S0)
     assert max_rel(S.cpu().numpy(), S_ref) < 1e-4 and max_rel(o.cpu().numpy(), o_ref) < 1e-4
+
+
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("bf16", [False, True])
+def test_forward_without_gradients_skips_nothing_visible(gate, bf16):
+    """Under torch.no_grad() the op sets forward_only (the kernels do not write what only the backward
+    reads); outputs and final state must be bit-identical to the differentiable call."""
+    x = make_inputs(66, 2, 2, 300, 128, 128, gate=gate, with_state=True)
+    x, dt = _prep(x, bf16)
+    with torch.no_grad():
+        o1, S1 = gpu_chunk_fwd(x, gate, dt)
+    import linearnexus_amd as la
+    q, k, v = (torch.from_numpy(x[n]).to(DEV).to(dt).requires_grad_(True) for n in ("q", "k", "v"))
+    beta, s0 = torch.from_numpy(x["beta"]).to(DEV), torch.from_numpy(x["S0"]).to(DEV)
+    if gate == "none":
+        o2, S2 = la.delta_rule_chunkwise(q, k, v, beta, s0)
+    else:
+        fn = la.gated_delta_rule_chunkwise if gate == "scalar" else la.kda_chunkwise
+        o2, S2 = fn(q, k, v, torch.from_numpy(x["g"]).to(DEV), beta, None, s0, 64, False)
+    assert o2.requires_grad and not o1.requires_grad
+    assert torch.equal(o1, o2.detach()) and torch.equal(S1, S2.detach())
