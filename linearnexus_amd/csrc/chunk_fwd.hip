@@ -148,14 +148,23 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
     T* sTw = sKa;
     T* sTu = sQa;
-    for (int idx = tid; idx < 64 * 64; idx += 256) {
-      const int r = idx >> 6, c = idx & 63;
-      if (p.save) TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
-      const float t = sT[r * LNX_LDA + c];
-      const float bu = sBeta[c];
-      const float bw = (GATE == LNX_GATE_NONE) ? bu : bu * __expf(sG[c]);
-      sTu[r * LDC + c] = from_f32<T>(t * bu);
-      sTw[r * LDC + c] = from_f32<T>(t * bw);
+    // one 4x4 block of Tm per thread: four-element row reads, the transpose taken in registers
+    const int r0 = (tid >> 4) * 4, c0 = (tid & 15) * 4;
+    floatx4 t[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = load4(sT + (r0 + i) * LNX_LDA + c0);
+    const floatx4 bu = load4(sBeta + c0);
+    floatx4 bw = bu;
+    if (GATE != LNX_GATE_NONE) {
+      const floatx4 g4 = load4(sG + c0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bw[e] = bu[e] * __expf(g4[e]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      store4(sTu + (r0 + i) * LDC + c0, t[i] * bu);
+      store4(sTw + (r0 + i) * LDC + c0, t[i] * bw);
+      if (p.save) store4(TmT + (c0 + i) * 64 + r0, floatx4{t[0][i], t[1][i], t[2][i], t[3][i]});
     }
   }
   const int nslab = NKS + p.dv / 64;
@@ -369,12 +378,17 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   T* sTu = sQ;
   {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
-    for (int idx = tid; idx < 64 * 64; idx += 256) {
-      const int r = idx >> 6, c = idx & 63;
-      if (p.save) TmT[idx] = from_f32<T>(sT[c * LNX_LDA + r]);
-      const float t = sT[r * LNX_LDA + c];
-      sTm[r * LDC + c] = from_f32<T>(t);
-      sTu[r * LDC + c] = from_f32<T>(t * sBeta[c]);
+    // one 4x4 block of Tm per thread: four-element row reads, the transpose taken in registers
+    const int r0 = (tid >> 4) * 4, c0 = (tid & 15) * 4;
+    floatx4 t[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = load4(sT + (r0 + i) * LNX_LDA + c0);
+    const floatx4 bu = load4(sBeta + c0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      store4(sTm + (r0 + i) * LDC + c0, t[i]);
+      store4(sTu + (r0 + i) * LDC + c0, t[i] * bu);
+      if (p.save) store4(TmT + (c0 + i) * 64 + r0, floatx4{t[0][i], t[1][i], t[2][i], t[3][i]});
     }
   }
   // ---- phase D: W = Tm (beta e^G K), U = Tu V, one 64-column slab at a time ----
