@@ -33,10 +33,9 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
 TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 865266704, ("gdn_chunk", "chunk_scan"): 1151563238,
-    ("gdn_chunk", "bwd_local"): 337689355, ("gdn_chunk", "bwd_scan"): 1084420419,
-    ("gdn_chunk", "bwd_dqk"): 1617062844, ("gdn_chunk", "bwd_wy"): 1485695358,
-    ("decode", "decode_step"): 1083425683,
+    ("gdn_chunk", "chunk_prepare"): 860879916, ("gdn_chunk", "chunk_scan"): 1151569502,
+    ("gdn_chunk", "bwd_scan"): 1019424981, ("gdn_chunk", "bwd_dqk"): 1617043803,
+    ("gdn_chunk", "bwd_wy"): 1485082613, ("decode", "decode_step"): 1083423645,
 }
 
 
