@@ -43,7 +43,27 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print(f"built {LIB} from {', '.join(srcs)}")
+    build_c_abi_smoke(verbose)
     return LIB
+
+
+def build_c_abi_smoke(verbose: bool = True) -> str:
+    """Compiles tests/c_abi/abi_smoke.c (plain C, gcc) against the library just built; the GPU test
+    tests/test_c_abi_gpu.py runs the binary."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "c_abi", "abi_smoke.c")
+    exe = os.path.join(root, "tests", "c_abi", "abi_smoke")
+    if not os.path.exists(src):
+        return ""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-O2", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", src, "-o", exe, f"-L{rocm}/lib", "-lamdhip64",
+           f"-L{HERE}", "-llinearnexus_hip", "-lm", "-Wl,-rpath,$ORIGIN/../../linearnexus_amd", f"-Wl,-rpath,{rocm}/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the C-ABI smoke program failed:\n" + r.stderr)
+    if verbose:
+        print(f"built {exe}")
+    return exe
 
 
 if __name__ == "__main__":
