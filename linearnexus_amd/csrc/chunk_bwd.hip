@@ -121,11 +121,11 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
-  const int sidx = blockIdx.x;
-  const int row = p.geom.tab ? sidx % H : sidx;
+  int sidx, row, seq;  // state index, (batch, head) row, sequence
+  scan_state(p.geom, blockIdx.x, sidx, row, seq);
   const int v0 = blockIdx.y * BV;
   int c0, c1;
-  seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+  seq_chunks(p.geom, seq, c0, c1);
 
   if (wave >= 4) {
     // ---------------- movers ----------------

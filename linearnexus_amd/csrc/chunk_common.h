@@ -27,7 +27,7 @@
 struct ChunkGeom {
   int H, T, N, nseq, rows;       // rows = B * H (dense) or H (packed); N = chunk slots per row
   const int32_t* cu;             // device cu_seqlens or nullptr
-  const int32_t* tab;            // packed only: [N][2] (token0, len) then seq_chunk0[nseq + 1]
+  const int32_t* tab;            // packed only: [N][2] (token0, len), seq_chunk0[nseq + 1], order[nseq]
 };
 
 __device__ __forceinline__ void chunk_span(const ChunkGeom& g, int n, int& tok0, int& len) {
@@ -37,6 +37,20 @@ __device__ __forceinline__ void chunk_span(const ChunkGeom& g, int n, int& tok0,
   } else {
     tok0 = n * LNX_C;
     len = min(LNX_C, g.T - tok0);
+  }
+}
+
+// The sequential kernels take one workgroup per (state, head): blockIdx.x -> state index and row.
+// Packed batches hand the sequences out longest first (order[] of the table), so that the longest
+// chains start first when there are more workgroups than fit the chip at once.
+__device__ __forceinline__ void scan_state(const ChunkGeom& g, int bx, int& sidx, int& row, int& seq) {
+  if (g.tab) {
+    seq = g.tab[2 * g.N + g.nseq + 1 + bx / g.H];
+    row = bx % g.H;
+    sidx = seq * g.H + row;
+  } else {
+    seq = 0;
+    sidx = row = bx;
   }
 }
 
@@ -80,7 +94,7 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   const uint64_t slots = rows * N, dk = a->dk, dv = a->dv, C = LNX_C;
   uint64_t off = 0;
   auto take = [&](uint64_t bytes) { uint64_t o = off; off = lnx_align256(off + bytes); return o; };
-  w.tab = take(a->cu_seqlens ? (2 * N + a->nseq + 1) * 4 : 0);
+  w.tab = take(a->cu_seqlens ? (2 * N + 2 * (uint64_t)a->nseq + 1) * 4 : 0);
   w.G = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
   w.X = take(a->gate == LNX_GATE_VECTOR ? slots * C * C * es : 0);

@@ -501,11 +501,11 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int H = p.geom.H, N = p.geom.N;
-  const int sidx = blockIdx.x;  // state index
-  const int row = p.geom.tab ? sidx % H : sidx;
+  int sidx, row, seq;  // state index, (batch, head) row, sequence
+  scan_state(p.geom, blockIdx.x, sidx, row, seq);
   const int v0 = blockIdx.y * BV;
   int c0, c1;
-  seq_chunks(p.geom, p.geom.tab ? sidx / H : 0, c0, c1);
+  seq_chunks(p.geom, seq, c0, c1);
 
   if (wave >= 4) {
     // ---------------- movers ----------------
@@ -757,9 +757,20 @@ __global__ void copy_state_kernel(const float* src, float* dst, int64_t n) {
   if (i < n) dst[i] = src ? src[i] : 0.f;
 }
 
-// packed batches: slot table [N][2] = (token0, len) followed by seq_chunk0[nseq + 1]
+// packed batches: slot table [N][2] = (token0, len), then seq_chunk0[nseq + 1], then the sequence
+// indices by decreasing length (ties by index).  One workgroup.
 __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* tab) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int32_t* order = tab + 2 * N + nseq + 1;
+  for (int s = threadIdx.x; s < nseq; s += blockDim.x) {
+    const int ls = cu[s + 1] - cu[s];
+    int rank = 0;
+    for (int u = 0; u < nseq; ++u) {
+      const int lu = cu[u + 1] - cu[u];
+      rank += (lu > ls) || (lu == ls && u < s);
+    }
+    order[rank] = s;
+  }
+  if (threadIdx.x != 0) return;
   int c = 0;
   for (int s = 0; s < nseq; ++s) {
     tab[2 * N + s] = c;
@@ -849,7 +860,7 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
 
 void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st) {
   if (!a->cu_seqlens) return;
-  hipLaunchKernelGGL(build_table_kernel, dim3(1), dim3(64), 0, st, a->cu_seqlens, a->nseq, lnx_chunk_slots(a),
+  hipLaunchKernelGGL(build_table_kernel, dim3(1), dim3(256), 0, st, a->cu_seqlens, a->nseq, lnx_chunk_slots(a),
                      reinterpret_cast<int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab));
 }
 
