@@ -85,9 +85,11 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 //   B2  dD is in LDS (plain and negated-transposed)  compute: dS update   movers: K of chunk n-1 -> LDS, dD -> workspace
 //   B3  all reads of chunk n's tiles are done     compute: dS^T -> LDS  movers: remaining tiles of chunk n-1 -> LDS
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct BScanCfg {
+// BVW = columns of dv per workgroup: 64 by default; 32 for dk = 128 with 4-byte inputs (LDS capacity) and,
+// on request, for dk = 128 with 2-byte inputs when 64-column slabs would leave most CUs idle.
+template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int BV = (DK == 128 && sizeof(T) == 4) ? 32 : 64;  // dv slab per workgroup (LDS capacity)
+  static constexpr int BV = (DK == 128 && sizeof(T) == 4) ? 32 : BVW;
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
@@ -99,9 +101,9 @@ template <typename T, int DK> struct BScanCfg {
   static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * 128;
 };
 
-template <typename T, int DK, int GATE>
+template <typename T, int DK, int GATE, int BVW = 64>
 __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
-  typedef BScanCfg<T, DK> L;
+  typedef BScanCfg<T, DK, BVW> L;
   constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV;
   constexpr bool FUSE = L::FUSE_LOCAL;
   constexpr int CT = BV / 32;                      // column tiles of the slab
@@ -881,10 +883,14 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
-  auto k1 = bwd_scan_kernel<T, DK, GATE>;
+  constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
+  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, (can_narrow ? 32 : 64)> : bwd_scan_kernel<T, DK, GATE, 64>;
+  const int bv = narrow ? 32 : BScanCfg<T, DK, 64>::BV;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
   auto k3 = bwd_wy2_kernel<T, DK, GATE>;
-  const size_t b1 = BScanCfg<T, DK>::bytes, b2 = DqkCfg<T, DK, GATE>::bytes, b3 = Wy2Cfg<T, DK, GATE>::bytes;
+  const size_t b1 = narrow ? BScanCfg<T, DK, (can_narrow ? 32 : 64)>::bytes : BScanCfg<T, DK, 64>::bytes;
+  const size_t b2 = DqkCfg<T, DK, GATE>::bytes, b3 = Wy2Cfg<T, DK, GATE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
@@ -895,7 +901,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
     hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
   }
   lnx_profile_mark("bwd_scan", st);
-  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / BScanCfg<T, DK>::BV)), dim3(512), b1, st, p);
+  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / bv)), dim3(512), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("bwd_wy", st);

@@ -22,6 +22,8 @@
 // and dG (fp32 partial gradient of the cumulative gate).
 #pragma once
 
+#include <stdlib.h>
+
 #include "mma_tiles.h"
 
 struct ChunkGeom {
@@ -111,6 +113,16 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.dG = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
   w.total = off;
   return w;
+}
+
+// Slab width of the two sequential kernels: 32 columns when 64-column slabs would give workgroups to at
+// most half of the 256 CUs.  LNX_SCAN_SLAB=32 or 64 in the environment overrides the choice (used by the
+// tests to cover both variants at small shapes).
+inline bool lnx_narrow_slabs(int64_t wide_workgroups) {
+  const char* e = getenv("LNX_SCAN_SLAB");
+  if (e && e[0] == '3') return true;
+  if (e && e[0] == '6') return false;
+  return wide_workgroups <= 128;
 }
 
 // Shared argument validation of the chunk entry points; returns LNX_OK or an error status.

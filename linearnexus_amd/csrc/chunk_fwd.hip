@@ -464,11 +464,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
 //   B3  all reads of chunk n's tiles are done
 //         compute: S_{n+1} -> LDS            movers: remaining tiles of chunk n+1 -> LDS, outputs -> global
 // ---------------------------------------------------------------------------------------
-template <typename T, int DK> struct ScanSmem {
+// BV = columns of dv per workgroup: 64, or 32 (dk = 128, 2-byte inputs) when 64-column slabs would
+// leave more than half of the CUs without a workgroup.
+template <typename T, int DK, int BVW = 64> struct ScanSmem {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
-  static constexpr int BV = 64;  // dv slab per workgroup
+  static constexpr int BV = BVW;
   static constexpr bool FUSE_OUT = sizeof(T) == 2;
   static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
   static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
@@ -477,16 +479,16 @@ template <typename T, int DK> struct ScanSmem {
                                   (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (128 + 4);
 };
 
-template <typename T, int DK, int GATE>
+template <typename T, int DK, int GATE, int BVW = 64>
 __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
-  typedef ScanSmem<T, DK> L;
+  typedef ScanSmem<T, DK, BVW> L;
   constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD, LDO = L::LDO;
   constexpr bool FUSE = L::FUSE_OUT;
   // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and all column tiles,
   // DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
   constexpr int CT = BV / 32;
   constexpr int NT = (DK == 128) ? CT : 1;
-  static_assert(BV == 64, "one 32x32 tile of the [64 x BV] products per wave");
+  static_assert(BV == 64 || (BV == 32 && DK == 128), "32-column slabs: the wave's state tile must be a full row tile");
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
   T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
@@ -588,7 +590,9 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   // ---------------- compute waves ----------------
   const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
   const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
-  const int wi = wave >> 1, wj = wave & 1;  // this wave's tile of the [64 x BV] products
+  // this wave's 32x32 tile of the [64 x BV] products (a 32-column slab has two tiles: waves 0 and 1)
+  const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
+  const bool has_tile = (CT == 2) || wave < 2;
 
   floatx16 S[1][NT];
   frag_zero(S);
@@ -606,7 +610,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   for (int n = c0; n < c1; ++n) {
     // D = U - W S  (one 32x32 tile per wave)
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
-    {
+    if (has_tile) {
       floatx16 d[1][1];
       frag_zero(d);
       mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
@@ -630,7 +634,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
     lds_barrier();  // B2
 
-    if (FUSE) {
+    if (FUSE && has_tile) {
       // o = scale e^G (Q S) + P D for this slab
       floatx16 o[1][1];
       frag_zero(o);
@@ -800,9 +804,14 @@ template <typename T, int DK, int GATE>
 int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   auto k1 = PrepSelect<T, DK, GATE>::kernel();
-  auto k2 = chunk_scan_kernel<T, DK, GATE>;
+  // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs)
+  constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
+  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, (can_narrow ? 32 : 64)> : chunk_scan_kernel<T, DK, GATE, 64>;
   auto k3 = chunk_output_kernel<T, DK, GATE>;
-  const size_t b1 = PrepSelect<T, DK, GATE>::bytes, b2 = ScanSmem<T, DK>::bytes, b3 = OutSmem<T, DK>::bytes;
+  const int bv = narrow ? 32 : 64;
+  const size_t b1 = PrepSelect<T, DK, GATE>::bytes, b3 = OutSmem<T, DK>::bytes;
+  const size_t b2 = narrow ? ScanSmem<T, DK, (can_narrow ? 32 : 64)>::bytes : ScanSmem<T, DK, 64>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
@@ -811,7 +820,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   lnx_profile_mark("chunk_prepare", st);
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
   lnx_profile_mark("chunk_scan", st);
-  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / ScanSmem<T, DK>::BV)), dim3(512), b2, st, p);
+  hipLaunchKernelGGL(k2, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / bv)), dim3(512), b2, st, p);
   if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
     hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
