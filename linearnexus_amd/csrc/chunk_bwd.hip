@@ -122,7 +122,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   float* sG = reinterpret_cast<float*>(sdOr + L::kRaw);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int H = p.geom.H, N = p.geom.N;
+  const int N = p.geom.N;
   int sidx, row, seq;  // state index, (batch, head) row, sequence
   scan_state(p.geom, blockIdx.x, sidx, row, seq);
   const int v0 = blockIdx.y * BV;
@@ -328,8 +328,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   constexpr int LDC = L::LDC, LDF = L::LDF;
   extern __shared__ __align__(16) char smem[];
   float* sG = reinterpret_cast<float*>(smem);
-  float* sdG = sG + 64;     // per-row gate-gradient accumulator
-  float* sSS = sdG + 64;    // vector gate: per key channel sum_v dS_n[c][v] S_n[c][v]
+  float* sSS = sG + 64;     // vector gate: per key channel sum_v dS_n[c][v] S_n[c][v]
   float* sMisc = sSS + 64;  // [0] = sum_j r_j <dKr_j, k_j>, [1] = <dS_n, S_n>
   float* sR = sMisc + 64;   // vector gate only: dP [64][LNX_LDA]
   T* sdO = reinterpret_cast<T*>(sMisc + 64 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0));
@@ -355,7 +354,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
 
   if (tid < 64) {
     sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sdG[tid] = 0.f;
     sSS[tid] = 0.f;
     sMisc[tid] = 0.f;
   }

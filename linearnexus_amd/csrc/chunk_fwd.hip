@@ -502,7 +502,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   int* sMeta = reinterpret_cast<int*>(sG + 128);  // first token and length of the chunk whose tiles are in LDS
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int H = p.geom.H, N = p.geom.N;
+  const int N = p.geom.N;
   int sidx, row, seq;  // state index, (batch, head) row, sequence
   scan_state(p.geom, blockIdx.x, sidx, row, seq);
   const int v0 = blockIdx.y * BV;

@@ -121,18 +121,6 @@ __device__ __forceinline__ void mma_x(floatx16 (&acc)[MT][NT], const T* A, int l
 __device__ __forceinline__ int frag_row(int e, int lane) { return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3); }
 __device__ __forceinline__ int frag_col(int lane) { return lane & 31; }
 
-// Calls f(row, col, value&) for every element of the fragments (rows/cols relative to the
-// wave's tile origin).
-template <int MT, int NT, typename F>
-__device__ __forceinline__ void frag_foreach(floatx16 (&acc)[MT][NT], int lane, F f) {
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) f(32 * i + frag_row(e, lane), 32 * j + frag_col(lane), acc[i][j][e]);
-}
-
 // dst[row][col] = acc (row-major tile with leading dimension ld); dst points at the tile origin.
 template <typename T, int MT, int NT>
 __device__ __forceinline__ void frag_store(const floatx16 (&acc)[MT][NT], T* dst, int64_t ld, int lane,
@@ -204,72 +192,12 @@ template <typename T, int ROWS, int COLS> struct TileRegs {
   }
 };
 
-// The same for a tile that goes to LDS transposed (dst[c][r] = f(r, c) * src[r][c]): each thread
-// holds 4-row x N-column micro-tiles (coalesced 16-byte loads, 4-element LDS stores). ROWS % 4 == 0.
-template <typename T, int ROWS, int COLS> struct TileRegsT {
-  static constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = (ROWS / 4) * VPR, IT = (TOTAL + 255) / 256;
-  typename Vec16<T>::V x[IT][4];
-  __device__ __forceinline__ void load(const T* src, int64_t stride, int valid, int tid) {
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = 4 * rg + i;
-        x[it][i] = vec_zero<T>();
-        if (idx < TOTAL && r < valid) x[it][i] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
-      }
-    }
-  }
-  template <typename F>
-  __device__ __forceinline__ void store(T* dst, int ld, int tid, F elem_scale) const {
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
-      if (idx < TOTAL) {
-#pragma unroll
-        for (int e = 0; e < N; ++e) {
-          floatx4 y;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) y[i] = to_f32(x[it][i][e]) * elem_scale(4 * rg + i, c + e);
-          store4(dst + (c + e) * ld + 4 * rg, y);
-        }
-      }
-    }
-  }
-  __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
-#pragma unroll
-    for (int it = 0; it < IT; ++it) {
-      const int idx = tid + 256 * it, rg = idx / VPR, c = (idx - rg * VPR) * N;
-      if (idx < TOTAL) {
-#pragma unroll
-        for (int e = 0; e < N; ++e) {
-          typename Mma<T>::Quad y = {x[it][0][e], x[it][1][e], x[it][2][e], x[it][3][e]};
-          *reinterpret_cast<typename Mma<T>::Quad*>(dst + (c + e) * ld + 4 * rg) = y;
-        }
-      }
-    }
-  }
-};
-
-// One-shot forms (load, then store) for single tiles.
+// One-shot form (load, then store) for a single tile.
 template <typename T, int ROWS, int COLS>
 __device__ __forceinline__ void stage_tile(T* dst, int ld, const T* src, int64_t stride, int valid, int tid) {
   TileRegs<T, ROWS, COLS> t;
   t.load(src, stride, valid, tid);
   t.store(dst, ld, tid);
-}
-template <typename T, int ROWS, int COLS>
-__device__ __forceinline__ void stage_tile_t(T* dst, int ld, const T* src, int64_t stride, int valid, int tid) {
-  TileRegsT<T, ROWS, COLS> t;
-  t.load(src, stride, valid, tid);
-  t.store(dst, ld, tid);
-}
-template <typename T, int ROWS, int COLS, typename F>
-__device__ __forceinline__ void stage_tile_t(T* dst, int ld, const T* src, int64_t stride, int valid, int tid, F f) {
-  TileRegsT<T, ROWS, COLS> t;
-  t.load(src, stride, valid, tid);
-  t.store(dst, ld, tid, f);
 }
 
 // LDS tile [ROWS][COLS] (leading dimension ld) -> global, 16-byte vectors, rows < valid only.
