@@ -5,7 +5,7 @@
 
 #include <mutex>
 
-#include "lnx_common.h"
+#include "mma_tiles.h"
 
 namespace {
 thread_local char g_error[512] = "";
@@ -109,6 +109,121 @@ __global__ __launch_bounds__(256) void l2norm_bwd_kernel(const T* x, const T* dy
   for (int i = lane; i < d; i += 64) dx[row * d + i] = from_f32<T>(to_f32(gr[i]) / s - to_f32(xr[i]) * c);
 }
 
+// Vector forms for rows of LPR 16-byte vectors (LPR a power of two <= 64): LPR lanes share a row, a
+// wavefront covers 64 / LPR rows per pass and four passes per step (all loads of a step issued
+// before the first reduction), so the kernels run at streaming bandwidth.
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void l2norm_fwd_vec_kernel(const T* x, T* y, int64_t rows) {
+  typedef typename Vec16<T>::V V;
+  constexpr int VN = Vec16<T>::N, RPW = 64 / LPR, UNR = 4, D = LPR * VN;
+  const int lane = threadIdx.x & 63, sub = lane / LPR, li = lane % LPR;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t r0 = wave * (RPW * UNR) + sub;
+  V xv[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    xv[u] = vec_zero<T>();
+    if (r < rows) xv[u] = *reinterpret_cast<const V*>(x + r * D + li * VN);
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) { const float t = to_f32(xv[u][e]); ss += t * t; }
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, LNX_WAVE);
+    const float inv = 1.f / (sqrtf(ss) + LNX_L2_EPS);
+    V out;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) out[e] = from_f32<T>(to_f32(xv[u][e]) * inv);
+    if (r < rows) *reinterpret_cast<V*>(y + r * D + li * VN) = out;
+  }
+}
+
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void l2norm_bwd_vec_kernel(const T* x, const T* dy, T* dx, int64_t rows) {
+  typedef typename Vec16<T>::V V;
+  constexpr int VN = Vec16<T>::N, RPW = 64 / LPR, UNR = 4, D = LPR * VN;
+  const int lane = threadIdx.x & 63, sub = lane / LPR, li = lane % LPR;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t r0 = wave * (RPW * UNR) + sub;
+  V xv[UNR], gv[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    xv[u] = vec_zero<T>();
+    gv[u] = vec_zero<T>();
+    if (r < rows) {
+      xv[u] = *reinterpret_cast<const V*>(x + r * D + li * VN);
+      gv[u] = *reinterpret_cast<const V*>(dy + r * D + li * VN);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    float ss = 0.f, dot = 0.f;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) {
+      const float t = to_f32(xv[u][e]);
+      ss += t * t;
+      dot += t * to_f32(gv[u][e]);
+    }
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) {
+      ss += __shfl_xor(ss, m, LNX_WAVE);
+      dot += __shfl_xor(dot, m, LNX_WAVE);
+    }
+    const float n = sqrtf(ss), sd = n + LNX_L2_EPS;
+    const float c = dot / (fmaxf(n, 1e-30f) * sd * sd);
+    V out;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) out[e] = from_f32<T>(to_f32(gv[u][e]) / sd - to_f32(xv[u][e]) * c);
+    if (r < rows) *reinterpret_cast<V*>(dx + r * D + li * VN) = out;
+  }
+}
+
+// lanes per row for the vector kernels, or 0 when the row length does not fit them
+template <typename T> int norm_lanes(int d) {
+  constexpr int VN = 16 / sizeof(T);
+  if (d % VN != 0) return 0;
+  const int l = d / VN;
+  return (l == 4 || l == 8 || l == 16 || l == 32 || l == 64) ? l : 0;
+}
+
+template <typename T>
+bool launch_norm_fwd(const T* x, T* y, int64_t rows, int d, hipStream_t st) {
+  const int l = norm_lanes<T>(d);
+  if (!l) return false;
+  const int64_t waves = (rows + (64 / l) * 4 - 1) / ((64 / l) * 4);
+  dim3 grid((unsigned)((waves + 3) / 4));
+  switch (l) {
+    case 4: hipLaunchKernelGGL((l2norm_fwd_vec_kernel<T, 4>), grid, dim3(256), 0, st, x, y, rows); break;
+    case 8: hipLaunchKernelGGL((l2norm_fwd_vec_kernel<T, 8>), grid, dim3(256), 0, st, x, y, rows); break;
+    case 16: hipLaunchKernelGGL((l2norm_fwd_vec_kernel<T, 16>), grid, dim3(256), 0, st, x, y, rows); break;
+    case 32: hipLaunchKernelGGL((l2norm_fwd_vec_kernel<T, 32>), grid, dim3(256), 0, st, x, y, rows); break;
+    default: hipLaunchKernelGGL((l2norm_fwd_vec_kernel<T, 64>), grid, dim3(256), 0, st, x, y, rows); break;
+  }
+  return true;
+}
+
+template <typename T>
+bool launch_norm_bwd(const T* x, const T* dy, T* dx, int64_t rows, int d, hipStream_t st) {
+  const int l = norm_lanes<T>(d);
+  if (!l) return false;
+  const int64_t waves = (rows + (64 / l) * 4 - 1) / ((64 / l) * 4);
+  dim3 grid((unsigned)((waves + 3) / 4));
+  switch (l) {
+    case 4: hipLaunchKernelGGL((l2norm_bwd_vec_kernel<T, 4>), grid, dim3(256), 0, st, x, dy, dx, rows); break;
+    case 8: hipLaunchKernelGGL((l2norm_bwd_vec_kernel<T, 8>), grid, dim3(256), 0, st, x, dy, dx, rows); break;
+    case 16: hipLaunchKernelGGL((l2norm_bwd_vec_kernel<T, 16>), grid, dim3(256), 0, st, x, dy, dx, rows); break;
+    case 32: hipLaunchKernelGGL((l2norm_bwd_vec_kernel<T, 32>), grid, dim3(256), 0, st, x, dy, dx, rows); break;
+    default: hipLaunchKernelGGL((l2norm_bwd_vec_kernel<T, 64>), grid, dim3(256), 0, st, x, dy, dx, rows); break;
+  }
+  return true;
+}
+
 int check_norm_args(const void* a, const void* b, int64_t rows, int d, int dtype) {
   if (rows < 0 || d <= 0) return lnx_set_error(LNX_ERR_SHAPE, "l2norm: rows=%lld d=%d", (long long)rows, d);
   if (rows > 0 && (!a || !b)) return lnx_set_error(LNX_ERR_NULL, "l2norm: NULL tensor");  // empty tensors may be null
@@ -127,11 +242,16 @@ int finish(const char* what) {
 extern "C" int lnx_l2norm_fwd(const void* x, void* y, int64_t rows, int32_t d, int32_t dtype, void* stream) {
   int rc = check_norm_args(x, y, rows, d, dtype);
   if (rc != LNX_OK || rows == 0) return rc;
-  dim3 grid((unsigned)((rows + 3) / 4));
-  if (dtype == LNX_BF16)
-    hipLaunchKernelGGL(l2norm_fwd_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (bf16_t*)y, rows, d);
-  else
-    hipLaunchKernelGGL(l2norm_fwd_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, (float*)y, rows, d);
+  hipStream_t st = (hipStream_t)stream;
+  const bool vec = (dtype == LNX_BF16) ? launch_norm_fwd<bf16_t>((const bf16_t*)x, (bf16_t*)y, rows, d, st)
+                                       : launch_norm_fwd<float>((const float*)x, (float*)y, rows, d, st);
+  if (!vec) {  // row lengths the vector kernels do not cover
+    dim3 grid((unsigned)((rows + 3) / 4));
+    if (dtype == LNX_BF16)
+      hipLaunchKernelGGL(l2norm_fwd_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, (bf16_t*)y, rows, d);
+    else
+      hipLaunchKernelGGL(l2norm_fwd_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (float*)y, rows, d);
+  }
   return finish("l2norm_fwd");
 }
 
@@ -139,12 +259,18 @@ extern "C" int lnx_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t r
                               void* stream) {
   int rc = check_norm_args(x, dy, rows, d, dtype);
   if (rc != LNX_OK) return rc;
-  if (!dx) return lnx_set_error(LNX_ERR_NULL, "l2norm_bwd: dx is NULL");
   if (rows == 0) return LNX_OK;
-  dim3 grid((unsigned)((rows + 3) / 4));
-  if (dtype == LNX_BF16)
-    hipLaunchKernelGGL(l2norm_bwd_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dx, rows, d);
-  else
-    hipLaunchKernelGGL(l2norm_bwd_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)x, (const float*)dy, (float*)dx, rows, d);
+  if (!dx) return lnx_set_error(LNX_ERR_NULL, "l2norm_bwd: dx is NULL");
+  hipStream_t st = (hipStream_t)stream;
+  const bool vec = (dtype == LNX_BF16)
+                       ? launch_norm_bwd<bf16_t>((const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dx, rows, d, st)
+                       : launch_norm_bwd<float>((const float*)x, (const float*)dy, (float*)dx, rows, d, st);
+  if (!vec) {
+    dim3 grid((unsigned)((rows + 3) / 4));
+    if (dtype == LNX_BF16)
+      hipLaunchKernelGGL(l2norm_bwd_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dx, rows, d);
+    else
+      hipLaunchKernelGGL(l2norm_bwd_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)dy, (float*)dx, rows, d);
+  }
   return finish("l2norm_bwd");
 }

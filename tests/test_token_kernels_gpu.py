@@ -151,12 +151,20 @@ def test_beta_zero_leaves_zero_state_on_gpu():
     assert torch.count_nonzero(S) == 0 and torch.count_nonzero(o) == 0
 
 
-def test_l2norm_rows_fwd_bwd():
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,d", [(37, 128), (1, 64), (1000, 256), (130, 16), (5, 100), (9, 512), (0, 128)])
+def test_l2norm_rows_fwd_bwd(rows, d, bf16):
+    """x / (|x| + 1e-6) and its gradient; covers the vector kernels (16-byte row pieces, 4..64 lanes per
+    row), the scalar fallback for other row lengths, ragged last passes and an empty tensor."""
     import linearnexus_amd as la
     from linearnexus_amd.linear_attn import _l2norm_rows_bwd
-    x = torch.randn(37, 128, device=DEV, requires_grad=True)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    x = torch.randn(rows, d, device=DEV).to(dt).float().requires_grad_(True)
     y_ref = x / (x.norm(dim=-1, keepdim=True) + 1e-6)
-    dy = torch.randn_like(x)
+    dy = torch.randn(rows, d, device=DEV).to(dt).float()
     y_ref.backward(dy)
-    assert torch.allclose(la.l2norm_rows(x.detach()), y_ref, atol=1e-6)
-    assert torch.allclose(_l2norm_rows_bwd(x.detach(), dy), x.grad, atol=1e-5)
+    tol = 1e-2 if bf16 else 1e-5
+    y = la.l2norm_rows(x.detach().to(dt))
+    dx = _l2norm_rows_bwd(x.detach().to(dt), dy.to(dt))
+    assert y.shape == (rows, d) and y.dtype == dt
+    assert torch.allclose(y.float(), y_ref, atol=tol) and torch.allclose(dx.float(), x.grad, atol=tol * 4)
