@@ -51,7 +51,9 @@ typedef struct lnx_scan_args {
   float scale;              /* multiplies q (after normalisation) */
   int32_t forward_only;     /* lnx_chunk_fwd: no backward pass will follow, do not write the per-chunk tensors
                                only lnx_chunk_bwd reads (inference / prefill); the workspace is still needed */
-  int32_t reserved;         /* must be 0 */
+  int32_t token_first;      /* 0: q, k, v, o, beta, g and their gradients are [B,H,T,.] (the reference's layout);
+                               1: they are [B,T,H,.] (what the reference's blocks hold before they transpose,
+                               delta_net.py:645-647) -- packed batches [1,T,H,.]; states are [B,H,dk,dv] either way */
 
   const void* q;
   const void* k;

@@ -27,7 +27,7 @@ class ScanArgs(C.Structure):
         ("B", C.c_int32), ("H", C.c_int32), ("T", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32),
         ("chunk", C.c_int32), ("dtype", C.c_int32), ("o_dtype", C.c_int32), ("gate", C.c_int32),
         ("use_qk_l2norm", C.c_int32), ("nseq", C.c_int32), ("scale", C.c_float),
-        ("forward_only", C.c_int32), ("reserved", C.c_int32),
+        ("forward_only", C.c_int32), ("token_first", C.c_int32),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("beta", C.c_void_p), ("g", C.c_void_p),
         ("initial_state", C.c_void_p), ("cu_seqlens", C.c_void_p), ("o", C.c_void_p),
         ("final_state", C.c_void_p),

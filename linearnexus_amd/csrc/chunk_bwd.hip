@@ -57,11 +57,11 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
   if (v0 == 0 && tid < 64 && p.gate == LNX_GATE_SCALAR) wsp<float>(p, p.off.dG)[slot * 64 + tid] = 0.f;  // accumulated by bwd_dqk
   TileRegs<T, 64, 64> rP, rdO;
   rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
-  rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
+  rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, tid);
   rP.store(sP, LDC, tid);
   rdO.store(sdO, LDC, tid);
   lds_barrier();
@@ -147,17 +147,18 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0, len;
       chunk_span(p.geom, n, tok0, len);
-      const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+      const int64_t tbase = tok_index(p.geom, row, tok0);
+      const int64_t tsk = (int64_t)p.geom.ts * DK;
       // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)
       if (GATE == LNX_GATE_VECTOR) {
         R.K.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
         R.Q.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
       } else {
-        R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, len, mt);
-        R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, len, mt);
+        R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
+        R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, mt);
       }
       R.W.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
-      R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, mt);
+      R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
       if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
 #pragma unroll
@@ -347,7 +348,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;  // row strides of the token tiles
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK + ch0;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK + ch0;
   const int wi = wave >> 1, wj = wave & 1;
@@ -364,7 +366,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   TileRegs<T, 64, SV> rdO, rD, rdD;
   TileRegs<T, SV, 64> rSn, rdSn;  // S_n and dS_n slabs stay [v][c]: contracted along their rows
   auto fetch = [&](int v0) {
-    rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, p.dv, len, tid);
+    rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, tsv, len, tid);
     rD.load(wsp<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
     rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
@@ -418,8 +420,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK + ch0;
     float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK + ch0;
     TileRegs<T, 64, 64> rk, rq;
-    rk.load(kg, DK, len, tid);
-    rq.load(qg, DK, len, tid);
+    rk.load(kg, tsk, len, tid);
+    rq.load(qg, tsk, len, tid);
     // dW half through sOut (fp32) -> global
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -455,7 +457,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     for (int idx = tid; idx < 64 * 16; idx += 256) {
       const int r = idx >> 4, c = (idx & 15) * 4;
       const floatx4 v = load4(sOut + r * LDF + c), qq = load4(sQr + r * LDC + c);
-      if (r < len) store4(dqg + (int64_t)r * DK + c, v);
+      if (r < len) store4(dqg + (int64_t)r * tsk + c, v);
       store4(dGg + r * DK + c, qq * v);
     }
     lds_barrier();
@@ -479,7 +481,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     for (int idx = tid; idx < 64 * 16; idx += 256) {
       const int r = idx >> 4, c = (idx & 15) * 4;
       const floatx4 v = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
-      if (r < len) store4(dkg + (int64_t)r * DK + c, v);
+      if (r < len) store4(dkg + (int64_t)r * tsk + c, v);
       floatx4 dgv = load4(dGg + r * DK + c) - kk * v;  // written above by this same thread
       if (r == 63) dgv += load4(sSS + c);
       store4(dGg + r * DK + c, dgv);
@@ -492,8 +494,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     T* sQr = sSn;     // Q rows
     T* sOut = sdSn;
     TileRegs<T, 64, 64> rKT, rQT;
-    rKT.load(kg, DK, len, tid);
-    rQT.load(qg, DK, len, tid);
+    rKT.load(kg, tsk, len, tid);
+    rQT.load(qg, tsk, len, tid);
     {
       floatx16 pe[1][1], nw[1][1];
 #pragma unroll
@@ -533,8 +535,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     frag_store<T, 1, 1>(aQ, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
     frag_store<T, 1, 1>(aK, sOut2 + 32 * wi * LDC + 32 * wj, LDC, lane);
     lds_barrier();
-    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, DK, sPe, LDC, len, tid);
-    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, DK, sOut2, LDC, len, tid);
+    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dq) + tbase * DK + ch0, tsk, sPe, LDC, len, tid);
+    unstage_tile<T, 64, 64>(reinterpret_cast<T*>(p.dk) + tbase * DK + ch0, tsk, sOut2, LDC, len, tid);
     if (GATE != LNX_GATE_NONE) {
       // d/dG_i = <q_i, dq_i> - <k_i, dk_i> over this half's channels (dk = its column-type parts), from the
       // staged tiles; thread = (row, quarter of the channels)
@@ -601,7 +603,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t ts = p.geom.ts, tsk = ts * DK, tsv = ts * p.dv;  // token stride, row strides of the token tiles
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
   const int wi = wave >> 1, wj = wave & 1;
@@ -609,7 +612,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 
   if (tid < 64) {
     sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+    sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
     sdB[tid] = 0.f;
     sdGk[tid] = 0.f;
     sRow[tid] = 0.f;
@@ -623,12 +626,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
       const int c0 = 64 * s_;
       rIn.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
       rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
-      rKs.load(kg + c0, DK, len, tid);
+      rKs.load(kg + c0, tsk, len, tid);
     } else {
       const int v0 = 64 * (s_ - NKS);
       rIn.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-      rKs.load(vg + v0, p.dv, len, tid);
+      rKs.load(vg + v0, tsv, len, tid);
     }
   };
   floatx16 aBw[NKS][1][1], aM[1][1], aX[1][1];
@@ -685,7 +688,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
           typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBt + r * LDC + c);
 #pragma unroll
           for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * sBeta[r]);
-          *reinterpret_cast<typename Vec16<T>::V*>(dvg + (int64_t)r * p.dv + c) = x;
+          *reinterpret_cast<typename Vec16<T>::V*>(dvg + (int64_t)r * tsv + c) = x;
         }
       }
     }
@@ -729,10 +732,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
       for (int it = 0; it < 4; ++it) {  // all global reads of the half first
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         up[it] = load4(Gg + r * DK + ch0 + c);
-        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * DK + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * tsk + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
         dg0[it] = load4(dGg + r * DK + ch0 + c);
       }
-      stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, DK, len, tid);
+      stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, tsk, len, tid);
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
@@ -779,12 +782,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
       for (int it = 0; it < 4; ++it) {
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         const floatx4 um = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
-        if (r < len) store4(dkg + (int64_t)r * DK + ch0 + c, dk0[it] + up[it] + um);
+        if (r < len) store4(dkg + (int64_t)r * tsk + ch0 + c, dk0[it] + up[it] + um);
         store4(dGg + r * DK + ch0 + c, dg0[it] + kk * (up[it] - um));
       }
     }
     __syncthreads();  // dG is read back below by other threads than wrote it: global memory must be ordered too
-    if (tid < 64 && tid < len) p.dbeta[tbase + tid] = sdB[tid];
+    if (tid < 64 && tid < len) p.dbeta[tbase + tid * ts] = sdB[tid];
     if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
       float gv[64];
 #pragma unroll
@@ -793,7 +796,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 #pragma unroll
       for (int r = 63; r >= 0; --r) {
         acc += gv[r];
-        if (r < len) p.dg[(tbase + r) * DK + tid] = acc;
+        if (r < len) p.dg[(tbase + r * ts) * DK + tid] = acc;
       }
     }
     return;
@@ -802,8 +805,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
 #pragma unroll
   for (int u = 0; u < NKS; ++u) {
-    rKT[u].load(kg + 64 * u, DK, len, tid);  // K rows again, for Y K
-    rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, DK, len, tid);
+    rKT[u].load(kg + 64 * u, tsk, len, tid);  // K rows again, for Y K
+    rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);
   }
   lds_barrier();  // loop tiles dead
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
@@ -854,7 +857,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
           typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBt + r * LDC + c);
 #pragma unroll
           for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) + to_f32(rdk[u].x[it][e]));
-          *reinterpret_cast<typename Vec16<T>::V*>(dkg + (int64_t)r * DK + c) = x;
+          *reinterpret_cast<typename Vec16<T>::V*>(dkg + (int64_t)r * tsk + c) = x;
         }
       }
     }
@@ -864,7 +867,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     const int t = lane;
     const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[t]);
     const float w = gm * sdGk[t], rs = sRow[t];
-    if (t < len) p.dbeta[tbase + t] = sdB[t] + w + rs;
+    if (t < len) p.dbeta[tbase + t * ts] = sdB[t] + w + rs;
     if (GATE != LNX_GATE_NONE) {
       float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - sCol[t];
 #pragma unroll
@@ -872,7 +875,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
         const float y = __shfl_down(d, s_, LNX_WAVE);
         if (t + s_ < 64) d += y;
       }
-      if (t < len) p.dg[tbase + t] = d;
+      if (t < len) p.dg[tbase + t * ts] = d;
     }
   }
 }
@@ -946,6 +949,7 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
                          (unsigned long long)a->workspace_bytes);
   BwdParams p;
   p.geom.H = a->H; p.geom.T = a->T; p.geom.N = lnx_chunk_slots(a); p.geom.nseq = a->nseq;
+  p.geom.ts = a->token_first ? a->H : 1;
   p.geom.rows = packed ? a->H : a->B * a->H;
   p.geom.cu = a->cu_seqlens;
   p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;

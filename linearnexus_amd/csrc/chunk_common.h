@@ -28,6 +28,7 @@
 
 struct ChunkGeom {
   int H, T, N, nseq, rows;       // rows = B * H (dense) or H (packed); N = chunk slots per row
+  int ts;                        // distance between consecutive tokens of a row, in tokens: 1 ([B,H,T,.]) or H ([B,T,H,.])
   const int32_t* cu;             // device cu_seqlens or nullptr
   const int32_t* tab;            // packed only: [N][2] (token0, len), seq_chunk0[nseq + 1], order[nseq]
 };
@@ -40,6 +41,12 @@ __device__ __forceinline__ void chunk_span(const ChunkGeom& g, int n, int& tok0,
     tok0 = n * LNX_C;
     len = min(LNX_C, g.T - tok0);
   }
+}
+
+// Position of token `tok` of (batch, head) row `row` in units of one token's vector (dk or dv elements, or one
+// scalar for beta / g); token tok + 1 of the same row is g.ts further on.
+__device__ __forceinline__ int64_t tok_index(const ChunkGeom& g, int row, int tok) {
+  return g.ts == 1 ? (int64_t)row * g.T + tok : ((int64_t)(row / g.H) * g.T + tok) * g.H + row % g.H;
 }
 
 // The sequential kernels take one workgroup per (state, head): blockIdx.x -> state index and row.

@@ -86,20 +86,21 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;  // row strides of the token tiles
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
   const int wi = wave >> 1, wj = wave & 1;
 
   TileRegs<T, 64, 64> rK, rQ;
-  rK.load(kg, DK, len, tid);
-  rQ.load(qg, DK, len, tid);
+  rK.load(kg, tsk, len, tid);
+  rQ.load(qg, tsk, len, tid);
   if (wave == 0) {
     const bool ok = lane < len;
-    sBeta[lane] = ok ? p.beta[tbase + lane] : 0.f;
+    sBeta[lane] = ok ? p.beta[tbase + (int64_t)lane * p.geom.ts] : 0.f;
     float gv = 0.f;
-    if (GATE == LNX_GATE_SCALAR && ok) gv = p.g[tbase + lane];
+    if (GATE == LNX_GATE_SCALAR && ok) gv = p.g[tbase + (int64_t)lane * p.geom.ts];
     gv = wave_cumsum(gv, lane);
     sG[lane] = gv;
     ws_ptr<float>(p, p.off.G)[slot * 64 + lane] = gv;
@@ -114,8 +115,8 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     rQ.store(sQa, LDC, tid);
     lds_barrier();
     if (s_ + 1 < NKS) {
-      rK.load(kg + 64 * (s_ + 1), DK, len, tid);
-      rQ.load(qg + 64 * (s_ + 1), DK, len, tid);
+      rK.load(kg + 64 * (s_ + 1), tsk, len, tid);
+      rQ.load(qg + 64 * (s_ + 1), tsk, len, tid);
     }
     if (!(wi == 0 && wj == 1)) {
       mma_nt<T, 1, 1>(ax, sKa + 32 * wi * LDC, LDC, sKa + 32 * wj * LDC, LDC, 64, lane);
@@ -125,8 +126,8 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   // first slab of the second loop, in flight during the inverse
   TileRegs<T, 64, 64> rIn;
   auto fetch = [&](int s_) {
-    if (s_ < NKS) rIn.load(kg + 64 * s_, DK, len, tid);
-    else rIn.load(vg + 64 * (s_ - NKS), p.dv, len, tid);
+    if (s_ < NKS) rIn.load(kg + 64 * s_, tsk, len, tid);
+    else rIn.load(vg + 64 * (s_ - NKS), tsv, len, tid);
   };
   fetch(0);
   lds_barrier();  // slab tiles dead
@@ -228,7 +229,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;  // row strides of the token tiles
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
@@ -239,12 +241,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   TileRegs<T, 64, 64> rK, rQ;
   TileRegs<float, 64, 64> rG;
   auto fetch_half = [&](int h) {
-    rK.load(kg + 64 * h, DK, len, tid);
-    rQ.load(qg + 64 * h, DK, len, tid);
-    rG.load(p.g + tbase * DK + 64 * h, DK, len, tid);
+    rK.load(kg + 64 * h, tsk, len, tid);
+    rQ.load(qg + 64 * h, tsk, len, tid);
+    rG.load(p.g + tbase * DK + 64 * h, tsk, len, tid);
   };
   fetch_half(0);
-  if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + tid] : 0.f;
+  if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + (int64_t)tid * p.geom.ts] : 0.f;
   floatx4 acc[3];  // this wave's three below-diagonal tasks (block, product), summed over the halves
 #pragma unroll
   for (int u = 0; u < 3; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -402,7 +404,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   floatx4 rGs[Slab::IT][VN / 4];  // K slabs: the gate values of exactly the elements this thread holds
   auto fetch_slab = [&](int s_) {
     if (s_ < NH) {
-      rIn.load(kg + 64 * s_, DK, len, tid);
+      rIn.load(kg + 64 * s_, tsk, len, tid);
 #pragma unroll
       for (int it = 0; it < Slab::IT; ++it) {
         const int idx = tid + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * VN;
@@ -410,7 +412,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         for (int j = 0; j < VN / 4; ++j) rGs[it][j] = load4(Gg + r * DK + 64 * s_ + c + 4 * j);
       }
     } else {
-      rIn.load(vg + 64 * (s_ - NH), p.dv, len, tid);
+      rIn.load(vg + 64 * (s_ - NH), tsv, len, tid);
     }
   };
   __syncthreads();  // G is read back from the workspace by other threads than wrote it: global memory must be ordered too
@@ -529,14 +531,15 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
     auto fetch = [&](Tiles& R, int n) {
       const int64_t slot = (int64_t)row * N + n;
       chunk_span(p.geom, n, R.tok0, R.len);
-      const int64_t tbase = (int64_t)row * p.geom.T + R.tok0;
+      const int64_t tbase = tok_index(p.geom, row, R.tok0);
+      const int64_t tsk = (int64_t)p.geom.ts * DK;
       R.W.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
       if (GATE == LNX_GATE_VECTOR) R.K.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
-      else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, DK, R.len, mt);
+      else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, R.len, mt);
       R.U.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
       if (FUSE) {
         if (GATE == LNX_GATE_VECTOR) R.Q.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
-        else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, DK, R.len, mt);
+        else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, R.len, mt);
         R.P.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       }
       if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = ws_ptr<float>(p, p.off.G)[slot * 64 + mt];
@@ -565,7 +568,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       lds_barrier();  // B3
       if (n + 1 < c1) commit_rest(nxt);
       if (FUSE && p.o_dtype == LNX_BF16)
-        unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + ((int64_t)row * p.geom.T + tok0) * p.dv + v0, p.dv, sO, LDO, len, mt);
+        unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
+                                     (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
@@ -649,8 +653,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
       } else {
         const int tok0 = sMeta[0], len = sMeta[1];
-        frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + ((int64_t)row * p.geom.T + tok0 + 32 * wi) * p.dv + v0 + 32 * wj,
-                                p.dv, lane, len - 32 * wi);
+        frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + (tok_index(p.geom, row, tok0) + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj,
+                                (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
       }
     }
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
@@ -713,7 +717,8 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
-  const int64_t tbase = (int64_t)row * p.geom.T + tok0;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;
 
   if (GATE == LNX_GATE_VECTOR) {
     constexpr int VN = Vec16<T>::N;
@@ -723,14 +728,14 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
       const int r = idx / (DK / VN), c = (idx % (DK / VN)) * VN;
       typename Vec16<T>::V x = vec_zero<T>();
       if (r < len) {
-        x = *reinterpret_cast<const typename Vec16<T>::V*>(qg + (int64_t)r * DK + c);
+        x = *reinterpret_cast<const typename Vec16<T>::V*>(qg + (int64_t)r * tsk + c);
 #pragma unroll
         for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) * p.scale * __expf(Gg[r * DK + c + e]));
       }
       *reinterpret_cast<typename Vec16<T>::V*>(sQ + r * LDK + c) = x;
     }
   } else {
-    stage_tile<T, 64, DK>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, DK, len, tid);
+    stage_tile<T, 64, DK>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, tid);
   }
   stage_tile<T, BV, DK>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, tid);
   stage_tile<T, 64, 64>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
@@ -748,11 +753,11 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
     acc[0][0][e] *= gm;
   }
   mma_x<T, 1, 1, false, true>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj, LDC, 64, lane);
-  const int64_t obase = (tbase + 32 * wi) * p.dv + v0 + 32 * wj;
+  const int64_t obase = (tbase + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj;
   if (p.o_dtype == LNX_BF16)
-    frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, p.dv, lane, len - 32 * wi);
+    frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, tsv, lane, len - 32 * wi);
   else
-    frag_store<float, 1, 1>(acc, reinterpret_cast<float*>(p.o) + obase, p.dv, lane, len - 32 * wi);
+    frag_store<float, 1, 1>(acc, reinterpret_cast<float*>(p.o) + obase, tsv, lane, len - 32 * wi);
 }
 
 // state-only path for T == 0: final = initial (or zeros)
@@ -860,7 +865,7 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
   if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);
   if (a->use_qk_l2norm) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take pre-normalised q, k (use lnx_l2norm_fwd)");
-  if (a->reserved != 0) return lnx_set_error(LNX_ERR_SHAPE, "reserved field must be 0");
+  if (a->token_first != 0 && a->token_first != 1) return lnx_set_error(LNX_ERR_SHAPE, "token_first must be 0 or 1");
   if (backward && a->forward_only) return lnx_set_error(LNX_ERR_SHAPE, "forward_only is set: the workspace holds nothing for a backward pass");
   if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
     return lnx_set_error(LNX_ERR_SHAPE, "packed batches need B == 1 and nseq > 0 (B=%d nseq=%d)", a->B, a->nseq);
@@ -901,6 +906,7 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   lnx_chunk_build_table(a, w, st);
   FwdParams p;
   p.geom.H = a->H; p.geom.T = a->T; p.geom.N = lnx_chunk_slots(a); p.geom.nseq = a->nseq;
+  p.geom.ts = a->token_first ? a->H : 1;
   p.geom.rows = packed ? a->H : a->B * a->H;
   p.geom.cu = a->cu_seqlens;
   p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;

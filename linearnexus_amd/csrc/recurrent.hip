@@ -24,6 +24,7 @@ struct TokenParams {
   void* o;
   const int32_t* cu_seqlens;
   int H, T, dv;
+  int ts;  // distance between consecutive tokens of a (batch, head) row, in tokens: 1 ([B,H,T,.]) or H ([B,T,H,.])
   float scale;
   int l2norm;
   int o_dtype;
@@ -172,24 +173,26 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(TokenParams p) {
     if (p.s_in && active) S[i] = load4(p.s_in + sbase + (int64_t)i * p.dv);
     else S[i] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-  const T* qb = reinterpret_cast<const T*>(p.q) + bh * p.T * DK;
-  const T* kb = reinterpret_cast<const T*>(p.k) + bh * p.T * DK;
-  const T* vb = reinterpret_cast<const T*>(p.v) + bh * p.T * p.dv + ccol;
-  const float* betab = p.beta + bh * p.T;
+  // position of token 0 of this row in units of one token's vector; token t is t * ts further on
+  const int64_t ts = p.ts, tok0 = (ts == 1) ? bh * p.T : (bh / p.H) * p.T * p.H + bh % p.H;
+  const T* qb = reinterpret_cast<const T*>(p.q) + tok0 * DK;
+  const T* kb = reinterpret_cast<const T*>(p.k) + tok0 * DK;
+  const T* vb = reinterpret_cast<const T*>(p.v) + tok0 * p.dv + ccol;
+  const float* betab = p.beta + tok0;
   const float* gb = nullptr;
-  if (GATE == LNX_GATE_SCALAR) gb = p.g + bh * p.T;
-  if (GATE == LNX_GATE_VECTOR) gb = p.g + bh * p.T * DK;
+  if (GATE == LNX_GATE_SCALAR) gb = p.g + tok0;
+  if (GATE == LNX_GATE_VECTOR) gb = p.g + tok0 * DK;
   for (int t = t0; t < t1; ++t) {
-    const float* gp = (GATE == LNX_GATE_VECTOR) ? gb + (int64_t)t * DK : nullptr;
-    const floatx4 v4 = load4(vb + (int64_t)t * p.dv);
-    const float beta = betab[t];
-    const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(gb[t]) : 1.f;
+    const int64_t tt = t * ts;
+    const float* gp = (GATE == LNX_GATE_VECTOR) ? gb + tt * DK : nullptr;
+    const floatx4 v4 = load4(vb + tt * p.dv);
+    const float beta = betab[tt];
+    const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(gb[tt]) : 1.f;
     __syncthreads();  // previous token's reads of sm are done
-    const float qk = stage_qk<T, DK, GATE>(qb + (int64_t)t * DK, kb + (int64_t)t * DK, gp, sm, lane, p.scale,
-                                           p.l2norm);
+    const float qk = stage_qk<T, DK, GATE>(qb + tt * DK, kb + tt * DK, gp, sm, lane, p.scale, p.l2norm);
     __syncthreads();
     const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, beta, v4, qk);
-    if ((lane >> 3) == 0 && active) store_o4(p.o, (bh * p.T + t) * p.dv + col0, o4, p.o_dtype);
+    if ((lane >> 3) == 0 && active) store_o4(p.o, (tok0 + tt) * p.dv + col0, o4, p.o_dtype);
   }
   if (active) {
 #pragma unroll
@@ -248,7 +251,7 @@ int token_entry(bool decode, const lnx_scan_args* a, void* stream) {
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.g = a->g;
   p.s_in = a->initial_state; p.s_out = a->final_state; p.o = a->o;
   p.cu_seqlens = packed ? a->cu_seqlens : nullptr;
-  p.H = a->H; p.T = a->T; p.dv = a->dv; p.scale = a->scale; p.l2norm = a->use_qk_l2norm; p.o_dtype = a->o_dtype;
+  p.H = a->H; p.T = a->T; p.dv = a->dv; p.ts = (!decode && a->token_first) ? a->H : 1; p.scale = a->scale; p.l2norm = a->use_qk_l2norm; p.o_dtype = a->o_dtype;
   dim3 grid((unsigned)(nstate * a->H), (unsigned)((a->dv + (decode ? 127 : 31)) / (decode ? 128 : 32)));
   hipStream_t st = (hipStream_t)stream;
   lnx_profile_mark(decode ? "decode_step" : "recurrent_fwd", st);

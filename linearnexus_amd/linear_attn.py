@@ -57,6 +57,39 @@ def _f32(t: Tensor) -> Tensor:
     return t.to(torch.float32).contiguous()
 
 
+# Memory layout of the token tensors.  The ops take the reference's head-first [B, H, T, .] shapes; a caller
+# whose data lives token-first -- [B, T, H, .], what the reference's blocks hold before they transpose
+# (delta_net.py:645-647) -- passes ``x.transpose(1, 2)`` views, and the kernels then read and write that
+# memory in place (``token_first`` in the argument block) instead of working on contiguous copies.
+
+def _is_token_first(x: Tensor) -> bool:
+    return x.dim() >= 3 and not x.is_contiguous() and x.transpose(1, 2).is_contiguous()
+
+
+def _as_layout(x: Optional[Tensor], token_first: bool) -> Optional[Tensor]:
+    """``x`` (logical [B, H, T, ...]) with dense memory in the chosen layout; no copy when it already has it."""
+    if x is None:
+        return None
+    if token_first:
+        return x if _is_token_first(x) else x.transpose(1, 2).contiguous().transpose(1, 2)
+    return x.contiguous()
+
+
+def _empty_layout(B, H, T, tail, dtype, device, token_first: bool) -> Tensor:
+    if token_first:
+        return torch.empty((B, T, H) + tuple(tail), dtype=dtype, device=device).transpose(1, 2)
+    return torch.empty((B, H, T) + tuple(tail), dtype=dtype, device=device)
+
+
+def _dense(x: Tensor):
+    """A contiguous tensor over x's memory (or a copy) and the function that maps results back to x's layout."""
+    if x.is_contiguous():
+        return x, (lambda y: y)
+    if _is_token_first(x):
+        return x.transpose(1, 2), (lambda y: y.transpose(1, 2))
+    return x.contiguous(), (lambda y: y)
+
+
 def _squeeze_beta(beta: Tensor, ndim: int) -> Tensor:
     # delta_net.py:166-167, :257-258, :378-379 -- a trailing singleton is accepted
     return beta.squeeze(-1) if beta.dim() == ndim else beta
@@ -194,14 +227,16 @@ def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):
     dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
     if scale is None:
         scale = dk ** -0.5
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    beta = _f32(beta)
-    g = None if g is None else _f32(g)
+    tf = all(_is_token_first(t) for t in (q, k, v))
+    q, k, v = _as_layout(q, tf), _as_layout(k, tf), _as_layout(v, tf)
+    beta = _as_layout(beta.to(torch.float32), tf)
+    g = None if g is None else _as_layout(g.to(torch.float32), tf)
     s0 = None if initial_state is None else _f32(initial_state)
-    o = torch.empty(B, H, T, dv, dtype=q.dtype, device=q.device)
+    o = _empty_layout(B, H, T, (dv,), q.dtype, q.device, tf)
     sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
     a = _base_args(B, H, T, dk, dv, dt, dt, gate, l2norm, scale)
     a.nseq = nseq
+    a.token_first = int(tf)
     a.q, a.k, a.v, a.beta, a.g = _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(g)
     a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
     lib = _lib.load()
@@ -231,20 +266,22 @@ def kda_recurrent(q, k, v, g, beta, scale=None, initial_state=None, use_qk_l2nor
 
 def l2norm_rows(x: Tensor) -> Tensor:
     """``x / (|x|_2 + 1e-6)`` over the last dimension, in x's dtype (gated_deltanet.py:273-275)."""
-    x = x.contiguous()
+    x, back = _dense(x)
     y = torch.empty_like(x)
     d = x.shape[-1]
     _lib.check(_lib.load().lnx_l2norm_fwd(_ptr(x), _ptr(y), x.numel() // d, d, _DT[x.dtype], _stream(x)), "lnx_l2norm_fwd")
-    return y
+    return back(y)
 
 
 def _l2norm_rows_bwd(x: Tensor, dy: Tensor) -> Tensor:
-    x, dy = x.contiguous(), dy.contiguous()
+    x, back = _dense(x)
+    dy = back(dy)  # same logical shape; bring it to x's dense memory order (back is its own inverse)
+    dy = dy if dy.is_contiguous() else dy.contiguous()
     dx = torch.empty_like(x)
     d = x.shape[-1]
     _lib.check(_lib.load().lnx_l2norm_bwd(_ptr(x), _ptr(dy), _ptr(dx), x.numel() // d, d, _DT[x.dtype], _stream(x)),
                "lnx_l2norm_bwd")
-    return dx
+    return back(dx)
 
 
 class _ChunkScan(torch.autograd.Function):
@@ -253,19 +290,21 @@ class _ChunkScan(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens):
         dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
-        q_in, k_in = q.contiguous(), k.contiguous()
+        tf = all(_is_token_first(t) for t in (q, k, v))  # [B,T,H,.] memory behind transposed views: used in place
+        q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
         # the reference's chunk path normalises in the input dtype before anything else
         # (gated_deltanet.py:273-275, kda.py:379-381)
         qn = l2norm_rows(q_in) if l2norm else q_in
         kn = l2norm_rows(k_in) if l2norm else k_in
-        v = v.contiguous()
-        beta_f = _f32(beta)
-        g_f = None if g is None else _f32(g)
+        v = _as_layout(v, tf)
+        beta_f = _as_layout(beta.to(torch.float32), tf)
+        g_f = None if g is None else _as_layout(g.to(torch.float32), tf)
         s0 = None if initial_state is None else _f32(initial_state)
-        o = torch.empty(B, H, T, dv, dtype=o_dtype, device=q.device)
+        o = _empty_layout(B, H, T, (dv,), o_dtype, q.device, tf)
         sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
         a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
         a.nseq = nseq
+        a.token_first = int(tf)
         # nothing to differentiate (inference, torch.no_grad()): the kernels skip what only the backward reads
         a.forward_only = int(not any(ctx.needs_input_grad))
         a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
@@ -279,15 +318,16 @@ class _ChunkScan(torch.autograd.Function):
         _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
         ctx.save_for_backward(q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
         ctx.meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
-                    None if g is None else g.dtype, initial_state is not None)
+                    None if g is None else g.dtype, initial_state is not None, tf)
         return o, sT
 
     @staticmethod
     def backward(ctx, d_o, d_sT):
         q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws = ctx.saved_tensors
-        dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0 = ctx.meta
+        dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0, tf = ctx.meta
         dev = qn.device
-        d_o = torch.zeros(B, H, T, dv, dtype=qn.dtype, device=dev) if d_o is None else d_o.to(qn.dtype).contiguous()
+        d_o = torch.zeros(B, H, T, dv, dtype=qn.dtype, device=dev) if d_o is None else d_o.to(qn.dtype)
+        d_o = _as_layout(d_o, tf)
         d_sT = None if d_sT is None else _f32(d_sT)
         dq, dk_, dv_ = torch.empty_like(qn), torch.empty_like(kn), torch.empty_like(v)
         dbeta = torch.empty_like(beta_f)
@@ -296,6 +336,7 @@ class _ChunkScan(torch.autograd.Function):
         ds0 = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=dev) if has_s0 else None
         a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
         a.nseq = nseq
+        a.token_first = int(tf)
         a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
         a.initial_state, a.cu_seqlens = _ptr(s0), _ptr(cu)
         a.d_o, a.d_final_state = _ptr(d_o), _ptr(d_sT)

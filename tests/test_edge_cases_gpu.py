@@ -168,3 +168,62 @@ def test_both_slab_widths_of_the_sequential_kernels(gate, slab, monkeypatch):
     xb, dt = _prep_bwd(x, True)
     ref = delta_rule_adjoint(xb["q"], xb["k"], xb["v"], xb["beta"], xb["dO"], xb.get("g"), xb["dS"], None, xb["S0"], False)
     check(gpu_grads(xb, gate, dt), ref, 2e-2)
+
+
+def _tf(x):
+    """The same logical [B, H, T, ...] tensor on [B, T, H, ...] memory."""
+    return x.transpose(1, 2).contiguous().transpose(1, 2)
+
+
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("packed", [False, True])
+def test_token_first_memory_is_used_in_place(gate, bf16, packed):
+    """Transposed views of [B, T, H, .] tensors (the layout the reference's blocks hold, delta_net.py:645-647)
+    go to the kernels without copies (token_first = 1); outputs and gradients come back on the same kind of
+    memory and are bit-identical to the head-first call."""
+    import linearnexus_amd as la
+    B, H, T, d = (1, 3, 200, 128) if packed else (2, 3, 150, 128)
+    x = make_inputs(68, B, H, T, d, d, gate=gate, with_grad=True)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    cu = torch.tensor([0, 70, 71, 200], dtype=torch.int32, device=DEV) if packed else None
+    nstate = 3 if packed else B
+    S0 = torch.randn(nstate, H, d, d, device=DEV) * 0.02
+    dS = torch.randn(nstate, H, d, d, device=DEV) * 0.1
+
+    def run(layout, l2, chunk):
+        leaves = {n: layout(torch.from_numpy(x[n]).to(DEV).to(dt if n in ("q", "k", "v") else torch.float32)).requires_grad_(True)
+                  for n in ("q", "k", "v", "beta") + (("g",) if gate != "none" else ())}
+        s0 = S0.clone().requires_grad_(True)
+        q, k, v, beta = leaves["q"], leaves["k"], leaves["v"], leaves["beta"]
+        if gate == "none":
+            fn = la.delta_rule_chunkwise if chunk else la.delta_rule_recurrent
+            o, S = fn(q, k, v, beta, s0, cu_seqlens=cu)
+        else:
+            fn = {("scalar", True): la.gated_delta_rule_chunkwise, ("scalar", False): la.gated_delta_rule_recurrent,
+                  ("vector", True): la.kda_chunkwise, ("vector", False): la.kda_recurrent}[(gate, chunk)]
+            o, S = fn(q, k, v, leaves["g"], beta, None, s0, use_qk_l2norm=l2, cu_seqlens=cu)
+        grads = None
+        if chunk:
+            dO = layout(torch.from_numpy(x["dO"]).to(DEV).to(o.dtype))
+            ((o * dO).sum() + (S * dS).sum()).backward()
+            grads = {n: t.grad for n, t in leaves.items()}
+            grads["S0"] = s0.grad
+        return o, S, grads
+
+    for l2 in ((False, True) if gate != "none" else (False,)):
+        o1, S1, g1 = run(lambda t: t, l2, True)
+        o2, S2, g2 = run(_tf, l2, True)
+        assert o2.transpose(1, 2).is_contiguous() and (not o2.is_contiguous() or H == 1)
+        assert torch.equal(o1, o2) and torch.equal(S1, S2)
+        for n in g1:
+            if n in ("beta", "g"):  # row sums go through LDS atomics, whose order is not fixed: equal up to fp32 rounding
+                scale_ = float(g1[n].float().abs().max())
+                assert float((g1[n].float() - g2[n].float()).abs().max()) <= 2e-5 * scale_, n
+            else:
+                assert torch.equal(g1[n], g2[n]), n
+        for n in ("q", "k", "v"):
+            assert g2[n].transpose(1, 2).is_contiguous(), n
+    o1, S1, _ = run(lambda t: t, False, False)
+    o2, S2, _ = run(_tf, False, False)
+    assert torch.equal(o1, o2) and torch.equal(S1, S2) and o2.transpose(1, 2).is_contiguous()
