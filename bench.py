@@ -33,9 +33,9 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
 TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 860879916, ("gdn_chunk", "chunk_scan"): 1151569502,
-    ("gdn_chunk", "bwd_scan"): 1019424981, ("gdn_chunk", "bwd_dqk"): 1617043803,
-    ("gdn_chunk", "bwd_wy"): 1485082613, ("decode", "decode_step"): 1083423645,
+    ("gdn_chunk", "chunk_prepare"): 864163746, ("gdn_chunk", "chunk_scan"): 1151594310,
+    ("gdn_chunk", "bwd_scan"): 1019454442, ("gdn_chunk", "bwd_dqk"): 1617029406,
+    ("gdn_chunk", "bwd_wy"): 1601705893, ("decode", "decode_step"): 1083428380,
 }
 
 
