@@ -240,12 +240,37 @@ def bench_decode(args, torch, la, _lib, steps=None):
     }
 
 
+def bench_decode_graph(torch, steps):
+    """Host cost per generated token of a 24-layer Gated DeltaNet decode (B=1 and 8, H=32, d=128): the layers'
+    steps replayed as one captured graph against one eager op call per layer."""
+    from linearnexus_amd.decode import DecodeGraph
+    res = []
+    for B in (1, 8):
+        H, d, L = 32, 128, 24
+        dg = DecodeGraph("gated", B, H, d, d, layers=L)
+        for i in range(L):
+            dg.q[i].normal_(), dg.k[i].normal_(), dg.v[i].normal_(), dg.beta[i].fill_(0.5), dg.g[i].fill_(-0.1)
+        us = {}
+        for name, fn in (("graph", dg.replay), ("eager", dg._run)):
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            us[name] = (time.perf_counter() - t0) / steps * 1e6
+        res.append({"B": B, "H": H, "dk": d, "dv": d, "layers": L, "graph_us_per_token": us["graph"],
+                    "eager_us_per_token": us["eager"]})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -264,6 +289,13 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "decode_graph":
+        res = bench_decode_graph(torch, max(args.steps, 200))
+        print(json.dumps({"metric": "decode host time per token, 24 layers", "value": res[0]["graph_us_per_token"],
+                          "unit": "us/token", "n_gpus": 1, "steps": max(args.steps, 200), "warmup": 10,
+                          "higher_is_better": False, "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                          "config": {"workload": "gated_deltanet_decode_graph"}, "cases": res}))
+        return
     if args.workload == "decode":
         dec = bench_decode(args, torch, la, _lib, steps=max(args.steps, 100))
         out = {"metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
