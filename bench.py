@@ -240,6 +240,46 @@ def bench_decode(args, torch, la, _lib, steps=None):
     }
 
 
+def bench_conv(torch, la, _lib, steps, warmup):
+    """Causal depthwise conv (K=4) + SiLU over the q|k|v projections of config 2's layer: [B8, T4096, D6144] bf16,
+    forward + backward.  Algorithmic bytes: x in, y out; x, dy in, dx out (weights are 100 KB)."""
+    B, T, D, K = 8, 4096, 6144, 4
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    x = torch.randn(B, T, D, generator=gen).to("cuda:0").bfloat16().requires_grad_(True)
+    dy = torch.randn(B, T, D, generator=gen).to("cuda:0").bfloat16()
+    w = (torch.randn(K, D, generator=gen) * 0.3).to("cuda:0").requires_grad_(True)
+
+    def step():
+        x.grad = w.grad = None
+        y, _ = la.depthwise_conv1d_causal(x, w, None, activation="silu")
+        y.backward(dy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    marks = _lib.profile_read()
+    _lib.profile_enable(False)
+    avg = {n: sum(ms for m, ms in marks if m == n) / max(1, sum(1 for m, _ in marks if m == n)) for n in ("conv1d_fwd", "conv1d_bwd")}
+    nb = {"conv1d_fwd": 2 * B * T * D * 2, "conv1d_bwd": 3 * B * T * D * 2}
+    dom = "conv1d_bwd"
+    ach = nb[dom] / (avg[dom] * 1e-3) / 1e9
+    return {"metric": "causal depthwise conv + SiLU fwd+bwd tokens/s", "value": B * T / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "conv1d_silu_fwd_bwd", "B": B, "T": T, "D": D, "K": K},
+            "kernel_ms": {n: round(v, 4) for n, v in avg.items()},
+            "roofline": {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": ach / PEAK_HBM, "traffic": None},
+            "roofline_fwd": {"bound": "hbm", "kernel": "conv1d_fwd", "achieved": nb["conv1d_fwd"] / (avg["conv1d_fwd"] * 1e-3) / 1e9,
+                             "peak": PEAK_HBM, "unit": "GB/s", "frac": nb["conv1d_fwd"] / (avg["conv1d_fwd"] * 1e-3) / 1e9 / PEAK_HBM}}
+
+
 def bench_decode_graph(torch, steps):
     """Host cost per generated token of a 24-layer Gated DeltaNet decode (B=1 and 8, H=32, d=128): the layers'
     steps replayed as one captured graph against one eager op call per layer."""
@@ -270,7 +310,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -289,6 +329,9 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "conv":
+        print(json.dumps(bench_conv(torch, la, _lib, args.steps, args.warmup)))
+        return
     if args.workload == "decode_graph":
         res = bench_decode_graph(torch, max(args.steps, 200))
         print(json.dumps({"metric": "decode host time per token, 24 layers", "value": res[0]["graph_us_per_token"],

@@ -126,6 +126,22 @@ int lnx_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_
                    void* hip_stream);
 
 /*
+ * Short causal depthwise convolution over [B, T, D] activations, kernel width K <= 4, with the SiLU the
+ * reference's blocks apply right after it fused in (activation: 0 = none, 1 = SiLU).  Replaces
+ * depthwise_conv1d_causal (linearnexus/core/conv.py:13-68) + jax.nn.silu (gated_deltanet.py:765-779):
+ *   xin = concat(cache, x) along T;  y[t] = act(bias + sum_j weight[j] * xin[t + j]);  new_cache = last K-1 rows of xin.
+ * x, y, dy, dx [B,T,D] and cache, new_cache [B,K-1,D] in `dtype` (D a multiple of 16 bytes of elements);
+ * weight [K,D], bias [D] and their gradients fp32.  bias, cache, new_cache, d_weight, d_bias may be NULL
+ * (cache NULL = zeros).  new_cache may alias cache for T <= 32 (decode).  The backward treats the cache as a
+ * constant and overwrites d_weight / d_bias (it clears them with a fill kernel, then accumulates atomically).
+ */
+int lnx_conv1d_fwd(const void* x, const float* weight, const float* bias, const void* cache, void* y, void* new_cache,
+                   int32_t B, int32_t T, int32_t D, int32_t K, int32_t dtype, int32_t activation, void* hip_stream);
+int lnx_conv1d_bwd(const void* x, const float* weight, const float* bias, const void* cache, const void* dy, void* dx,
+                   float* d_weight, float* d_bias, int32_t B, int32_t T, int32_t D, int32_t K, int32_t dtype,
+                   int32_t activation, void* hip_stream);
+
+/*
  * Optional per-kernel timing for benchmarks (no counterpart in the reference; its micro-benchmark
  * times whole jitted ops, bench_kda_kernels.py:216-249).  While enabled (process-wide),
  * every entry point records HIP events around each kernel it launches, on the caller's stream.

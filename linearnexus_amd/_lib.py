@@ -16,7 +16,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
-    "lnx_profile_enable", "lnx_profile_read",
+    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_profile_enable", "lnx_profile_read",
 )
 
 
@@ -63,6 +63,10 @@ def load() -> C.CDLL:
     lib.lnx_l2norm_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
     lib.lnx_l2norm_bwd.restype = C.c_int
     lib.lnx_l2norm_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p]
+    lib.lnx_conv1d_fwd.restype = C.c_int
+    lib.lnx_conv1d_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int32] * 6 + [C.c_void_p]
+    lib.lnx_conv1d_bwd.restype = C.c_int
+    lib.lnx_conv1d_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int32] * 6 + [C.c_void_p]
     lib.lnx_profile_enable.restype = C.c_int
     lib.lnx_profile_enable.argtypes = [C.c_int]
     lib.lnx_profile_read.restype = C.c_int

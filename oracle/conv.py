@@ -1,0 +1,66 @@
+"""fp64 restatement of the reference's short causal depthwise convolution -- TEST INFRASTRUCTURE ONLY.
+
+Follows linearnexus/core/conv.py:13-68 (``depthwise_conv1d_causal``) and the SiLU the blocks apply to its
+output (gated_deltanet.py:765-779).  Pinned in tests/test_oracle_conv.py by scipy's FIR filter
+(``lfilter`` with the taps reversed), by the step-by-step == whole-sequence property the reference tests
+(tests/test_comprehensive.py:57-83), by a brute-force triple loop, and -- the gradient -- by central finite
+differences and an independent ``torch.nn.functional.conv1d`` + autograd.
+"""
+import numpy as np
+
+
+def silu(z):
+    return z / (1.0 + np.exp(-z))
+
+
+def depthwise_conv1d_causal(inputs, weight, bias=None, cache=None, activation=None):
+    """inputs [B,T,D], weight [K,D], bias [D]|None, cache [B,K-1,D]|None -> (y [B,T,D], new_cache [B,K-1,D]).
+
+    conv.py:56-67: the cache (zeros when absent) is put in front of the inputs, a VALID cross-correlation
+    runs over that, the last T outputs are kept, and the new cache is the last K-1 rows of the
+    concatenation.  conv.py:39-44: a width-1 kernel is the identity (+ bias) with an empty cache."""
+    x = np.asarray(inputs, np.float64)
+    w = np.asarray(weight, np.float64)
+    B, T, D = x.shape
+    K = w.shape[0]
+    if K < 1:
+        raise ValueError("kernel_size must be >= 1")
+    if cache is None:
+        cache = np.zeros((B, K - 1, D))
+    cache = np.asarray(cache, np.float64)
+    if cache.shape != (B, K - 1, D):
+        raise ValueError(f"cache shape must be (batch, kernel-1, channels); got {cache.shape}")
+    xin = np.concatenate([cache, x], axis=1)
+    z = np.zeros((B, T, D))
+    for j in range(K):
+        z += w[j] * xin[:, j:j + T]
+    if bias is not None:
+        z = z + np.asarray(bias, np.float64)
+    y = silu(z) if activation == "silu" else z
+    return y, xin[:, xin.shape[1] - (K - 1):]
+
+
+def depthwise_conv1d_causal_grad(inputs, weight, bias, dy, cache=None, activation=None):
+    """Gradients of <y, dy> with respect to inputs, weight and bias (the cache is a constant)."""
+    x = np.asarray(inputs, np.float64)
+    w = np.asarray(weight, np.float64)
+    dy = np.asarray(dy, np.float64)
+    B, T, D = x.shape
+    K = w.shape[0]
+    if cache is None:
+        cache = np.zeros((B, K - 1, D))
+    xin = np.concatenate([np.asarray(cache, np.float64), x], axis=1)
+    z = sum(w[j] * xin[:, j:j + T] for j in range(K))
+    if bias is not None:
+        z = z + np.asarray(bias, np.float64)
+    if activation == "silu":
+        s = 1.0 / (1.0 + np.exp(-z))
+        dz = dy * s * (1.0 + z * (1.0 - s))
+    else:
+        dz = dy
+    dxin = np.zeros_like(xin)
+    dw = np.zeros_like(w)
+    for j in range(K):
+        dxin[:, j:j + T] += w[j] * dz
+        dw[j] = (dz * xin[:, j:j + T]).sum((0, 1))
+    return dxin[:, K - 1:], dw, dz.sum((0, 1))
