@@ -280,6 +280,37 @@ def bench_conv(torch, la, _lib, steps, warmup):
                              "peak": PEAK_HBM, "unit": "GB/s", "frac": nb["conv1d_fwd"] / (avg["conv1d_fwd"] * 1e-3) / 1e9 / PEAK_HBM}}
 
 
+def bench_dplr_step(torch, la, _lib, steps):
+    """RWKV-7 DPLR decode step at config 4's shape (B=256, H=32, dk=dv=128), fp32 state updated in place.
+    Algorithmic bytes: the state read and written once, five bf16 dk-vectors, gk fp32, v in, o out."""
+    B, H, d = 256, 32, 128
+    gen = torch.Generator(device="cpu").manual_seed(7)
+    rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    S = (rn(B, H, d, d) * 0.02).to("cuda:0")
+    q, k, v = (rn(B, H, d).to("cuda:0").bfloat16() for _ in range(3))
+    a, b = ((rn(B, H, d) * 0.1).to("cuda:0").bfloat16() for _ in range(2))
+    gk = (-rn(B, H, d).abs() * 0.1).to("cuda:0")
+    for _ in range(20):
+        la.dplr_delta_rule_step(q, k, v, a, b, gk, S, inplace=True)
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        la.dplr_delta_rule_step(q, k, v, a, b, gk, S, inplace=True)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    kern = [ms for _, ms in _lib.profile_read()]
+    _lib.profile_enable(False)
+    nbytes = 2 * S.numel() * 4 + 6 * B * H * d * 2 + B * H * d * 4
+    kms = sum(kern) / len(kern)
+    ach = nbytes / (kms * 1e-3) / 1e9
+    return {"metric": "DPLR decode-step HBM GB/s", "value": ach, "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": 20,
+            "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic", "config": {"workload": "rwkv7_dplr_decode_step", "B": B, "H": H, "dk": d, "dv": d},
+            "roofline": {"bound": "hbm", "kernel": "dplr_step", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": ach / PEAK_HBM, "traffic": None}}
+
+
 def bench_decode_graph(torch, steps):
     """Host cost per generated token of a 24-layer Gated DeltaNet decode (B=1 and 8, H=32, d=128): the layers'
     steps replayed as one captured graph against one eager op call per layer."""
@@ -310,7 +341,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -329,6 +360,9 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "dplr_decode":
+        print(json.dumps(bench_dplr_step(torch, la, _lib, max(args.steps, 500))))
+        return
     if args.workload == "conv":
         print(json.dumps(bench_conv(torch, la, _lib, args.steps, args.warmup)))
         return

@@ -142,6 +142,32 @@ int lnx_conv1d_bwd(const void* x, const float* weight, const float* bias, const 
                    int32_t activation, void* hip_stream);
 
 /*
+ * RWKV-7's diagonal-plus-low-rank delta rule (linearnexus/modules/linear_attn/rwkv7.py:114-265), the sibling
+ * recurrence of the delta rule:  u = h^T a;  h <- exp(gk) (.) h + b u^T + k v^T;  o = h^T (scale * q).
+ * q, k, a, b [B,H,T,dk] and v, o [B,H,T,dv] in `dtype` / `o_dtype`; gk [B,H,T,dk] and the states [B,H,dk,dv] fp32.
+ * lnx_dplr_recurrent_fwd replaces dplr_delta_rule_recurrent (rwkv7.py:114-213; initial_state NULL = zeros),
+ * lnx_dplr_step replaces dplr_delta_rule_step (rwkv7.py:216-265; token tensors [B,H,d], T ignored, the state is
+ * updated in place when final_state == initial_state).  dk in {8,16,32,64,128}, dv a multiple of 4.
+ */
+typedef struct lnx_dplr_args {
+  int32_t B, H, T, dk, dv;
+  int32_t dtype;            /* lnx_dtype of q, k, v, a, b */
+  int32_t o_dtype;          /* lnx_dtype of o */
+  float scale;              /* multiplies q */
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* a;
+  const void* b;
+  const float* gk;
+  const float* initial_state;
+  void* o;
+  float* final_state;
+} lnx_dplr_args;
+int lnx_dplr_recurrent_fwd(const lnx_dplr_args* a, void* hip_stream);
+int lnx_dplr_step(const lnx_dplr_args* a, void* hip_stream);
+
+/*
  * Optional per-kernel timing for benchmarks (no counterpart in the reference; its micro-benchmark
  * times whole jitted ops, bench_kda_kernels.py:216-249).  While enabled (process-wide),
  * every entry point records HIP events around each kernel it launches, on the caller's stream.

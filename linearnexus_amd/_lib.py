@@ -16,7 +16,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
-    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_profile_enable", "lnx_profile_read",
+    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_profile_enable", "lnx_profile_read",
 )
 
 
@@ -34,6 +34,17 @@ class ScanArgs(C.Structure):
         ("d_o", C.c_void_p), ("d_final_state", C.c_void_p), ("d_q", C.c_void_p), ("d_k", C.c_void_p),
         ("d_v", C.c_void_p), ("d_beta", C.c_void_p), ("d_g", C.c_void_p), ("d_initial_state", C.c_void_p),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
+    ]
+
+
+class DplrArgs(C.Structure):
+    """Mirror of ``struct lnx_dplr_args``."""
+
+    _fields_ = [
+        ("B", C.c_int32), ("H", C.c_int32), ("T", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32),
+        ("dtype", C.c_int32), ("o_dtype", C.c_int32), ("scale", C.c_float),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("a", C.c_void_p), ("b", C.c_void_p),
+        ("gk", C.c_void_p), ("initial_state", C.c_void_p), ("o", C.c_void_p), ("final_state", C.c_void_p),
     ]
 
 
@@ -67,6 +78,10 @@ def load() -> C.CDLL:
     lib.lnx_conv1d_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int32] * 6 + [C.c_void_p]
     lib.lnx_conv1d_bwd.restype = C.c_int
     lib.lnx_conv1d_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int32] * 6 + [C.c_void_p]
+    for name in ("lnx_dplr_recurrent_fwd", "lnx_dplr_step"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.POINTER(DplrArgs), C.c_void_p]
     lib.lnx_profile_enable.restype = C.c_int
     lib.lnx_profile_enable.argtypes = [C.c_int]
     lib.lnx_profile_read.restype = C.c_int

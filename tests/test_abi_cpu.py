@@ -47,6 +47,10 @@ def test_argument_validation_without_gpu():
     for fn in (lib.lnx_decode_step, lib.lnx_recurrent_fwd, lib.lnx_chunk_fwd, lib.lnx_chunk_bwd):
         assert fn(a, None) == 0
     assert lib.lnx_l2norm_fwd(None, None, 4, 8, 0, None) == -1
+    d = _lib.DplrArgs()
+    assert lib.lnx_dplr_step(d, None) == -2 and lib.lnx_dplr_recurrent_fwd(d, None) == -2
+    d.B, d.H, d.T, d.dk, d.dv = 1, 1, 1, 64, 64
+    assert lib.lnx_dplr_step(d, None) == -1 and lib.lnx_dplr_recurrent_fwd(d, None) == -1
     assert lib.lnx_conv1d_fwd(None, None, None, None, None, None, 1, 4, 16, 5, 0, 0, None) == -2  # K > 4
     assert lib.lnx_conv1d_fwd(None, None, None, None, None, None, 1, 4, 18, 4, 0, 0, None) == -2  # D % 4
     assert lib.lnx_conv1d_bwd(None, None, None, None, None, None, None, None, 1, 4, 16, 4, 0, 0, None) == -1
