@@ -575,7 +575,9 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   // vector-gate epilogue inside the tile region: G and out [64][LDF] fp32, K rows [64][LDC]
   static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * kTile;
   static_assert(GATE != LNX_GATE_VECTOR || vec_bytes <= sizeof(T) * 5 * kTile, "epilogue tiles overlay the loop tiles");
-  static constexpr size_t bytes = sizeof(T) * 5 * kTile + sizeof(float) * nfloat;
+  // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and (vector gate only) the W/U slab
+  static constexpr int ntile = GATE == LNX_GATE_VECTOR ? 5 : 4;
+  static constexpr size_t bytes = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
 };
 
 template <typename T, int DK, int GATE>
@@ -591,10 +593,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   float* sCol = sRow + 64;   // sum_i beta_i dA_ij E_ij X_ij
   float* sR = sCol + 64;     // vector gate only: dA, then beta dA  [64][LNX_LDA]
   T* sTmT = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
-  T* sIn = sTmT + L::kTile;   // dW^T / dD^T slab  [col][token]
-  T* sWU = sIn + L::kTile;    // W / U slab        [token][col]
-  T* sdBt = sWU + L::kTile;   // dB slab           [token][col]
+  T* sIn = sTmT + L::kTile;   // dW / dD slab      [token][col]
+  T* sdBt = sIn + L::kTile;   // dB slab           [token][col]
   T* sKs = sdBt + L::kTile;   // K / V slab        [token][col]
+  T* sWU = sKs + L::kTile;    // W / U slab        [token][col]; vector gate only
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -620,24 +622,29 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   }
   stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
 
+  // dA needs M = dBw W^T + dBu U^T.  With a per-channel gate W and U are read back from the workspace.  Otherwise
+  // W = Tm diag(beta e^G) K and U = Tm diag(beta) V give M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T with
+  // Zw = dBw K^T and Zu = dBu V^T summed over the slabs already in LDS: W and U are never loaded.
+  constexpr bool LOAD_WU = GATE == LNX_GATE_VECTOR;
   TileRegs<T, 64, 64> rIn, rWU, rKs;  // dW / dD slab [token][col], W / U slab, K / V slab
   auto fetch = [&](int s_) {
     if (s_ < NKS) {
       const int c0 = 64 * s_;
       rIn.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
-      rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
+      if (LOAD_WU) rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
       rKs.load(kg + c0, tsk, len, tid);
     } else {
       const int v0 = 64 * (s_ - NKS);
       rIn.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
-      rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+      if (LOAD_WU) rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       rKs.load(vg + v0, tsv, len, tid);
     }
   };
-  floatx16 aBw[NKS][1][1], aM[1][1], aX[1][1];
+  floatx16 aBw[NKS][1][1], aM[1][1], aZu[1][1], aX[1][1];  // aM doubles as Zw inside the loop
 #pragma unroll
   for (int s_ = 0; s_ < NKS; ++s_) frag_zero(aBw[s_]);
   frag_zero(aM);
+  frag_zero(aZu);
   frag_zero(aX);
 
   fetch(0);
@@ -646,7 +653,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     const bool is_k = s_ < NKS;
     lds_barrier();
     rIn.store(sIn, LDC, tid);
-    rWU.store(sWU, LDC, tid);
+    if (LOAD_WU) rWU.store(sWU, LDC, tid);
     rKs.store(sKs, LDC, tid);
     lds_barrier();
     if (s_ + 1 < nslab) fetch(s_ + 1);
@@ -665,7 +672,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
         mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
     }
     lds_barrier();
-    mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
+    if (LOAD_WU) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
+    else if (is_k) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
+    else mma_nt<T, 1, 1>(aZu, sdBt + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
     if (GATE != LNX_GATE_VECTOR || !is_k) {  // <dB row, k row> / <dB row, v row>; thread = (row, quarter of the slab)
       const int r = tid >> 2, q0 = (tid & 3) * 16;
       float t = 0.f;
@@ -803,12 +812,24 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   }
   // K slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
   TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
-#pragma unroll
-  for (int u = 0; u < NKS; ++u) {
-    rKT[u].load(kg + 64 * u, tsk, len, tid);  // K rows again, for Y K
-    rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);
-  }
   lds_barrier();  // loop tiles dead
+  {  // M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T
+    floatx16 z[1][1];
+    const int j = 32 * wj + frag_col(lane);
+    const float cu = sBeta[j], cw = (GATE == LNX_GATE_NONE) ? cu : cu * __expf(sG[j]);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) z[0][0][e] = aM[0][0][e] * cw + aZu[0][0][e] * cu;
+    frag_store<T, 1, 1>(z, sIn + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_zero(aM);
+#pragma unroll
+    for (int u = 0; u < NKS; ++u) {
+      rKT[u].load(kg + 64 * u, tsk, len, tid);  // K rows again, for Y K
+      rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);
+    }
+    lds_barrier();
+    mma_x<T, 1, 1, false, true>(aM, sIn + 32 * wi * LDC, LDC, sTmT + 32 * wj, LDC, 64, lane);
+    lds_barrier();  // Z and Tm^T are overwritten below
+  }
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
     floatx16 y[1][1];
