@@ -311,6 +311,44 @@ def bench_dplr_step(torch, la, _lib, steps):
                          "frac": ach / PEAK_HBM, "traffic": None}}
 
 
+def bench_rmsnorm_gated(torch, la, _lib, steps, warmup):
+    """Gated RMSNorm epilogue over config 2's outputs: x, gate [B8, T4096, H16, d128] bf16, forward + backward.
+    Algorithmic bytes: x, gate in, y out; x, gate, dy in, dx, dgate out."""
+    shape = (8, 4096, 16, 128)
+    gen = torch.Generator(device="cpu").manual_seed(8)
+    x, g, dy = (torch.randn(*shape, generator=gen).to("cuda:0").bfloat16() for _ in range(3))
+    x.requires_grad_(True), g.requires_grad_(True)
+    w = torch.ones(128, device="cuda:0", requires_grad=True)
+
+    def step():
+        x.grad = g.grad = w.grad = None
+        la.rmsnorm_gated(x, g, w).backward(dy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    marks = _lib.profile_read()
+    _lib.profile_enable(False)
+    names = ("rmsnorm_gated_fwd", "rmsnorm_gated_bwd")
+    avg = {n: sum(ms for m, ms in marks if m == n) / max(1, sum(1 for m, _ in marks if m == n)) for n in names}
+    n_el = x.numel()
+    nb = {"rmsnorm_gated_fwd": 3 * n_el * 2, "rmsnorm_gated_bwd": 5 * n_el * 2}
+    roof = {n: {"bound": "hbm", "kernel": n, "achieved": nb[n] / (avg[n] * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                "frac": nb[n] / (avg[n] * 1e-3) / 1e9 / PEAK_HBM, "traffic": None} for n in names}
+    return {"metric": "gated RMSNorm fwd+bwd tokens/s", "value": shape[0] * shape[1] / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "rmsnorm_gated_fwd_bwd", "B": 8, "T": 4096, "H": 16, "d": 128},
+            "kernel_ms": {n: round(v, 4) for n, v in avg.items()}, "roofline": roof["rmsnorm_gated_bwd"],
+            "roofline_fwd": roof["rmsnorm_gated_fwd"]}
+
+
 def bench_decode_graph(torch, steps):
     """Host cost per generated token of a 24-layer Gated DeltaNet decode (B=1 and 8, H=32, d=128): the layers'
     steps replayed as one captured graph against one eager op call per layer."""
@@ -341,7 +379,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -360,6 +398,9 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "rmsnorm_gated":
+        print(json.dumps(bench_rmsnorm_gated(torch, la, _lib, args.steps, args.warmup)))
+        return
     if args.workload == "dplr_decode":
         print(json.dumps(bench_dplr_step(torch, la, _lib, max(args.steps, 500))))
         return

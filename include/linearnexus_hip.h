@@ -168,6 +168,21 @@ int lnx_dplr_recurrent_fwd(const lnx_dplr_args* a, void* hip_stream);
 int lnx_dplr_step(const lnx_dplr_args* a, void* hip_stream);
 
 /*
+ * RMSNorm with an optional sigmoid gate over the rows of [rows, d] matrices, the output epilogue of the reference's
+ * blocks: y = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate).  Replaces FusedRMSNormGated.__call__
+ * (linearnexus/modules/linear_attn/kda.py:664-700) and o_norm(o) * sigmoid(g_out) (gated_deltanet.py:854-862).
+ * x, gate, y, dy, dx, d_gate in `dtype`; weight, d_weight [d] fp32; gate NULL = no gate; d a multiple of 16 bytes
+ * of elements with 4..64 such vectors per row.  d_weight (may be NULL) is summed without atomics through partial rows
+ * in a caller-owned workspace of lnx_rmsnorm_gated_bwd_workspace_bytes bytes.
+ */
+int lnx_rmsnorm_gated_fwd(const void* x, const void* gate, const float* weight, void* y, int64_t rows, int32_t d,
+                          float eps, int32_t dtype, void* hip_stream);
+uint64_t lnx_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int32_t d, int32_t dtype);
+int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const float* weight, const void* dy, void* dx, void* d_gate,
+                          float* d_weight, int64_t rows, int32_t d, float eps, int32_t dtype, void* workspace,
+                          uint64_t workspace_bytes, void* hip_stream);
+
+/*
  * Optional per-kernel timing for benchmarks (no counterpart in the reference; its micro-benchmark
  * times whole jitted ops, bench_kda_kernels.py:216-249).  While enabled (process-wide),
  * every entry point records HIP events around each kernel it launches, on the caller's stream.

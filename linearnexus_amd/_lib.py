@@ -16,7 +16,8 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
-    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_profile_enable", "lnx_profile_read",
+    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
+    "lnx_profile_enable", "lnx_profile_read",
 )
 
 
@@ -78,6 +79,13 @@ def load() -> C.CDLL:
     lib.lnx_conv1d_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int32] * 6 + [C.c_void_p]
     lib.lnx_conv1d_bwd.restype = C.c_int
     lib.lnx_conv1d_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int32] * 6 + [C.c_void_p]
+    lib.lnx_rmsnorm_gated_fwd.restype = C.c_int
+    lib.lnx_rmsnorm_gated_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
+    lib.lnx_rmsnorm_gated_bwd.restype = C.c_int
+    lib.lnx_rmsnorm_gated_bwd.argtypes = [C.c_void_p] * 7 + [C.c_int64, C.c_int32, C.c_float, C.c_int32, C.c_void_p, C.c_uint64,
+                                          C.c_void_p]
+    lib.lnx_rmsnorm_gated_bwd_workspace_bytes.restype = C.c_uint64
+    lib.lnx_rmsnorm_gated_bwd_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     for name in ("lnx_dplr_recurrent_fwd", "lnx_dplr_step"):
         fn = getattr(lib, name)
         fn.restype = C.c_int

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void conv1d_fwd_kernel(ConvParams p) {
 // Backward of one run [t0, t1): sweeps u = t0 .. t1+2, recomputes z[u] from the window of x, forms
 // dz[u] = dy[u] * act'(z[u]) and emits dx[u-3] = sum_j w[j] dz[u-j] once its four terms are known.
 // dw, dbias: per-thread sums over the run's own tokens, reduced over the workgroup's four runs in LDS and
-// added to the fp32 outputs with one atomic per (tap, channel) and workgroup.  The workgroup is 64 channel
+// added to the fp32 outputs with one hardware fp32 atomic (not a compare-and-swap loop) per (tap, channel) and workgroup.  The workgroup is 64 channel
 // groups x 4 runs here whatever the row length.
 template <typename T, int N>
 __global__ __launch_bounds__(256) void conv1d_bwd_kernel(ConvParams p) {
@@ -245,14 +245,14 @@ __global__ __launch_bounds__(256) void conv1d_bwd_kernel(ConvParams p) {
     for (int i = 0; i < N; ++i) {
       float sb = gb[i];
       for (int r = 0; r < BWD_RUNS - 1; ++r) sb += red[r][KMAX][lane * N + i];
-      if (p.dbias) atomicAdd(p.dbias + c + i, sb);
+      if (p.dbias) unsafeAtomicAdd(p.dbias + c + i, sb);
 #pragma unroll
       for (int j = 0; j < KMAX; ++j) {
         const int jr = j - (KMAX - p.K);
         if (jr < 0) continue;
         float s = gw[j][i];
         for (int r = 0; r < BWD_RUNS - 1; ++r) s += red[r][j][lane * N + i];
-        atomicAdd(p.dw + (size_t)jr * p.D + c + i, s);
+        unsafeAtomicAdd(p.dw + (size_t)jr * p.D + c + i, s);
       }
     }
   }

@@ -1,0 +1,273 @@
+// RMSNorm with an optional sigmoid gate over the rows of a [rows, d] matrix, forward and backward: the
+// output epilogue of the reference's blocks (FusedRMSNormGated, linearnexus/modules/linear_attn/kda.py:664-700,
+// used as o_norm(o) * sigmoid(gate) in gated_deltanet.py:854-862):
+//   y = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate)        (gate NULL: no gate)
+// Streaming kernels: LPR lanes share a row of LPR 16-byte vectors, a wavefront covers 64 / LPR rows per pass,
+// and the loads of four passes are issued together.  The backward also keeps d_weight partial sums in
+// registers over all passes of a wavefront and adds them with one atomic per column and workgroup.
+#include "lnx_common.h"
+#include "mma_tiles.h"
+
+namespace {
+
+constexpr int UNR = 4;         // passes whose loads are in flight together
+constexpr int SUM_SLICES = 64;  // first-level slices of the d_weight partial rows
+constexpr int BWD_STEPS = 8;   // steps (of UNR passes) per wavefront in the backward: rows per d_weight atomic
+
+__device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + __expf(-z)); }
+
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void rmsnorm_gated_fwd_kernel(const T* x, const T* gate, const float* w, T* y,
+                                                                int64_t rows, float eps) {
+  typedef typename Vec16<T>::V V;
+  constexpr int VN = Vec16<T>::N, RPW = 64 / LPR, D = LPR * VN;
+  const int lane = threadIdx.x & 63, sub = lane / LPR, li = lane % LPR;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t r0 = wave * (RPW * UNR) + sub;
+  float wv[VN];
+#pragma unroll
+  for (int e = 0; e < VN; ++e) wv[e] = w[li * VN + e];
+  V xv[UNR], gv[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    xv[u] = vec_zero<T>();
+    gv[u] = vec_zero<T>();
+    if (r < rows) {
+      xv[u] = *reinterpret_cast<const V*>(x + r * D + li * VN);
+      if (gate) gv[u] = *reinterpret_cast<const V*>(gate + r * D + li * VN);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t r = r0 + u * RPW;
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) { const float t = to_f32(xv[u][e]); ss += t * t; }
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, LNX_WAVE);
+    const float rstd = rsqrtf(ss * (1.f / D) + eps);
+    V out;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) {
+      const float s = gate ? sigmoidf(to_f32(gv[u][e])) : 1.f;
+      out[e] = from_f32<T>(to_f32(xv[u][e]) * rstd * wv[e] * s);
+    }
+    if (r < rows) *reinterpret_cast<V*>(y + r * D + li * VN) = out;
+  }
+}
+
+// With xn = x rstd, s = sigmoid(gate), u = dy s w:
+//   dx = rstd (u - xn mean(u xn));  dgate = dy xn w s (1 - s);  dweight = sum over rows of dy xn s.
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void rmsnorm_gated_bwd_kernel(const T* x, const T* gate, const float* w, const T* dy,
+                                                                T* dx, T* dgate, float* dw, int64_t rows, float eps) {
+  typedef typename Vec16<T>::V V;
+  constexpr int VN = Vec16<T>::N, RPW = 64 / LPR, D = LPR * VN;
+  const int lane = threadIdx.x & 63, sub = lane / LPR, li = lane % LPR;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  float wv[VN], dwv[VN];
+#pragma unroll
+  for (int e = 0; e < VN; ++e) wv[e] = w[li * VN + e], dwv[e] = 0.f;
+  for (int step = 0; step < BWD_STEPS; ++step) {
+    const int64_t r0 = (wave * BWD_STEPS + step) * (RPW * UNR) + sub;
+    if (r0 - sub >= rows) break;
+    V xv[UNR], gv[UNR], yv[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int64_t r = r0 + u * RPW;
+      xv[u] = vec_zero<T>();
+      gv[u] = vec_zero<T>();
+      yv[u] = vec_zero<T>();
+      if (r < rows) {
+        xv[u] = *reinterpret_cast<const V*>(x + r * D + li * VN);
+        yv[u] = *reinterpret_cast<const V*>(dy + r * D + li * VN);
+        if (gate) gv[u] = *reinterpret_cast<const V*>(gate + r * D + li * VN);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int64_t r = r0 + u * RPW;
+      float ss = 0.f, dot = 0.f, uu[VN], sg[VN];
+#pragma unroll
+      for (int e = 0; e < VN; ++e) {
+        const float t = to_f32(xv[u][e]);
+        sg[e] = gate ? sigmoidf(to_f32(gv[u][e])) : 1.f;
+        uu[e] = to_f32(yv[u][e]) * sg[e] * wv[e];
+        ss += t * t;
+        dot += uu[e] * t;
+      }
+#pragma unroll
+      for (int m = LPR / 2; m >= 1; m >>= 1) {
+        ss += __shfl_xor(ss, m, LNX_WAVE);
+        dot += __shfl_xor(dot, m, LNX_WAVE);
+      }
+      const float rstd = rsqrtf(ss * (1.f / D) + eps);
+      const float c = dot * rstd * rstd * (1.f / D);  // mean(u xn) rstd / rstd: applied to x below
+      V ox, og;
+#pragma unroll
+      for (int e = 0; e < VN; ++e) {
+        const float t = to_f32(xv[u][e]), xn = t * rstd, g = to_f32(yv[u][e]);
+        ox[e] = from_f32<T>(rstd * (uu[e] - t * c));
+        og[e] = from_f32<T>(g * xn * wv[e] * sg[e] * (1.f - sg[e]));
+        dwv[e] += g * xn * sg[e];  // rows past the end contribute zeros (x, dy loaded as zeros)
+      }
+      if (r < rows) {
+        *reinterpret_cast<V*>(dx + r * D + li * VN) = ox;
+        if (gate) *reinterpret_cast<V*>(dgate + r * D + li * VN) = og;
+      }
+    }
+  }
+  if (!dw) return;
+  // d_weight: over the rows of a pass by shuffles, over the four wavefronts in LDS, then one row of partial sums
+  // per workgroup in the workspace (a second kernel adds the rows: no atomics, the result is deterministic)
+  __shared__ float red[3][D];
+  const int wv_i = threadIdx.x >> 6;
+#pragma unroll
+  for (int e = 0; e < VN; ++e) {
+    float t = dwv[e];
+#pragma unroll
+    for (int m = LPR; m < 64; m <<= 1) t += __shfl_xor(t, m, LNX_WAVE);
+    dwv[e] = t;
+    if (sub == 0 && wv_i > 0) red[wv_i - 1][li * VN + e] = t;
+  }
+  __syncthreads();
+  if (wv_i == 0 && sub == 0) {
+#pragma unroll
+    for (int e = 0; e < VN; ++e)
+      dw[(size_t)blockIdx.x * D + li * VN + e] = dwv[e] + red[0][li * VN + e] + red[1][li * VN + e] + red[2][li * VN + e];
+  }
+}
+
+// out[y][c] = sum of part[r][c] over the rows r of slice y = blockIdx.y (`per` rows each, `n` rows in all; d a
+// multiple of 4); 256 threads = 16 groups of four columns x 16 interleaved row sets, eight independent loads in
+// flight per thread.  Run twice -- many slices, then one -- so that no single CU has to read all partial rows.
+__global__ __launch_bounds__(256) void sum_rows_kernel(const float* part, int64_t n, int64_t per, int d, float* out) {
+  part += (int64_t)blockIdx.y * per * d;
+  out += (int64_t)blockIdx.y * d;
+  n = min(per, n - (int64_t)blockIdx.y * per);
+  __shared__ floatx4 red[16][16];
+  const int cg = threadIdx.x & 15, rs = threadIdx.x >> 4;
+  const int c = (blockIdx.x * 16 + cg) * 4;
+  floatx4 acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  if (c < d) {
+    for (int64_t r = rs; r < n; r += 16 * 8) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (r + 16 * u < n) acc[u] += load4(part + (r + 16 * u) * d + c);
+    }
+  }
+  red[rs][cg] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+  __syncthreads();
+  if (rs == 0 && c < d) {
+    floatx4 t = red[0][cg];
+#pragma unroll
+    for (int q = 1; q < 16; ++q) t += red[q][cg];
+    store4(out + c, t);
+  }
+}
+
+template <typename T> int lanes_for(int d) {
+  constexpr int VN = 16 / sizeof(T);
+  if (d % VN != 0) return 0;
+  const int l = d / VN;
+  return (l == 4 || l == 8 || l == 16 || l == 32 || l == 64) ? l : 0;
+}
+
+#define LNX_LPR_SWITCH(KERNEL, ...)                                                              \
+  switch (l) {                                                                                   \
+    case 4: hipLaunchKernelGGL((KERNEL<T, 4>), grid, dim3(256), 0, st, __VA_ARGS__); break;      \
+    case 8: hipLaunchKernelGGL((KERNEL<T, 8>), grid, dim3(256), 0, st, __VA_ARGS__); break;      \
+    case 16: hipLaunchKernelGGL((KERNEL<T, 16>), grid, dim3(256), 0, st, __VA_ARGS__); break;    \
+    case 32: hipLaunchKernelGGL((KERNEL<T, 32>), grid, dim3(256), 0, st, __VA_ARGS__); break;    \
+    default: hipLaunchKernelGGL((KERNEL<T, 64>), grid, dim3(256), 0, st, __VA_ARGS__); break;    \
+  }
+
+template <typename T>
+void launch_fwd(int l, const void* x, const void* gate, const float* w, void* y, int64_t rows, float eps, hipStream_t st) {
+  const int64_t waves = (rows + (64 / l) * UNR - 1) / ((64 / l) * UNR);
+  dim3 grid((unsigned)((waves + 3) / 4));
+  LNX_LPR_SWITCH(rmsnorm_gated_fwd_kernel, (const T*)x, (const T*)gate, w, (T*)y, rows, eps)
+}
+
+int64_t bwd_blocks(int l, int64_t rows) {
+  const int64_t per_wave = (int64_t)(64 / l) * UNR * BWD_STEPS;
+  return ((rows + per_wave - 1) / per_wave + 3) / 4;
+}
+
+template <typename T>
+void launch_bwd(int l, const void* x, const void* gate, const float* w, const void* dy, void* dx, void* dgate, float* dw,
+                int64_t rows, float eps, hipStream_t st) {
+  dim3 grid((unsigned)bwd_blocks(l, rows));
+  LNX_LPR_SWITCH(rmsnorm_gated_bwd_kernel, (const T*)x, (const T*)gate, w, (const T*)dy, (T*)dx, (T*)dgate, dw, rows, eps)
+}
+
+int check(const void* x, const float* w, int64_t rows, int d, int dtype) {
+  if (rows < 0 || d <= 0) return lnx_set_error(LNX_ERR_SHAPE, "rmsnorm_gated: rows=%lld d=%d", (long long)rows, d);
+  if (dtype != LNX_F32 && dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "rmsnorm_gated: dtype %d", dtype);
+  const int l = dtype == LNX_BF16 ? lanes_for<bf16_t>(d) : lanes_for<float>(d);
+  if (!l)
+    return lnx_set_error(LNX_ERR_SHAPE, "rmsnorm_gated: d=%d must be 4, 8, 16, 32 or 64 vectors of 16 bytes", d);
+  if (!w || (rows > 0 && !x)) return lnx_set_error(LNX_ERR_NULL, "rmsnorm_gated: x and weight are required");
+  return LNX_OK;
+}
+
+}  // namespace
+
+extern "C" int lnx_rmsnorm_gated_fwd(const void* x, const void* gate, const float* weight, void* y, int64_t rows, int32_t d,
+                                     float eps, int32_t dtype, void* hip_stream) {
+  if (int rc = check(x, weight, rows, d, dtype)) return rc;
+  if (rows == 0) return LNX_OK;
+  if (!y) return lnx_set_error(LNX_ERR_NULL, "rmsnorm_gated_fwd: y is NULL");
+  hipStream_t st = static_cast<hipStream_t>(hip_stream);
+  lnx_profile_mark("rmsnorm_gated_fwd", st);
+  if (dtype == LNX_BF16) launch_fwd<bf16_t>(lanes_for<bf16_t>(d), x, gate, weight, y, rows, eps, st);
+  else launch_fwd<float>(lanes_for<float>(d), x, gate, weight, y, rows, eps, st);
+  lnx_profile_mark(nullptr, st);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? LNX_OK : lnx_set_error(LNX_ERR_LAUNCH, "rmsnorm_gated_fwd: %s", hipGetErrorString(e));
+}
+
+extern "C" uint64_t lnx_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int32_t d, int32_t dtype) {
+  const int l = dtype == LNX_BF16 ? lanes_for<bf16_t>(d) : lanes_for<float>(d);
+  if (!l || rows <= 0) return 0;
+  return (uint64_t)(bwd_blocks(l, rows) + SUM_SLICES) * d * sizeof(float);
+}
+
+extern "C" int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const float* weight, const void* dy, void* dx,
+                                     void* d_gate, float* d_weight, int64_t rows, int32_t d, float eps, int32_t dtype,
+                                     void* workspace, uint64_t workspace_bytes, void* hip_stream) {
+  if (int rc = check(x, weight, rows, d, dtype)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(hip_stream);
+  const int l = dtype == LNX_BF16 ? lanes_for<bf16_t>(d) : lanes_for<float>(d);
+  float* part = nullptr;
+  if (rows > 0) {
+    if (!dy || !dx || (gate && !d_gate)) return lnx_set_error(LNX_ERR_NULL, "rmsnorm_gated_bwd: dy, dx (and d_gate) are required");
+    if (d_weight) {
+      const uint64_t need = lnx_rmsnorm_gated_bwd_workspace_bytes(rows, d, dtype);
+      if (!workspace || workspace_bytes < need)
+        return lnx_set_error(LNX_ERR_WORKSPACE, "rmsnorm_gated_bwd: d_weight needs a workspace of %llu bytes", (unsigned long long)need);
+      part = static_cast<float*>(workspace);
+    }
+    lnx_profile_mark("rmsnorm_gated_bwd", st);
+    if (dtype == LNX_BF16) launch_bwd<bf16_t>(l, x, gate, weight, dy, dx, d_gate, part, rows, eps, st);
+    else launch_bwd<float>(l, x, gate, weight, dy, dx, d_gate, part, rows, eps, st);
+  }
+  if (d_weight) {
+    lnx_profile_mark("rmsnorm_dweight", st);
+    const int64_t n = rows > 0 ? bwd_blocks(l, rows) : 0, per = (n + SUM_SLICES - 1) / SUM_SLICES;
+    if (per > 1) {  // two levels: SUM_SLICES rows of sums behind the partial rows, then their sum
+      float* part2 = part + n * d;
+      const int slices = (int)((n + per - 1) / per);
+      sum_rows_kernel<<<dim3((d + 63) / 64, slices), 256, 0, st>>>(part, n, per, d, part2);
+      sum_rows_kernel<<<dim3((d + 63) / 64, 1), 256, 0, st>>>(part2, slices, slices, d, d_weight);
+    } else {
+      sum_rows_kernel<<<dim3((d + 63) / 64, 1), 256, 0, st>>>(part, n, n, d, d_weight);
+    }
+  }
+  lnx_profile_mark(nullptr, st);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? LNX_OK : lnx_set_error(LNX_ERR_LAUNCH, "rmsnorm_gated_bwd: %s", hipGetErrorString(e));
+}
