@@ -349,6 +349,46 @@ def bench_rmsnorm_gated(torch, la, _lib, steps, warmup):
             "roofline_fwd": roof["rmsnorm_gated_fwd"]}
 
 
+def bench_kda_gate(torch, la, _lib, steps, warmup):
+    """KDA gate activation for config 3's gate tensor: raw gate [B4, T8192, H16*dk128] bf16 -> fp32 log-decay, forward
+    + backward.  Algorithmic bytes: g (bf16) in, g_out (fp32) out; g, d_out (fp32) in, d_g (bf16) out."""
+    B, T, H, dk = 4, 8192, 16, 128
+    gen = torch.Generator(device="cpu").manual_seed(9)
+    raw = torch.randn(B, T, H * dk, generator=gen).to("cuda:0").bfloat16().requires_grad_(True)
+    dy = torch.randn(B, T, H, dk, generator=gen).to("cuda:0")
+    A = torch.zeros(H, device="cuda:0", requires_grad=True)
+    bias = torch.zeros(H * dk, device="cuda:0", requires_grad=True)
+
+    def step():
+        raw.grad = A.grad = bias.grad = None
+        g, _ = la.kda_gate(raw, A, dk, bias, out_dtype=torch.float32)
+        g.backward(dy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    marks = _lib.profile_read()
+    _lib.profile_enable(False)
+    names = ("kda_gate_fwd", "kda_gate_bwd")
+    avg = {n: sum(ms for m, ms in marks if m == n) / max(1, sum(1 for m, _ in marks if m == n)) for n in names}
+    n_el = raw.numel()
+    nb = {"kda_gate_fwd": n_el * (2 + 4), "kda_gate_bwd": n_el * (2 + 4 + 2)}
+    roof = {n: {"bound": "hbm", "kernel": n, "achieved": nb[n] / (avg[n] * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s",
+                "frac": nb[n] / (avg[n] * 1e-3) / 1e9 / PEAK_HBM, "traffic": None} for n in names}
+    return {"metric": "KDA gate activation fwd+bwd tokens/s", "value": B * T / dt, "unit": "tokens/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "kda_gate_fwd_bwd", "B": B, "T": T, "H": H, "dk": dk},
+            "kernel_ms": {n: round(v, 4) for n, v in avg.items()}, "roofline": roof["kda_gate_bwd"],
+            "roofline_fwd": roof["kda_gate_fwd"]}
+
+
 def bench_decode_graph(torch, steps):
     """Host cost per generated token of a 24-layer Gated DeltaNet decode (B=1 and 8, H=32, d=128): the layers'
     steps replayed as one captured graph against one eager op call per layer."""
@@ -379,7 +419,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated", "kda_gate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -398,6 +438,9 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "kda_gate":
+        print(json.dumps(bench_kda_gate(torch, la, _lib, args.steps, args.warmup)))
+        return
     if args.workload == "rmsnorm_gated":
         print(json.dumps(bench_rmsnorm_gated(torch, la, _lib, args.steps, args.warmup)))
         return

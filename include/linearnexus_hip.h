@@ -183,6 +183,23 @@ int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const float* weight, 
                           uint64_t workspace_bytes, void* hip_stream);
 
 /*
+ * KDA's gate activation (kda_gate, linearnexus/modules/linear_attn/kda.py:120-172) and its gradient:
+ *   g_out[r, h, c] = -exp(A_log[h]) * softplus(g[r, h*dk + c] + g_bias[h*dk + c]),  softplus(x) = x for x > threshold
+ * g, d_g [rows, H*dk] in `dtype`; g_out, d_out [rows, H, dk] in `out_dtype` (fp32 feeds lnx_chunk_fwd's vector gate
+ * without a cast; the reference returns the input dtype, kda.py:172); A_log [H], g_bias [H*dk] (may be NULL) and their
+ * gradients fp32 (may be NULL; they are summed without atomics through a caller-owned workspace).  dk % 4 == 0.
+ * lnx_sigmoid_fwd / lnx_sigmoid_bwd are the beta = sigmoid(.) of the same function (kda.py:168-170) on fp32 vectors.
+ */
+int lnx_kda_gate_fwd(const void* g, const float* A_log, const float* g_bias, void* g_out, int64_t rows, int32_t H,
+                     int32_t dk, float threshold, int32_t dtype, int32_t out_dtype, void* hip_stream);
+uint64_t lnx_kda_gate_bwd_workspace_bytes(int64_t rows, int32_t H, int32_t dk);
+int lnx_kda_gate_bwd(const void* g, const float* A_log, const float* g_bias, const void* d_out, void* d_g, float* d_A_log,
+                     float* d_bias, int64_t rows, int32_t H, int32_t dk, float threshold, int32_t dtype, int32_t out_dtype,
+                     void* workspace, uint64_t workspace_bytes, void* hip_stream);
+int lnx_sigmoid_fwd(const float* x, float* y, int64_t n, void* hip_stream);
+int lnx_sigmoid_bwd(const float* y, const float* dy, float* dx, int64_t n, void* hip_stream);
+
+/*
  * Optional per-kernel timing for benchmarks (no counterpart in the reference; its micro-benchmark
  * times whole jitted ops, bench_kda_kernels.py:216-249).  While enabled (process-wide),
  * every entry point records HIP events around each kernel it launches, on the caller's stream.

@@ -7,11 +7,11 @@
 // registers over all passes of a wavefront and adds them with one atomic per column and workgroup.
 #include "lnx_common.h"
 #include "mma_tiles.h"
+#include "reduce_rows.h"
 
 namespace {
 
 constexpr int UNR = 4;         // passes whose loads are in flight together
-constexpr int SUM_SLICES = 64;  // first-level slices of the d_weight partial rows
 constexpr int BWD_STEPS = 8;   // steps (of UNR passes) per wavefront in the backward: rows per d_weight atomic
 
 __device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + __expf(-z)); }
@@ -139,36 +139,6 @@ __global__ __launch_bounds__(256) void rmsnorm_gated_bwd_kernel(const T* x, cons
   }
 }
 
-// out[y][c] = sum of part[r][c] over the rows r of slice y = blockIdx.y (`per` rows each, `n` rows in all; d a
-// multiple of 4); 256 threads = 16 groups of four columns x 16 interleaved row sets, eight independent loads in
-// flight per thread.  Run twice -- many slices, then one -- so that no single CU has to read all partial rows.
-__global__ __launch_bounds__(256) void sum_rows_kernel(const float* part, int64_t n, int64_t per, int d, float* out) {
-  part += (int64_t)blockIdx.y * per * d;
-  out += (int64_t)blockIdx.y * d;
-  n = min(per, n - (int64_t)blockIdx.y * per);
-  __shared__ floatx4 red[16][16];
-  const int cg = threadIdx.x & 15, rs = threadIdx.x >> 4;
-  const int c = (blockIdx.x * 16 + cg) * 4;
-  floatx4 acc[8];
-#pragma unroll
-  for (int u = 0; u < 8; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-  if (c < d) {
-    for (int64_t r = rs; r < n; r += 16 * 8) {
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (r + 16 * u < n) acc[u] += load4(part + (r + 16 * u) * d + c);
-    }
-  }
-  red[rs][cg] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
-  __syncthreads();
-  if (rs == 0 && c < d) {
-    floatx4 t = red[0][cg];
-#pragma unroll
-    for (int q = 1; q < 16; ++q) t += red[q][cg];
-    store4(out + c, t);
-  }
-}
-
 template <typename T> int lanes_for(int d) {
   constexpr int VN = 16 / sizeof(T);
   if (d % VN != 0) return 0;
@@ -233,7 +203,7 @@ extern "C" int lnx_rmsnorm_gated_fwd(const void* x, const void* gate, const floa
 extern "C" uint64_t lnx_rmsnorm_gated_bwd_workspace_bytes(int64_t rows, int32_t d, int32_t dtype) {
   const int l = dtype == LNX_BF16 ? lanes_for<bf16_t>(d) : lanes_for<float>(d);
   if (!l || rows <= 0) return 0;
-  return (uint64_t)(bwd_blocks(l, rows) + SUM_SLICES) * d * sizeof(float);
+  return lnx_sum_rows_bytes(bwd_blocks(l, rows), d);
 }
 
 extern "C" int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const float* weight, const void* dy, void* dx,
@@ -257,15 +227,7 @@ extern "C" int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const floa
   }
   if (d_weight) {
     lnx_profile_mark("rmsnorm_dweight", st);
-    const int64_t n = rows > 0 ? bwd_blocks(l, rows) : 0, per = (n + SUM_SLICES - 1) / SUM_SLICES;
-    if (per > 1) {  // two levels: SUM_SLICES rows of sums behind the partial rows, then their sum
-      float* part2 = part + n * d;
-      const int slices = (int)((n + per - 1) / per);
-      sum_rows_kernel<<<dim3((d + 63) / 64, slices), 256, 0, st>>>(part, n, per, d, part2);
-      sum_rows_kernel<<<dim3((d + 63) / 64, 1), 256, 0, st>>>(part2, slices, slices, d, d_weight);
-    } else {
-      sum_rows_kernel<<<dim3((d + 63) / 64, 1), 256, 0, st>>>(part, n, n, d, d_weight);
-    }
+    lnx_sum_rows(part, rows > 0 ? bwd_blocks(l, rows) : 0, d, d_weight, st);
   }
   lnx_profile_mark(nullptr, st);
   hipError_t e = hipGetLastError();
