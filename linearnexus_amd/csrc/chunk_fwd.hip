@@ -59,9 +59,16 @@ template <typename T, int DK> struct Prep2Cfg {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kTile = 64 * LDC;
-  static constexpr size_t f32_bytes = sizeof(float) * (2 * 64 * LNX_LDA);  // A and Tm; the merge scratch overlays the Q slab
-  static constexpr size_t regionF = (2 * kTile * sizeof(T) > f32_bytes) ? 2 * kTile * sizeof(T) : f32_bytes;
-  static constexpr size_t bytes = regionF + 2 * kTile * sizeof(T) + sizeof(float) * 128;
+  static constexpr size_t cmax(size_t a, size_t b) { return a > b ? a : b; }
+  static constexpr size_t mat = sizeof(float) * 64 * LNX_LDA;  // one fp32 64x64 matrix
+  static constexpr size_t scr = sizeof(float) * 32 * 36;       // scratch of the inverse's block merges
+  // Two regions, each used by one thing at a time (2-byte inputs: 18 + 0.5 + 21.5 KB = 40 KB, four workgroups per CU):
+  //   region 0: A (fp32)                      -> after the inverse: Tw, Tu tiles
+  //   region 2: K, Q slab tiles, then P       -> Tm (fp32) + merge scratch -> loop-2 slab and result tiles
+  static constexpr size_t r0 = cmax(mat, 2 * kTile * sizeof(T));
+  static constexpr size_t r1 = sizeof(float) * 128;  // beta, G
+  static constexpr size_t r2 = cmax(mat + scr, 2 * kTile * sizeof(T));
+  static constexpr size_t bytes = r0 + r1 + r2;
 };
 
 template <typename T, int DK, int GATE>
@@ -69,15 +76,18 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   typedef Prep2Cfg<T, DK> L;
   constexpr int LDC = L::LDC, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
-  float* sA = reinterpret_cast<float*>(smem);
-  float* sT = sA + 64 * LNX_LDA;
-  T* sIn = reinterpret_cast<T*>(smem);  // overlays the fp32 matrices once Tw / Tu exist
-  T* sOut = sIn + L::kTile;
-  T* sKa = reinterpret_cast<T*>(smem + L::regionF);  // K slab, then Tw
-  T* sQa = sKa + L::kTile;                           // Q slab, then the inverse's scratch, then Tu
-  float* sX = reinterpret_cast<float*>(sQa);
-  float* sBeta = reinterpret_cast<float*>(sQa + L::kTile);
+  float* sA = reinterpret_cast<float*>(smem);      // region 0
+  T* sTw = reinterpret_cast<T*>(smem);             //   Tw, Tu once the inverse is done with A
+  T* sTu = sTw + L::kTile;
+  float* sBeta = reinterpret_cast<float*>(smem + L::r0);
   float* sG = sBeta + 64;
+  char* reg2 = smem + L::r0 + L::r1;               // region 2
+  T* sKa = reinterpret_cast<T*>(reg2);             //   K slab of the first loop, then P
+  T* sQa = sKa + L::kTile;                         //   Q slab
+  float* sT = reinterpret_cast<float*>(reg2);      //   Tm
+  float* sX = reinterpret_cast<float*>(reg2 + L::mat);
+  T* sIn = sKa;                                    //   second loop: slab in, result out
+  T* sOut = sQa;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -144,11 +154,10 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   }
   lds_barrier();
   unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sKa, LDC, 64, tid);
+  lds_barrier();  // Tm is built over the P tile
   tri_inverse_64(sA, sT, sX, tid);
   {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
-    T* sTw = sKa;
-    T* sTu = sQa;
     // one 4x4 block of Tm per thread: four-element row reads, the transpose taken in registers
     const int r0 = (tid >> 4) * 4, c0 = (tid & 15) * 4;
     floatx4 t[4];
@@ -179,7 +188,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     floatx16 acc[1][1];
     frag_zero(acc);
     // W = Tw K, U = Tu V: the slab is [token][column], contracted along its rows
-    mma_x<T, 1, 1, false, true>(acc, (is_k ? sKa : sQa) + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
+    mma_x<T, 1, 1, false, true>(acc, (is_k ? sTw : sTu) + 32 * wi * LDC, LDC, sIn + 32 * wj, LDC, 64, lane);
     frag_store<T, 1, 1>(acc, sOut + 32 * wi * LDC + 32 * wj, LDC, lane);
     lds_barrier();
     if (is_k)
