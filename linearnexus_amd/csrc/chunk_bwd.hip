@@ -640,12 +640,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
       rKs.load(vg + v0, tsv, len, tid);
     }
   };
-  floatx16 aBw[NKS][1][1], aM[1][1], aZu[1][1], aX[1][1];  // aM doubles as Zw inside the loop
+  floatx16 aBw[NKS][1][1], aM[1][1], aZu[1][1];  // aM doubles as Zw inside the loop
 #pragma unroll
   for (int s_ = 0; s_ < NKS; ++s_) frag_zero(aBw[s_]);
   frag_zero(aM);
   frag_zero(aZu);
-  frag_zero(aX);
 
   fetch(0);
 #pragma unroll 1
@@ -668,8 +667,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 #pragma unroll
           for (int e = 0; e < 16; ++e) aBw[u][0][0][e] = b[0][0][e];
         }
-      if (GATE != LNX_GATE_VECTOR && !(wi == 0 && wj == 1))
-        mma_nt<T, 1, 1>(aX, sKs + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
     }
     lds_barrier();
     if (LOAD_WU) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
@@ -810,8 +807,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     }
     return;
   }
-  // K slabs and the partial dk of bwd_dqk, fetched while the pair terms are formed
-  TileRegs<T, 64, 64> rKT[NKS], rdk[NKS];
+  // K slabs, fetched while the pair terms are formed; the partial dk of bwd_dqk one slab at a time
+  TileRegs<T, 64, 64> rKT[NKS], rdk;
   lds_barrier();  // loop tiles dead
   {  // M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T
     floatx16 z[1][1];
@@ -824,15 +821,30 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 #pragma unroll
     for (int u = 0; u < NKS; ++u) {
       rKT[u].load(kg + 64 * u, tsk, len, tid);  // K rows again, for Y K
-      rdk[u].load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);
     }
     lds_barrier();
     mma_x<T, 1, 1, false, true>(aM, sIn + 32 * wi * LDC, LDC, sTmT + 32 * wj, LDC, 64, lane);
     lds_barrier();  // Z and Tm^T are overwritten below
   }
+  // K rows of both slabs into LDS (over the K/V slab tile and Tm^T); X = K K^T is formed here rather than in the
+  // slab loop, where its accumulator would not fit the register budget of three workgroups per CU
+#pragma unroll
+  for (int u = 0; u < NKS; ++u) {
+    T* sKT = (u == 0) ? sKs : sTmT;
+    rKT[u].store(sKT, LDC, tid);
+  }
+  lds_barrier();
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
-    floatx16 y[1][1];
+    floatx16 aX[1][1], y[1][1];
+    frag_zero(aX);
+    if (!(wi == 0 && wj == 1)) {
+#pragma unroll
+      for (int u = 0; u < NKS; ++u) {
+        const T* sKT = (u == 0) ? sKs : sTmT;
+        mma_nt<T, 1, 1>(aX, sKT + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
+      }
+    }
     float v[16], cs = 0.f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -848,15 +860,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     cs += __shfl_xor(cs, 32, LNX_WAVE);
     if (lane < 32) atomicAdd(&sCol[32 * wj + lane], cs);
   }
-#pragma unroll
-  for (int u = 0; u < NKS; ++u) {
-    T* sKT = (u == 0) ? sKs : sTmT;
-    rKT[u].store(sKT, LDC, tid);
-  }
   lds_barrier();
 #pragma unroll
   for (int u = 0; u < NKS; ++u) {
     const T* sKT = (u == 0) ? sKs : sTmT;
+    rdk.load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);  // partial dk of bwd_dqk
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane);
@@ -877,7 +885,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
         if (r < len) {
           typename Vec16<T>::V x = *reinterpret_cast<const typename Vec16<T>::V*>(sdBt + r * LDC + c);
 #pragma unroll
-          for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) + to_f32(rdk[u].x[it][e]));
+          for (int e = 0; e < VN; ++e) x[e] = from_f32<T>(to_f32(x[e]) + to_f32(rdk.x[it][e]));
           *reinterpret_cast<typename Vec16<T>::V*>(dkg + (int64_t)r * tsk + c) = x;
         }
       }
