@@ -137,7 +137,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       TileRegs<T, 64, DK> K, Q, W;
       Slab dO, dD;                       // dD: the chunk-local part from bwd_local (not fused only)
       TileRegs<T, 64, FUSE ? 64 : 8> P;  // fused only
-      float os[Slab::IT];  // scale * e^{G_i} of the dO row each vector belongs to
+      float os[Slab::IT];  // G_i of the dO row each vector belongs to (scalar gate)
       float G;
     };
     constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;  // chunks fetched ahead (register sets in use)
@@ -161,12 +161,11 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
       if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+      // only the load here: anything computed from it would make the fetch wait for all loads issued before it
 #pragma unroll
       for (int it = 0; it < Slab::IT; ++it) {
         const int r = min((mt + 256 * it) / Slab::VPR, 63);
-        R.os[it] = (GATE == LNX_GATE_VECTOR) ? 1.f
-                   : (GATE == LNX_GATE_NONE) ? p.scale
-                                             : p.scale * __expf(wsp<float>(p, p.off.G)[slot * 64 + r]);
+        R.os[it] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + r] : 0.f;
       }
       if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = wsp<float>(p, p.off.G)[slot * 64 + mt];
       if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
@@ -185,8 +184,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
         typename Vec16<T>::V o = R.dO.x[it];
         if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}: (scale Q e^G)^T dO = Q^T (that)
+          const float os = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(R.os[it]);
 #pragma unroll
-          for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * R.os[it]);
+          for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * os);
         }
         if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
       }
@@ -553,7 +553,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
       d += __shfl_xor(d, 2, LNX_WAVE);
       if ((tid & 3) == 0) {
         if (r == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
-        atomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + r], d);
+        unsafeAtomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + r], d);  // hardware fp32 atomic: the two channel halves share dG
       }
     }
   }
