@@ -143,32 +143,37 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;  // chunks fetched ahead (register sets in use)
     Tiles ta, tb;
     ta.G = tb.G = 0.f;
-    auto fetch = [&](Tiles& R, int n) {
+    // Loads of chunk n into a register set, in three parts (part < 0: all at once).  A CU accepts vector memory
+    // instructions at a limited rate, so the parts are issued in different phases of a chunk instead of holding up
+    // the first one.  Nothing is computed from loaded values here: that would wait for every load issued before.
+    auto fetch = [&](Tiles& R, int n, int part) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0, len;
       chunk_span(p.geom, n, tok0, len);
       const int64_t tbase = tok_index(p.geom, row, tok0);
       const int64_t tsk = (int64_t)p.geom.ts * DK;
       // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)
-      if (GATE == LNX_GATE_VECTOR) {
-        R.K.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
-        R.Q.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
-      } else {
-        R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
-        R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, mt);
+      if (part < 0 || part == 0) {
+        if (GATE == LNX_GATE_VECTOR) R.K.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
       }
-      R.W.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
-      R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
-      if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
-      else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
-      // only the load here: anything computed from it would make the fetch wait for all loads issued before it
+      if (part < 0 || part == 1) {
+        R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
+        if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+        else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+        if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = wsp<float>(p, p.off.G)[slot * 64 + mt];
+        if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+      }
+      if (part < 0 || part == 2) {
+        if (GATE == LNX_GATE_VECTOR) R.Q.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+        else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, mt);
+        R.W.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
 #pragma unroll
-      for (int it = 0; it < Slab::IT; ++it) {
-        const int r = min((mt + 256 * it) / Slab::VPR, 63);
-        R.os[it] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + r] : 0.f;
+        for (int it = 0; it < Slab::IT; ++it) {
+          const int r = min((mt + 256 * it) / Slab::VPR, 63);
+          R.os[it] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + r] : 0.f;
+        }
       }
-      if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = wsp<float>(p, p.off.G)[slot * 64 + mt];
-      if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
     };
     auto commit_rest = [&](const Tiles& R) {
       R.Q.store(sQ, LDK, mt);
@@ -194,22 +199,25 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     };
     auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n - 1
       const int64_t slot = (int64_t)row * N + n;
-      if (n - AHEAD >= c0) fetch(cur, n - AHEAD);  // chunk n's registers are free again
+      const bool more = n - AHEAD >= c0;  // chunk n's registers are free again: they take chunk n - AHEAD
+      if (more) fetch(cur, n - AHEAD, AHEAD == 2 ? 0 : -1);
       if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       lds_barrier();  // B2
       if (n - 1 >= c0) nxt.K.store(sK, LDK, mt);
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+      if (more && AHEAD == 2) fetch(cur, n - AHEAD, 1);
       lds_barrier();  // B3
+      if (more && AHEAD == 2) fetch(cur, n - AHEAD, 2);
       if (n - 1 >= c0) commit_rest(nxt);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
-      fetch(ta, c1 - 1);
+      fetch(ta, c1 - 1, -1);
       ta.K.store(sK, LDK, mt);
       commit_rest(ta);
     }
-    if (AHEAD == 2 && c1 - 2 >= c0) fetch(tb, c1 - 2);
+    if (AHEAD == 2 && c1 - 2 >= c0) fetch(tb, c1 - 2, -1);
     lds_barrier();  // B1 of the first chunk
     if (AHEAD == 2) {
       for (int n = c1 - 1; n >= c0; n -= 2) {
