@@ -128,6 +128,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   const int v0 = blockIdx.y * BV;
   int c0, c1;
   seq_chunks(p.geom, seq, c0, c1);
+  const SeqSpan span = seq_span(p.geom, seq, c0);
 
   if (wave >= 4) {
     // ---------------- movers ----------------
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     auto fetch = [&](Tiles& R, int n, int part) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0, len;
-      chunk_span(p.geom, n, tok0, len);
+      chunk_span(span, n, tok0, len);
       const int64_t tbase = tok_index(p.geom, row, tok0);
       const int64_t tsk = (int64_t)p.geom.ts * DK;
       // vector gate: K e^{G_last - G} and scale Q e^G were stored by the forward pass (all 64 rows defined)

@@ -74,6 +74,25 @@ __device__ __forceinline__ void seq_chunks(const ChunkGeom& g, int s, int& c0, i
   }
 }
 
+// Token range [t0, t1) of the sequence (or batch row) a sequential kernel works on.  Its chunk slots c0, c0 + 1, ...
+// start 64 tokens apart from t0, so the span of a chunk is arithmetic on these three numbers -- the movers of the
+// sequential kernels must not read the chunk table per chunk: a load in the address computation of a fetch makes
+// the fetch wait for every load issued before it.
+struct SeqSpan {
+  int t0, t1, c0;
+};
+__device__ __forceinline__ SeqSpan seq_span(const ChunkGeom& g, int seq, int c0) {
+  SeqSpan s;
+  s.t0 = g.cu ? g.cu[seq] : 0;
+  s.t1 = g.cu ? g.cu[seq + 1] : g.T;
+  s.c0 = c0;
+  return s;
+}
+__device__ __forceinline__ void chunk_span(const SeqSpan& s, int n, int& tok0, int& len) {
+  tok0 = s.t0 + (n - s.c0) * LNX_C;
+  len = min(LNX_C, s.t1 - tok0);
+}
+
 // 1-D launch of `parts` workgroups per chunk slot such that the parts of one slot run on the same
 // XCD (workgroups are dealt round-robin to the 8 XCDs, each with its own L2) and back to back, so
 // the tiles they share are read from HBM once.  Grid size: lnx_xcd_grid(slots, parts).

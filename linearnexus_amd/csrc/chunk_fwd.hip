@@ -519,6 +519,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   const int v0 = blockIdx.y * BV;
   int c0, c1;
   seq_chunks(p.geom, seq, c0, c1);
+  const SeqSpan span = seq_span(p.geom, seq, c0);
 
   if (wave >= 4) {
     // ---------------- movers ----------------
@@ -539,7 +540,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
     ta.tok0 = ta.len = tb.tok0 = tb.len = 0;
     auto fetch = [&](Tiles& R, int n) {
       const int64_t slot = (int64_t)row * N + n;
-      chunk_span(p.geom, n, R.tok0, R.len);
+      chunk_span(span, n, R.tok0, R.len);
       const int64_t tbase = tok_index(p.geom, row, R.tok0);
       const int64_t tsk = (int64_t)p.geom.ts * DK;
       R.W.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
