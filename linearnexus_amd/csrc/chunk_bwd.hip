@@ -124,8 +124,13 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
   int sidx, row, seq;  // state index, (batch, head) row, sequence
-  scan_state(p.geom, blockIdx.x, sidx, row, seq);
-  const int v0 = blockIdx.y * BV;
+  // 1-D grid: the slabs of one (state, head) row get workgroup ids 8 apart, i.e. the same XCD and the same
+  // dispatch wave, so the W / K / Q tiles they both load come from HBM once
+  int64_t chain;
+  int slab;
+  if (!xcd_slot_part((int64_t)(p.geom.tab ? p.geom.nseq : p.geom.rows / p.geom.H) * p.geom.H, p.dv / BV, chain, slab)) return;
+  scan_state(p.geom, (int)chain, sidx, row, seq);
+  const int v0 = slab * BV;
   int c0, c1;
   seq_chunks(p.geom, seq, c0, c1);
   const SeqSpan span = seq_span(p.geom, seq, c0);
@@ -940,7 +945,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
     hipLaunchKernelGGL(bwd_local_kernel<T>, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), 0, st, p);
   }
   lnx_profile_mark("bwd_scan", st);
-  hipLaunchKernelGGL(k1, dim3((unsigned)(nstate * p.geom.H), (unsigned)(p.dv / bv)), dim3(512), b1, st, p);
+  hipLaunchKernelGGL(k1, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(512), b1, st, p);
   lnx_profile_mark("bwd_dqk", st);
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid(slots, DK / 64)), dim3(256), b2, st, p);
   lnx_profile_mark("bwd_wy", st);
