@@ -368,12 +368,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK + ch0;
   const int wi = wave >> 1, wj = wave & 1;
 
-  if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sSS[tid] = 0.f;
-    sMisc[tid] = 0.f;
-  }
-
   // dv is consumed in slabs of SV columns; narrow slabs keep the prefetch registers few enough
   // for three waves per SIMD
   constexpr int SV = 32, LDS_ = SV + Mma<T>::PAD;
@@ -392,7 +386,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   frag_zero(aW);
   frag_zero(aK);
   float ss = 0.f;
-  fetch(0);
+  fetch(0);  // first, so that the small load below does not hold it up
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
+    sSS[tid] = 0.f;
+    sMisc[tid] = 0.f;
+  }
   for (int v0 = 0; v0 < p.dv; v0 += SV) {
     lds_barrier();
     rdO.store(sdO, LDS_, tid);
@@ -626,16 +625,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   const int wi = wave >> 1, wj = wave & 1;
   const int nslab = NKS + p.dv / 64;
 
-  if (tid < 64) {
-    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-    sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
-    sdB[tid] = 0.f;
-    sdGk[tid] = 0.f;
-    sRow[tid] = 0.f;
-    sCol[tid] = 0.f;
-  }
-  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
-
   // dA needs M = dBw W^T + dBu U^T.  With a per-channel gate W and U are read back from the workspace.  Otherwise
   // W = Tm diag(beta e^G) K and U = Tm diag(beta) V give M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T with
   // Zw = dBw K^T and Zu = dBu V^T summed over the slabs already in LDS: W and U are never loaded.
@@ -660,7 +649,17 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   frag_zero(aM);
   frag_zero(aZu);
 
-  fetch(0);
+  fetch(0);  // first, so that the small loads below do not hold it up
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
+    sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
+    sdB[tid] = 0.f;
+    sdGk[tid] = 0.f;
+    sRow[tid] = 0.f;
+    sCol[tid] = 0.f;
+  }
+  stage_tile<T, 64, 64>(sTmT, LDC, wsp<T>(p, p.off.TmT) + slot * 64 * 64, 64, 64, tid);
+
 #pragma unroll 1
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ < NKS;
