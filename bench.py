@@ -33,9 +33,9 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
 TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 864163746, ("gdn_chunk", "chunk_scan"): 1151594310,
-    ("gdn_chunk", "bwd_scan"): 1019454442, ("gdn_chunk", "bwd_dqk"): 1617029406,
-    ("gdn_chunk", "bwd_wy"): 1601705893, ("decode", "decode_step"): 1083428380,
+    ("gdn_chunk", "chunk_prepare"): 895855887, ("gdn_chunk", "chunk_scan"): 1151598250,
+    ("gdn_chunk", "bwd_scan"): 1019451708, ("gdn_chunk", "bwd_dqk"): 1617061650,
+    ("gdn_chunk", "bwd_wy"): 1148897488, ("decode", "decode_step"): 1083425435,
 }
 
 
