@@ -193,7 +193,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
       for (int it = 0; it < Slab::IT; ++it) {
         const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
-        typename Vec16<T>::V o = R.dO.x[it];
+        typename Vec16<T>::V o = R.dO.get(it, mt);
         if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}: (scale Q e^G)^T dO = Q^T (that)
           const float os = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(R.os[it]);
 #pragma unroll
@@ -211,8 +211,8 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       lds_barrier();  // B2
       if (n - 1 >= c0) nxt.K.store(sK, LDK, mt);
+      if (more && AHEAD == 2) fetch(cur, n - AHEAD, 1);  // before the stores below: see the forward scan
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
-      if (more && AHEAD == 2) fetch(cur, n - AHEAD, 1);
       lds_barrier();  // B3
       if (more && AHEAD == 2) fetch(cur, n - AHEAD, 2);
       if (n - 1 >= c0) commit_rest(nxt);

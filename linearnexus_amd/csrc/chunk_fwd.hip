@@ -14,6 +14,8 @@
 // (delta_net.py:296-330 without a gate, kda.py:569-648 with a vector gate); E_ij =
 // exp(G_i - G_j) with G the cumulative log-decay inside the chunk.
 
+#include <type_traits>
+
 #include "chunk_common.h"
 
 namespace {
@@ -573,18 +575,25 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         sMeta[1] = R.len;
       }
     };
-    auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n + 1
+    // cur: chunk n (in LDS already), nxt: chunk n + 1.  `steady` (a std::bool_constant) says that chunks n + 1 and
+    // n + AHEAD exist, so the fetch and the commits are unconditional: behind a conditional fetch the compiler
+    // cannot count how many younger loads are in flight and waits for all of them (the fetch just issued included)
+    // before the first tile store.
+    auto step = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
+      constexpr bool STEADY = decltype(steady)::value;
       const int64_t slot = (int64_t)row * N + n;
       const int tok0 = cur.tok0, len = cur.len;
-      if (n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
+      if (STEADY || n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
       lds_barrier();  // B2
-      if (n + 1 < c1) nxt.W.store(sW, LDK, mt);
+      if (STEADY || n + 1 < c1) nxt.W.store(sW, LDK, mt);
       if (p.save) unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
       lds_barrier();  // B3
-      if (n + 1 < c1) commit_rest(nxt);
+      // the output rows first: the next fetch recycles the registers these stores read, which the compiler
+      // protects with a wait for the stores -- the tile commits in between give them time to complete
       if (FUSE && p.o_dtype == LNX_BF16)
         unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
                                      (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
+      if (STEADY || n + 1 < c1) commit_rest(nxt);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
@@ -596,12 +605,17 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
     lds_barrier();  // B1 of the first chunk
     if (AHEAD == 2) {
       // chunk c0 is in LDS, so set a is free: it takes chunk c0 + 2 in the first step
-      for (int n = c0; n < c1; n += 2) {
-        step(ta, tb, n);
-        if (n + 1 < c1) step(tb, ta, n + 1);
+      int n = c0;
+      for (; n + 3 < c1; n += 2) {  // chunks n + 2 and n + 3 exist
+        step(ta, tb, n, std::true_type{});
+        step(tb, ta, n + 1, std::true_type{});
+      }
+      for (; n < c1; n += 2) {
+        step(ta, tb, n, std::false_type{});
+        if (n + 1 < c1) step(tb, ta, n + 1, std::false_type{});
       }
     } else {
-      for (int n = c0; n < c1; ++n) step(ta, ta, n);
+      for (int n = c0; n < c1; ++n) step(ta, ta, n, std::false_type{});
     }
     return;
   }

@@ -171,23 +171,33 @@ __device__ __forceinline__ typename Vec16<T>::V vec_zero() {
 
 // A [ROWS x COLS] tile held in registers between its global loads and its LDS stores, so that a
 // kernel can issue the loads of all tiles of a phase before it waits for any of them.
-// Rows >= valid are zero-filled.  COLS % VEC == 0.
+// Rows >= valid read as zero.  COLS % VEC == 0.  valid >= 1 (row 0 of the tile must exist).
+// The loads are unconditional and nothing is done to the loaded values until they are used: rows past the end
+// re-read the last valid row and are zeroed when the registers are read (get / store).  A load behind a branch,
+// or under a select, would keep the compiler from counting the loads in flight exactly, and it would then make
+// the next tile store wait for (nearly) all of them, younger prefetches included.
 template <typename T, int ROWS, int COLS> struct TileRegs {
   static constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = (TOTAL + 255) / 256;
-  typename Vec16<T>::V x[IT];
+  typename Vec16<T>::V x[IT];  // raw: use get() unless rows >= valid are excluded otherwise
+  int nvalid;
   __device__ __forceinline__ void load(const T* src, int64_t stride, int valid, int tid) {
+    nvalid = valid;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
-      x[it] = vec_zero<T>();
-      if (idx < TOTAL && r < valid) x[it] = *reinterpret_cast<const typename Vec16<T>::V*>(src + r * stride + c);
+      const int rr = max(min(r, valid - 1), 0);
+      x[it] = *reinterpret_cast<const typename Vec16<T>::V*>(src + rr * stride + c);
     }
+  }
+  __device__ __forceinline__ typename Vec16<T>::V get(int it, int tid) const {
+    const int r = (tid + 256 * it) / VPR;
+    return (r < nvalid) ? x[it] : vec_zero<T>();
   }
   __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
-      if (idx < TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = x[it];
+      if (idx < TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = get(it, tid);
     }
   }
 };
