@@ -171,33 +171,33 @@ __device__ __forceinline__ typename Vec16<T>::V vec_zero() {
 
 // A [ROWS x COLS] tile held in registers between its global loads and its LDS stores, so that a
 // kernel can issue the loads of all tiles of a phase before it waits for any of them.
-// Rows >= valid read as zero.  COLS % VEC == 0.  valid >= 1 (row 0 of the tile must exist).
-// The loads are unconditional and nothing is done to the loaded values until they are used: rows past the end
-// re-read the last valid row and are zeroed when the registers are read (get / store).  A load behind a branch,
-// or under a select, would keep the compiler from counting the loads in flight exactly, and it would then make
-// the next tile store wait for (nearly) all of them, younger prefetches included.
+// Rows >= valid read as zero (valid <= 0: the whole tile).  COLS % VEC == 0.
+// The loads are buffer loads through a descriptor that covers exactly the valid rows: the hardware's range check
+// returns zeros past the end, the per-thread offsets do not depend on the chunk (no address arithmetic in vector
+// registers per load), and no load sits behind a branch or a select -- either would keep the compiler from
+// counting the loads in flight exactly, and it would then make the next tile store wait for (nearly) all of
+// them, younger prefetches included.
 template <typename T, int ROWS, int COLS> struct TileRegs {
   static constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = (TOTAL + 255) / 256;
-  typename Vec16<T>::V x[IT];  // raw: use get() unless rows >= valid are excluded otherwise
-  int nvalid;
+  typename Vec16<T>::V x[IT];
   __device__ __forceinline__ void load(const T* src, int64_t stride, int valid, int tid) {
-    nvalid = valid;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const int bytes = valid > 0 ? (int)(valid * stride * (int64_t)sizeof(T)) : 0;
+    // raw buffer (no stride, no swizzle) of `bytes` bytes; 0x00020000: 32-bit data format, as untyped loads need
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, bytes, 0x00020000);
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
-      const int rr = max(min(r, valid - 1), 0);
-      x[it] = *reinterpret_cast<const typename Vec16<T>::V*>(src + rr * stride + c);
+      const u32x4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)((r * stride + c) * (int64_t)sizeof(T)), 0, 0);
+      x[it] = __builtin_bit_cast(typename Vec16<T>::V, raw);
     }
   }
-  __device__ __forceinline__ typename Vec16<T>::V get(int it, int tid) const {
-    const int r = (tid + 256 * it) / VPR;
-    return (r < nvalid) ? x[it] : vec_zero<T>();
-  }
+  __device__ __forceinline__ typename Vec16<T>::V get(int it, int) const { return x[it]; }
   __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
-      if (idx < TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = get(it, tid);
+      if (idx < TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * ld + c) = x[it];
     }
   }
 };
