@@ -588,8 +588,9 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   // vector-gate epilogue inside the tile region: G and out [64][LDF] fp32, K rows [64][LDC]
   static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * kTile;
   static_assert(GATE != LNX_GATE_VECTOR || vec_bytes <= sizeof(T) * 5 * kTile, "epilogue tiles overlay the loop tiles");
-  // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and (vector gate only) the W/U slab
-  static constexpr int ntile = GATE == LNX_GATE_VECTOR ? 5 : 4;
+  // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and the W/U slab (vector gate) or the first K slab kept for the
+  // epilogue (other gates, dk = 128)
+  static constexpr int ntile = (GATE == LNX_GATE_VECTOR || DK == 128) ? 5 : 4;
   static constexpr size_t bytes = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
 };
 
@@ -610,6 +611,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   T* sdBt = sIn + L::kTile;   // dB slab           [token][col]
   T* sKs = sdBt + L::kTile;   // K / V slab        [token][col]
   T* sWU = sKs + L::kTile;    // W / U slab        [token][col]; vector gate only
+  T* sK0 = sWU;               // other gates: K slab 0 stays here until the epilogue (dk = 128)
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -623,7 +625,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
   const int wi = wave >> 1, wj = wave & 1;
-  const int nslab = NKS + p.dv / 64;
+  // V slabs first, K slabs last: without a per-channel gate the K slabs then stay in LDS for the epilogue
+  const int nvs = p.dv / 64, nslab = NKS + nvs;
+  constexpr bool KEEP_K = GATE != LNX_GATE_VECTOR;
 
   // dA needs M = dBw W^T + dBu U^T.  With a per-channel gate W and U are read back from the workspace.  Otherwise
   // W = Tm diag(beta e^G) K and U = Tm diag(beta) V give M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T with
@@ -631,13 +635,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   constexpr bool LOAD_WU = GATE == LNX_GATE_VECTOR;
   TileRegs<T, 64, 64> rIn, rWU, rKs;  // dW / dD slab [token][col], W / U slab, K / V slab
   auto fetch = [&](int s_) {
-    if (s_ < NKS) {
-      const int c0 = 64 * s_;
+    if (s_ >= nvs) {
+      const int c0 = 64 * (s_ - nvs);
       rIn.load(wsp<T>(p, p.off.dW) + slot * 64 * DK + c0, DK, 64, tid);
       if (LOAD_WU) rWU.load(wsp<T>(p, p.off.W) + slot * 64 * DK + c0, DK, 64, tid);
       rKs.load(kg + c0, tsk, len, tid);
     } else {
-      const int v0 = 64 * (s_ - NKS);
+      const int v0 = 64 * s_;
       rIn.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       if (LOAD_WU) rWU.load(wsp<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, tid);
       rKs.load(vg + v0, tsv, len, tid);
@@ -662,11 +666,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 
 #pragma unroll 1
   for (int s_ = 0; s_ < nslab; ++s_) {
-    const bool is_k = s_ < NKS;
+    const bool is_k = s_ >= nvs;
+    // the K/V slab tile of this iteration: K slab 0 of two goes to its own tile when it is kept
+    T* sKc = (KEEP_K && NKS == 2 && s_ == nvs) ? sK0 : sKs;
     lds_barrier();
     rIn.store(sIn, LDC, tid);
     if (LOAD_WU) rWU.store(sWU, LDC, tid);
-    rKs.store(sKs, LDC, tid);
+    rKs.store(sKc, LDC, tid);
     lds_barrier();
     if (s_ + 1 < nslab) fetch(s_ + 1);
     floatx16 b[1][1];
@@ -676,21 +682,21 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     if (is_k) {
 #pragma unroll
       for (int u = 0; u < NKS; ++u)
-        if (u == s_) {
+        if (u == s_ - nvs) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) aBw[u][0][0][e] = b[0][0][e];
         }
     }
     lds_barrier();
     if (LOAD_WU) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
-    else if (is_k) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
-    else mma_nt<T, 1, 1>(aZu, sdBt + 32 * wi * LDC, LDC, sKs + 32 * wj * LDC, LDC, 64, lane);
+    else if (is_k) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sKc + 32 * wj * LDC, LDC, 64, lane);
+    else mma_nt<T, 1, 1>(aZu, sdBt + 32 * wi * LDC, LDC, sKc + 32 * wj * LDC, LDC, 64, lane);
     if (GATE != LNX_GATE_VECTOR || !is_k) {  // <dB row, k row> / <dB row, v row>; thread = (row, quarter of the slab)
       const int r = tid >> 2, q0 = (tid & 3) * 16;
       float t = 0.f;
 #pragma unroll
       for (int u = 0; u < 16; u += 4) {
-        const floatx4 b4 = load4(sdBt + r * LDC + q0 + u), k4 = load4(sKs + r * LDC + q0 + u);
+        const floatx4 b4 = load4(sdBt + r * LDC + q0 + u), k4 = load4(sKc + r * LDC + q0 + u);
 #pragma unroll
         for (int e = 0; e < 4; ++e) t += b4[e] * k4[e];
       }
@@ -700,7 +706,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     }
     if (!is_k) {  // dv = beta dBu, 16-byte stores
       constexpr int VN = Vec16<T>::N;
-      T* dvg = reinterpret_cast<T*>(p.dv_out) + tbase * p.dv + 64 * (s_ - NKS);
+      T* dvg = reinterpret_cast<T*>(p.dv_out) + tbase * p.dv + 64 * s_;
       for (int idx = tid; idx < 64 * 64 / VN; idx += 256) {
         const int r = idx / (64 / VN), c = (idx % (64 / VN)) * VN;
         if (r < len) {
@@ -820,8 +826,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     }
     return;
   }
-  // K slabs, fetched while the pair terms are formed; the partial dk of bwd_dqk one slab at a time
-  TileRegs<T, 64, 64> rKT[NKS], rdk;
+  // The K slabs are still in LDS (slab 0 of two in its own tile, the last one in the slab tile); the partial dk of
+  // bwd_dqk is fetched one slab at a time.
+  TileRegs<T, 64, 64> rdk;
+  auto k_tile = [&](int u) -> const T* { return (NKS == 2 && u == 0) ? sK0 : sKs; };
   lds_barrier();  // loop tiles dead
   {  // M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T
     floatx16 z[1][1];
@@ -831,22 +839,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     for (int e = 0; e < 16; ++e) z[0][0][e] = aM[0][0][e] * cw + aZu[0][0][e] * cu;
     frag_store<T, 1, 1>(z, sIn + 32 * wi * LDC + 32 * wj, LDC, lane);
     frag_zero(aM);
-#pragma unroll
-    for (int u = 0; u < NKS; ++u) {
-      rKT[u].load(kg + 64 * u, tsk, len, tid);  // K rows again, for Y K
-    }
     lds_barrier();
     mma_x<T, 1, 1, false, true>(aM, sIn + 32 * wi * LDC, LDC, sTmT + 32 * wj, LDC, 64, lane);
-    lds_barrier();  // Z and Tm^T are overwritten below
+    lds_barrier();  // Z is overwritten below
   }
-  // K rows of both slabs into LDS (over the K/V slab tile and Tm^T); X = K K^T is formed here rather than in the
-  // slab loop, where its accumulator would not fit the register budget of three workgroups per CU
-#pragma unroll
-  for (int u = 0; u < NKS; ++u) {
-    T* sKT = (u == 0) ? sKs : sTmT;
-    rKT[u].store(sKT, LDC, tid);
-  }
-  lds_barrier();
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
     floatx16 aX[1][1], y[1][1];
@@ -854,7 +850,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     if (!(wi == 0 && wj == 1)) {
 #pragma unroll
       for (int u = 0; u < NKS; ++u) {
-        const T* sKT = (u == 0) ? sKs : sTmT;
+        const T* sKT = k_tile(u);
         mma_nt<T, 1, 1>(aX, sKT + 32 * wi * LDC, LDC, sKT + 32 * wj * LDC, LDC, 64, lane);
       }
     }
@@ -876,7 +872,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   lds_barrier();
 #pragma unroll
   for (int u = 0; u < NKS; ++u) {
-    const T* sKT = (u == 0) ? sKs : sTmT;
+    const T* sKT = k_tile(u);
     rdk.load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);  // partial dk of bwd_dqk
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
