@@ -33,9 +33,9 @@ PEAK_FP32_MFMA = 157.3  # TFLOP/s
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (see profiles/); None until measured for that (workload, kernel).
 TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 895855887, ("gdn_chunk", "chunk_scan"): 1151598250,
-    ("gdn_chunk", "bwd_scan"): 1019451708, ("gdn_chunk", "bwd_dqk"): 1617061650,
-    ("gdn_chunk", "bwd_wy"): 1148897488, ("decode", "decode_step"): 1083425435,
+    ("gdn_chunk", "chunk_prepare"): 892791394, ("gdn_chunk", "chunk_scan"): 1151619330,
+    ("gdn_chunk", "bwd_scan"): 1019418003, ("gdn_chunk", "bwd_dqk"): 1617145429,
+    ("gdn_chunk", "bwd_wy"): 1084088355, ("decode", "decode_step"): 1083426478,
 }
 
 
