@@ -1,7 +1,7 @@
 """Benchmark of the chunked delta-rule scan on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload gdn_chunk|kda_chunk|deltanet_varlen|deltanet_fp32|decode]
+                    [--workload gdn_chunk|kda_chunk|deltanet_varlen|deltanet_fp32|gdn_dk256|decode|...]
 
 Default workload: Gated DeltaNet chunked forward+backward at B=8, H=16, T=4096, dk=dv=128,
 bf16 q/k/v/dO, fp32 beta/g, chunk 64 (benchmark configuration 2).  One "step" is one forward
@@ -54,15 +54,16 @@ def chunk_flops(dk, dv):
     }
 
 
-def make_gdn_inputs(torch, B, H, T, d, seed, device):
+def make_gdn_inputs(torch, B, H, T, d, seed, device, dv=None):
+    dv = dv or d
     gen = torch.Generator(device="cpu").manual_seed(seed)
     rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
     nrm = lambda x: x / (x.norm(dim=-1, keepdim=True) + 1e-6)
     q, k = nrm(rn(B, H, T, d)), nrm(rn(B, H, T, d))
-    v = rn(B, H, T, d)
+    v = rn(B, H, T, dv)
     beta = torch.sigmoid(rn(B, H, T))
     g = -torch.nn.functional.softplus(rn(B, H, T)) * 0.1
-    dO = rn(B, H, T, d)
+    dO = rn(B, H, T, dv)
     return {n: t.to(device) for n, t in dict(q=q, k=k, v=v, beta=beta, g=g, dO=dO).items()}
 
 
@@ -93,14 +94,17 @@ CHUNK_CONFIGS = {
     "kda_chunk": ("kda", 4, 16, 8192, 128, 0, True, True),           # configuration 3
     "deltanet_varlen": ("delta", 1, 32, 32768, 128, 8, False, True),  # configuration 5
     "deltanet_fp32": ("delta32", 2, 4, 512, 64, 0, False, False),     # configuration 1 (forward only)
+    # head shape of the reference's Gated DeltaNet presets (models.py:142-143: head_dim 256, expand_v 2), 2048 wide
+    "gdn_dk256": ("gated", 8, 8, 4096, (256, 512), 0, False, True),
 }
 
 
 def bench_chunk(args, torch, la, _lib, name):
     variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
-    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5}[name]
-    x = make_gdn_inputs(torch, B, H, T, d, seed, dev)
+    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6}[name]
+    d, dv = d if isinstance(d, tuple) else (d, d)
+    x = make_gdn_inputs(torch, B, H, T, d, seed, dev, dv)
     dt = torch.float32 if variant == "delta32" else torch.bfloat16
     q, k, v, dO = (x[n].to(dt) for n in ("q", "k", "v", "dO"))
     beta, g = x["beta"], x["g"]
@@ -114,7 +118,7 @@ def bench_chunk(args, torch, la, _lib, name):
         cu_np = make_cu_seqlens(seed, nseq, T, 1024, 8192)
         cu = torch.from_numpy(cu_np).to(dev)
         nstate = nseq
-    s0 = (torch.randn(nstate, H, d, d, generator=gen) * 0.02).to(dev) if (with_s0 or nseq) else None
+    s0 = (torch.randn(nstate, H, d, dv, generator=gen) * 0.02).to(dev) if (with_s0 or nseq) else None
     leaves = [q, k, v, beta] + ([g] if variant in ("gated", "kda") else []) + ([s0] if s0 is not None else [])
     if backward:
         for t in leaves:
@@ -166,7 +170,7 @@ def bench_chunk(args, torch, la, _lib, name):
         nchunks = H * int(sum(-(-int(l) // C) for l in (cu_np[1:] - cu_np[:-1])))
     else:
         nchunks = B * H * (-(-T // C))
-    fl = chunk_flops(d, d)
+    fl = chunk_flops(d, dv)
     avg = {n: sum(v_) / len(v_) for n, v_ in per_kernel.items()}
     if "chunk_output" not in avg:  # 2-byte inputs: the scan kernel also forms the outputs
         fl["chunk_scan"] += fl.pop("chunk_output")
@@ -175,14 +179,14 @@ def bench_chunk(args, torch, la, _lib, name):
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
     peak = PEAK_FP32_MFMA if variant == "delta32" else PEAK_BF16
-    total_fl = (3 if backward else 1) * (2 * C * C * (3 * d + 2 * d) + 6 * C * d * d) * nchunks
+    total_fl = (3 if backward else 1) * (2 * C * C * (3 * d + 2 * dv) + 6 * C * d * dv) * nchunks
     out = {
         "metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
         "value": B * T / dtm, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dtm * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if variant == "delta32" else "bf16", "data": "synthetic",
         "config": {"workload": name + ("_fwd_bwd" if backward else "_fwd"), "variant": variant, "B": B, "H": H, "T": T,
-                   "dk": d, "dv": d, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
+                   "dk": d, "dv": dv, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
                    "use_qk_l2norm": False, "inputs": "q,k pre-normalised; fp32 beta/g"},
         "tflops_algorithmic": total_fl / dtm / 1e12,
         "mfma_peak_frac": total_fl / dtm / 1e12 / peak,

@@ -104,6 +104,8 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  * gated_delta_rule_chunkwise (gated_deltanet.py:232-534), kda_chunkwise (kda.py:350-655).
  * The workspace keeps the per-chunk tensors the backward pass re-uses; pass the same
  * workspace, unchanged, to lnx_chunk_bwd (unless forward_only was set).
+ * Shapes: dk in {64, 128, 256} (256 for 2-byte inputs only: the 4-byte tiles of a 256-wide key do not fit LDS;
+ * it is the head_dim of the reference's Gated DeltaNet presets, models.py:142-143), dv a multiple of 64.
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);
@@ -147,7 +149,7 @@ int lnx_conv1d_bwd(const void* x, const float* weight, const float* bias, const 
  * q, k, a, b [B,H,T,dk] and v, o [B,H,T,dv] in `dtype` / `o_dtype`; gk [B,H,T,dk] and the states [B,H,dk,dv] fp32.
  * lnx_dplr_recurrent_fwd replaces dplr_delta_rule_recurrent (rwkv7.py:114-213; initial_state NULL = zeros),
  * lnx_dplr_step replaces dplr_delta_rule_step (rwkv7.py:216-265; token tensors [B,H,d], T ignored, the state is
- * updated in place when final_state == initial_state).  dk in {8,16,32,64,128}, dv a multiple of 4.
+ * updated in place when final_state == initial_state).  dk in {8,16,32,64,128,256}, dv a multiple of 4.
  */
 typedef struct lnx_dplr_args {
   int32_t B, H, T, dk, dv;

@@ -97,8 +97,9 @@ template <typename T, int DK, int BVW = 64> struct BScanCfg {
   // tile fit LDS), so bwd_local does not run
   static constexpr bool FUSE_LOCAL = sizeof(T) == 2;
   static constexpr int kP = FUSE_LOCAL ? 64 * LDC : 0, kRaw = FUSE_LOCAL ? kSlab : 0;
+  static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
-  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * 128;
+  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
 };
 
 template <typename T, int DK, int GATE, int BVW = 64>
@@ -107,8 +108,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   constexpr int LDK = L::LDK, LDU = L::LDU, LDC = L::LDC, BV = L::BV;
   constexpr bool FUSE = L::FUSE_LOCAL;
   constexpr int CT = BV / 32;                      // column tiles of the slab
-  constexpr int NT = (DK == 128) ? CT : 1;         // state tiles per wave (row tile = wave or wave & 1)
-  static_assert(DK == 128 || BV == 64, "dk = 64 needs a 64-column slab");
+  constexpr int RT = (DK >= 128) ? DK / 128 : 1;   // state tiles per wave: RT row tiles (from RT * wave, or wave & 1
+  constexpr int NT = (DK >= 128) ? CT : 1;         //   for dk = 64) x NT column tiles
+  static_assert(DK >= 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
   T* sK = reinterpret_cast<T*>(smem);
   T* sQ = sK + L::kRow;
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       float os[Slab::IT];  // G_i of the dO row each vector belongs to (scalar gate)
       float G;
     };
-    constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;  // chunks fetched ahead (register sets in use)
+    constexpr int AHEAD = (sizeof(T) == 2 && DK <= 128) ? 2 : 1;  // chunks fetched ahead (register sets in use)
     Tiles ta, tb;
     ta.G = tb.G = 0.f;
     // Loads of chunk n into a register set, in three parts (part < 0: all at once).  A CU accepts vector memory
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         }
         if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
       }
-      if (mt < 128) sG[mt] = R.G;
+      if (mt < L::kG) sG[mt] = R.G;
     };
     auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n - 1
       const int64_t slot = (int64_t)row * N + n;
@@ -237,24 +239,26 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   }
 
   // ---------------- compute waves ----------------
-  const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
-  const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
+  const int srow = (DK >= 128) ? 32 * RT * wave : 32 * (wave & 1);
+  const int scol = (DK >= 128) ? 0 : 32 * (wave >> 1);
   // tile of the [64 x BV] token-by-value products owned by this wave (none for CT == 1, wave >= 2)
   const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
   const bool has_tile = (CT == 2) || wave < 2;
 
-  floatx16 dS[1][NT];
+  floatx16 dS[RT][NT];
   frag_zero(dS);
   if (p.d_sT) {
     const float* src = p.d_sT + (int64_t)sidx * DK * p.dv + v0;
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        dS[0][j][e] = src[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          dS[i][j][e] = src[(int64_t)(srow + 32 * i + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
   }
   // dS (gradient of the state leaving the chunk) -> LDS, transposed [dv][dk]; the movers copy it to the workspace
-  if (c0 < c1) frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
+  if (c0 < c1) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
   lds_barrier();  // B1 of the first chunk
   for (int n = c1 - 1; n >= c0; --n) {
     const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
@@ -294,29 +298,35 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
     if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) dS[0][j][e] *= dec;
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) dS[i][j][e] *= dec;
     }
     if (GATE == LNX_GATE_VECTOR) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) dS[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) dS[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
     }
-    mma_x<T, 1, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
-    mma_x<T, 1, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
+    mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+    mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     lds_barrier();  // B3
-    if (n > c0) frag_store_t<T, 1, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
+    if (n > c0) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
     lds_barrier();  // B1 of the next chunk
   }
   if (p.ds0) {
     float* out = p.ds0 + (int64_t)sidx * DK * p.dv + v0;
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        out[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = dS[0][j][e];
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          out[(int64_t)(srow + 32 * i + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = dS[i][j][e];
   }
 }
 
@@ -588,14 +598,14 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   // vector-gate epilogue inside the tile region: G and out [64][LDF] fp32, K rows [64][LDC]
   static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * kTile;
   static_assert(GATE != LNX_GATE_VECTOR || vec_bytes <= sizeof(T) * 5 * kTile, "epilogue tiles overlay the loop tiles");
-  // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and the W/U slab (vector gate) or the first K slab kept for the
-  // epilogue (other gates, dk = 128)
-  static constexpr int ntile = (GATE == LNX_GATE_VECTOR || DK == 128) ? 5 : 4;
+  // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and the W/U slab (vector gate) or all K slabs but the last kept
+  // for the epilogue (other gates)
+  static constexpr int ntile = (GATE == LNX_GATE_VECTOR) ? 5 : 4 + (DK / 64 - 1);
   static constexpr size_t bytes = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2 : 3) : 1)) void bwd_wy2_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || DK > 128 ? 2 : 3) : 1)) void bwd_wy2_kernel(BwdParams p) {
   typedef Wy2Cfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
@@ -611,7 +621,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
   T* sdBt = sIn + L::kTile;   // dB slab           [token][col]
   T* sKs = sdBt + L::kTile;   // K / V slab        [token][col]
   T* sWU = sKs + L::kTile;    // W / U slab        [token][col]; vector gate only
-  T* sK0 = sWU;               // other gates: K slab 0 stays here until the epilogue (dk = 128)
+  T* sK0 = sWU;               // other gates: the K slabs before the last stay here until the epilogue
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -667,8 +677,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
 #pragma unroll 1
   for (int s_ = 0; s_ < nslab; ++s_) {
     const bool is_k = s_ >= nvs;
-    // the K/V slab tile of this iteration: K slab 0 of two goes to its own tile when it is kept
-    T* sKc = (KEEP_K && NKS == 2 && s_ == nvs) ? sK0 : sKs;
+    // the K/V slab tile of this iteration: the K slabs before the last go to tiles of their own when they are kept
+    T* sKc = (KEEP_K && s_ >= nvs && s_ + 1 < nslab) ? sK0 + (s_ - nvs) * L::kTile : sKs;
     lds_barrier();
     rIn.store(sIn, LDC, tid);
     if (LOAD_WU) rWU.store(sWU, LDC, tid);
@@ -826,10 +836,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR ? 2
     }
     return;
   }
-  // The K slabs are still in LDS (slab 0 of two in its own tile, the last one in the slab tile); the partial dk of
+  // The K slabs are still in LDS (the last one in the slab tile, the others in tiles of their own); the partial dk of
   // bwd_dqk is fetched one slab at a time.
   TileRegs<T, 64, 64> rdk;
-  auto k_tile = [&](int u) -> const T* { return (NKS == 2 && u == 0) ? sK0 : sKs; };
+  auto k_tile = [&](int u) -> const T* { return (u + 1 < NKS) ? sK0 + u * L::kTile : sKs; };
   lds_barrier();  // loop tiles dead
   {  // M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T
     floatx16 z[1][1];
@@ -923,12 +933,13 @@ template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
+  constexpr int WIDE = (DK > 128) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;  // dk = 256: only 32 columns fit LDS
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
-  auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, (can_narrow ? 32 : 64)> : bwd_scan_kernel<T, DK, GATE, 64>;
-  const int bv = narrow ? 32 : BScanCfg<T, DK, 64>::BV;
+  auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, NARROW> : bwd_scan_kernel<T, DK, GATE, WIDE>;
+  const int bv = narrow ? BScanCfg<T, DK, NARROW>::BV : BScanCfg<T, DK, WIDE>::BV;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
   auto k3 = bwd_wy2_kernel<T, DK, GATE>;
-  const size_t b1 = narrow ? BScanCfg<T, DK, (can_narrow ? 32 : 64)>::bytes : BScanCfg<T, DK, 64>::bytes;
+  const size_t b1 = narrow ? BScanCfg<T, DK, NARROW>::bytes : BScanCfg<T, DK, WIDE>::bytes;
   const size_t b2 = DqkCfg<T, DK, GATE>::bytes, b3 = Wy2Cfg<T, DK, GATE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
@@ -996,7 +1007,9 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.dv = a->dv; p.gate = a->gate; p.scale = a->scale;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
-    rc = (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+    rc = (a->dk == 256)   ? launch_bwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
+         : (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
+                          : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
   else
     rc = (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st) : launch_bwd_gate<float, 64>(a->gate, p, nstate, st);
   if (rc != LNX_OK) return rc;

@@ -488,8 +488,9 @@ template <typename T, int DK, int BVW = 64> struct ScanSmem {
   static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
   static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr int kQ = FUSE_OUT ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
+  static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
-                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (128 + 4);
+                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (kG + 4);
 };
 
 template <typename T, int DK, int GATE, int BVW = 64>
@@ -497,11 +498,12 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   typedef ScanSmem<T, DK, BVW> L;
   constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDU = BV + L::PAD, LDO = L::LDO;
   constexpr bool FUSE = L::FUSE_OUT;
-  // state tiles: (DK/32) x (BV/32); DK=128: wave w owns row tile w and all column tiles,
-  // DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
+  // state tiles: (DK/32) x (BV/32); DK>=128: wave w owns the RT = DK/128 row tiles from RT * w on and all column
+  // tiles, DK=64: wave w owns row tile (w & 1) and column tile (w >> 1)
   constexpr int CT = BV / 32;
-  constexpr int NT = (DK == 128) ? CT : 1;
-  static_assert(BV == 64 || (BV == 32 && DK == 128), "32-column slabs: the wave's state tile must be a full row tile");
+  constexpr int RT = (DK >= 128) ? DK / 128 : 1;
+  constexpr int NT = (DK >= 128) ? CT : 1;
+  static_assert(BV == 64 || (BV == 32 && DK >= 128), "32-column slabs: the wave's state tile must be a full row tile");
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
   T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   T* sP = sQ + L::kQ;
   bf16_t* sO = reinterpret_cast<bf16_t*>(sP + L::kP);
   float* sG = reinterpret_cast<float*>(sO + (FUSE ? 64 * LDO : 0));
-  int* sMeta = reinterpret_cast<int*>(sG + 128);  // first token and length of the chunk whose tiles are in LDS
+  int* sMeta = reinterpret_cast<int*>(sG + L::kG);  // first token and length of the chunk whose tiles are in LDS
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -539,9 +541,9 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       float G;
       int tok0, len;
     };
-    // register sets: 2-byte inputs are fetched two chunks ahead (two sets used alternately), 4-byte
-    // inputs one chunk ahead (a second set would not fit the register file)
-    constexpr int AHEAD = (sizeof(T) == 2) ? 2 : 1;
+    // register sets: 2-byte inputs are fetched two chunks ahead (two sets used alternately); 4-byte
+    // inputs and dk = 256 one chunk ahead (a second set would not fit the register file)
+    constexpr int AHEAD = (sizeof(T) == 2 && DK <= 128) ? 2 : 1;
     Tiles ta, tb;
     ta.G = tb.G = 0.f;
     ta.tok0 = ta.len = tb.tok0 = tb.len = 0;
@@ -569,7 +571,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         R.Q.store(sQ, LDK, mt);
         R.P.store(sP, LDC, mt);
       }
-      if (mt < 128) sG[mt] = R.G;
+      if (mt < L::kG) sG[mt] = R.G;
       if (mt == 0) {
         sMeta[0] = R.tok0;
         sMeta[1] = R.len;
@@ -621,24 +623,26 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   }
 
   // ---------------- compute waves ----------------
-  const int srow = (DK == 128) ? 32 * wave : 32 * (wave & 1);
-  const int scol = (DK == 128) ? 0 : 32 * (wave >> 1);
+  const int srow = (DK >= 128) ? 32 * RT * wave : 32 * (wave & 1);
+  const int scol = (DK >= 128) ? 0 : 32 * (wave >> 1);
   // this wave's 32x32 tile of the [64 x BV] products (a 32-column slab has two tiles: waves 0 and 1)
   const int wi = (CT == 2) ? (wave >> 1) : wave, wj = (CT == 2) ? (wave & 1) : 0;
   const bool has_tile = (CT == 2) || wave < 2;
 
-  floatx16 S[1][NT];
+  floatx16 S[RT][NT];
   frag_zero(S);
   if (p.s0) {
     const float* s0 = p.s0 + (int64_t)sidx * DK * p.dv + v0;
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        S[0][j][e] = s0[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          S[i][j][e] = s0[(int64_t)(srow + 32 * i + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)];
   }
   // entering state -> LDS, transposed [dv][dk] (B operand of W S and Q S; the movers copy it to the workspace)
-  if (c0 < c1) frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
+  if (c0 < c1) frag_store_t<T, RT, NT>(S, sST + scol * LDK + srow, LDK, lane);
   lds_barrier();  // B1 of the first chunk
   for (int n = c0; n < c1; ++n) {
     // D = U - W S  (one 32x32 tile per wave)
@@ -690,28 +694,34 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
     if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) S[0][j][e] *= dec;
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) S[i][j][e] *= dec;
     }
     if (GATE == LNX_GATE_VECTOR) {  // per state row (key channel)
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) S[0][j][e] *= __expf(sG[srow + frag_row(e, lane)]);
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) S[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
     }
-    mma_x<T, 1, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
+    mma_x<T, RT, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
     lds_barrier();  // B3
-    if (n + 1 < c1) frag_store_t<T, 1, NT>(S, sST + scol * LDK + srow, LDK, lane);
+    if (n + 1 < c1) frag_store_t<T, RT, NT>(S, sST + scol * LDK + srow, LDK, lane);
     lds_barrier();  // B1 of the next chunk
   }
 
   float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0;
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
+  for (int i = 0; i < RT; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e)
-      out[(int64_t)(srow + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = S[0][j][e];
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        out[(int64_t)(srow + 32 * i + frag_row(e, lane)) * p.dv + scol + 32 * j + frag_col(lane)] = S[i][j][e];
 }
 
 // ---------------------------------------------------------------------------------------
@@ -838,14 +848,16 @@ template <typename T, int DK, int GATE>
 int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   auto k1 = PrepSelect<T, DK, GATE>::kernel();
-  // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs)
+  // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs); always for dk = 256,
+  // whose tiles leave no room in LDS for a wider slab
   constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
+  constexpr int WIDE = (DK > 128) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
-  auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, (can_narrow ? 32 : 64)> : chunk_scan_kernel<T, DK, GATE, 64>;
+  auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, NARROW> : chunk_scan_kernel<T, DK, GATE, WIDE>;
   auto k3 = chunk_output_kernel<T, DK, GATE>;
-  const int bv = narrow ? 32 : 64;
+  const int bv = narrow ? NARROW : WIDE;
   const size_t b1 = PrepSelect<T, DK, GATE>::bytes, b3 = OutSmem<T, DK>::bytes;
-  const size_t b2 = narrow ? ScanSmem<T, DK, (can_narrow ? 32 : 64)>::bytes : ScanSmem<T, DK, 64>::bytes;
+  const size_t b2 = narrow ? ScanSmem<T, DK, NARROW>::bytes : ScanSmem<T, DK, WIDE>::bytes;
   hipError_t e;
   if ((e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b1)) != hipSuccess ||
       (e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b2)) != hipSuccess ||
@@ -888,7 +900,10 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (tokens && a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
   if (backward && tokens && a->gate != LNX_GATE_NONE && !a->d_g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs d_g", a->gate);
   if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
-  if (a->dk != 64 && a->dk != 128) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128}, got %d", a->dk);
+  if (a->dk != 64 && a->dk != 128 && a->dk != 256)
+    return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128, 256}, got %d", a->dk);
+  if (a->dk == 256 && a->dtype == LNX_F32)
+    return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take dk = 256 for 2-byte inputs only (the 4-byte tiles do not fit LDS)");
   if (a->dv <= 0 || a->dv % 64 != 0) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dv %% 64 == 0, got %d", a->dv);
   if (a->chunk != LNX_C) return lnx_set_error(LNX_ERR_SHAPE, "chunk length must be %d, got %d", LNX_C, a->chunk);
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
@@ -909,7 +924,7 @@ void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t
 
 extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
   // only the geometry matters here; tensor pointers may still be unset
-  if (!a || a->H <= 0 || a->T < 0 || a->B < 0 || (a->dk != 64 && a->dk != 128) || a->dv <= 0 || a->dv % 64 != 0 ||
+  if (!a || a->H <= 0 || a->T < 0 || a->B < 0 || (a->dk != 64 && a->dk != 128 && a->dk != 256) || a->dv <= 0 || a->dv % 64 != 0 ||
       (a->cu_seqlens && a->nseq <= 0))
     return 0;
   return lnx_chunk_ws_layout(a).total;
@@ -945,7 +960,9 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
-    rc = (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st) : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+    rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
+         : (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
+                          : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
   else
     rc = (a->dk == 128) ? launch_fwd_gate<float, 128>(a->gate, p, nstate, st) : launch_fwd_gate<float, 64>(a->gate, p, nstate, st);
   if (rc != LNX_OK) return rc;
