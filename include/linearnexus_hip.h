@@ -104,8 +104,8 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  * gated_delta_rule_chunkwise (gated_deltanet.py:232-534), kda_chunkwise (kda.py:350-655).
  * The workspace keeps the per-chunk tensors the backward pass re-uses; pass the same
  * workspace, unchanged, to lnx_chunk_bwd (unless forward_only was set).
- * Shapes: dk in {64, 128, 256} (256 for 2-byte inputs only: the 4-byte tiles of a 256-wide key do not fit LDS;
- * it is the head_dim of the reference's Gated DeltaNet presets, models.py:142-143), dv a multiple of 64.
+ * Shapes: dk in {64, 128, 256} (256 is the head_dim of the reference's Gated DeltaNet presets,
+ * models.py:142-143), dv a multiple of 64.
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);

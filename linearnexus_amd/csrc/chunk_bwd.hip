@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 // on request, for dk = 128 with 2-byte inputs when 64-column slabs would leave most CUs idle.
 template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int BV = (DK == 128 && sizeof(T) == 4) ? 32 : BVW;
+  static constexpr int BV = (DK >= 128 && sizeof(T) == 4) ? 32 : BVW;
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
@@ -98,8 +98,11 @@ template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr bool FUSE_LOCAL = sizeof(T) == 2;
   static constexpr int kP = FUSE_LOCAL ? 64 * LDC : 0, kRaw = FUSE_LOCAL ? kSlab : 0;
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
+  // 4-byte inputs with dk = 256: K (read for dD), Q and W (read for the dS update) of a chunk take turns in one tile
+  static constexpr bool SHARE = sizeof(T) == 4 && DK > 128;
+  static constexpr int nRow = SHARE ? 1 : 3;
   // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
-  static constexpr size_t bytes = sizeof(T) * (3 * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
+  static constexpr size_t bytes = sizeof(T) * (nRow * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
 };
 
 template <typename T, int DK, int GATE, int BVW = 64>
@@ -113,9 +116,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   static_assert(DK >= 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
   T* sK = reinterpret_cast<T*>(smem);
-  T* sQ = sK + L::kRow;
-  T* sW = sQ + L::kRow;
-  T* sdO = sW + L::kRow;
+  T* sQ = L::SHARE ? sK : sK + L::kRow;
+  T* sW = L::SHARE ? sK : sQ + L::kRow;
+  T* sdO = sK + L::nRow * L::kRow;
   T* sdDl = sdO + L::kSlab;
   T* sdDT = sdDl + L::kSlab;
   T* sdST = sdDT + L::kdDT;
@@ -137,7 +140,91 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   seq_chunks(p.geom, seq, c0, c1);
   const SeqSpan span = seq_span(p.geom, seq, c0);
 
-  if (wave >= 4) {
+  if constexpr (L::SHARE) {
+    if (wave >= 4) {
+      // ---------------- movers, one tile shared by K, Q and W ----------------
+      // Three more barriers separate the tile's uses; the tiles not in LDS wait in registers.
+      //   B1   K of chunk n in LDS            -> loads of Q, W of chunk n; dS -> workspace
+      //   B2   dD done, K dead                -> Q -> LDS, dD -> workspace
+      //   B2a  Q in LDS (compute: Q^T dO)     -> loads of K and the slabs of chunk n-1
+      //   B2b  Q dead                         -> W -> LDS
+      //   B2c  W in LDS (compute: W^T dD)
+      //   B3   W dead                         -> K and the slabs of chunk n-1 -> LDS
+      const int mt = tid - 256;
+      typedef TileRegs<T, 64, BV> Slab;
+      TileRegs<T, 64, DK> rX, rY;  // X: K, then Q; Y: W
+      Slab rdO, rdD;
+      float os[Slab::IT], rG = 0.f;
+      const int64_t tsk = (int64_t)p.geom.ts * DK;
+      auto tok_base = [&](int n, int& len) {
+        int tok0;
+        chunk_span(span, n, tok0, len);
+        return tok_index(p.geom, row, tok0);
+      };
+      auto fetch_k = [&](int n) {  // K and the slabs of chunk n
+        const int64_t slot = (int64_t)row * N + n;
+        int len;
+        const int64_t tbase = tok_base(n, len);
+        if (GATE == LNX_GATE_VECTOR) rX.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else rX.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
+        rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
+        rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+        if (GATE == LNX_GATE_SCALAR && mt < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + mt];
+        if (GATE == LNX_GATE_VECTOR && mt < DK) rG = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+#pragma unroll
+        for (int it = 0; it < Slab::IT; ++it) {
+          const int r = min((mt + 256 * it) / Slab::VPR, 63);
+          os[it] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + r] : 0.f;
+        }
+      };
+      auto fetch_qw = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        int len;
+        const int64_t tbase = tok_base(n, len);
+        if (GATE == LNX_GATE_VECTOR) rX.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+        else rX.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, mt);
+        rY.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+      };
+      auto commit_k = [&]() {
+        rX.store(sK, LDK, mt);
+        rdD.store(sdDl, LDU, mt);
+#pragma unroll
+        for (int it = 0; it < Slab::IT; ++it) {
+          const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
+          typename Vec16<T>::V o = rdO.get(it, mt);
+          if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}
+            const float f = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(os[it]);
+#pragma unroll
+            for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * f);
+          }
+          if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
+        }
+        if (mt < L::kG) sG[mt] = rG;
+      };
+      if (c0 < c1) {
+        fetch_k(c1 - 1);
+        commit_k();
+      }
+      lds_barrier();  // B1 of the first chunk
+      for (int n = c1 - 1; n >= c0; --n) {
+        const int64_t slot = (int64_t)row * N + n;
+        fetch_qw(n);
+        unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
+        lds_barrier();  // B2
+        rX.store(sQ, LDK, mt);
+        unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+        lds_barrier();  // B2a
+        if (n - 1 >= c0) fetch_k(n - 1);
+        lds_barrier();  // B2b
+        rY.store(sW, LDK, mt);
+        lds_barrier();  // B2c
+        lds_barrier();  // B3
+        if (n - 1 >= c0) commit_k();
+        lds_barrier();  // B1 of the next chunk
+      }
+      return;
+    }
+  } else if (wave >= 4) {
     // ---------------- movers ----------------
     const int mt = tid - 256;
     typedef TileRegs<T, 64, BV> Slab;
@@ -312,7 +399,12 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) dS[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
     }
+    if (L::SHARE) lds_barrier();  // B2a: Q has replaced K in the shared tile
     mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+    if (L::SHARE) {
+      lds_barrier();  // B2b
+      lds_barrier();  // B2c: W has replaced Q
+    }
     mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     lds_barrier();  // B3
     if (n > c0) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
@@ -1011,7 +1103,9 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
          : (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
                           : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
   else
-    rc = (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st) : launch_bwd_gate<float, 64>(a->gate, p, nstate, st);
+    rc = (a->dk == 256)   ? launch_bwd_gate<float, 256>(a->gate, p, nstate, st)
+         : (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st)
+                          : launch_bwd_gate<float, 64>(a->gate, p, nstate, st);
   if (rc != LNX_OK) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk backward launch: %s", hipGetErrorString(e));

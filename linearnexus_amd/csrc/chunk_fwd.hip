@@ -486,7 +486,9 @@ template <typename T, int DK, int BVW = 64> struct ScanSmem {
   static constexpr int BV = BVW;
   static constexpr bool FUSE_OUT = sizeof(T) == 2;
   static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
-  static constexpr int kW = 64 * LDK, kKT = 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
+  // 4-byte inputs with dk = 256: W (read for D) and K (read for the state update) of a chunk take turns in one tile
+  static constexpr bool SHARE = sizeof(T) == 4 && DK > 128;
+  static constexpr int kW = 64 * LDK, kKT = SHARE ? 0 : 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr int kQ = FUSE_OUT ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
@@ -506,8 +508,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   static_assert(BV == 64 || (BV == 32 && DK >= 128), "32-column slabs: the wave's state tile must be a full row tile");
   extern __shared__ __align__(16) char smem[];
   T* sW = reinterpret_cast<T*>(smem);
-  T* sK = sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
-  T* sU = sK + L::kKT; // U rows [token][v], replaced by D
+  T* sK = L::SHARE ? sW : sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
+  T* sU = sW + L::kW + L::kKT;         // U rows [token][v], replaced by D
   T* sST = sU + L::kU;
   T* sDT = sST + L::kST;
   T* sQ = sDT + L::kDT;  // fused output only: Q rows (vector gate: scale Q e^G), P, output staging
@@ -530,7 +532,56 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   seq_chunks(p.geom, seq, c0, c1);
   const SeqSpan span = seq_span(p.geom, seq, c0);
 
-  if (wave >= 4) {
+  if constexpr (L::SHARE) {
+    if (wave >= 4) {
+      // ---------------- movers, one tile shared by W and K ----------------
+      // A fourth barrier (B2') separates the tile's two uses; whichever of W(n+1) and K(n) is not in LDS waits in
+      // registers.  B1: W, U of chunk n in LDS -> loads of W, U of chunk n+1;  B2: K of chunk n -> LDS, D -> workspace;
+      // B2': loads of K of chunk n+1;  B3: W, U of chunk n+1 -> LDS.
+      const int mt = tid - 256;
+      TileRegs<T, 64, DK> rW, rK;
+      TileRegs<T, 64, BV> rU;
+      float rG = 0.f;
+      auto fetch_w = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        rW.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+        rU.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+        if (GATE == LNX_GATE_SCALAR && mt < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + mt];
+        if (GATE == LNX_GATE_VECTOR && mt < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+      };
+      auto fetch_k = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        int tok0, len;
+        chunk_span(span, n, tok0, len);
+        if (GATE == LNX_GATE_VECTOR) rK.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else rK.load(reinterpret_cast<const T*>(p.k) + tok_index(p.geom, row, tok0) * DK, (int64_t)p.geom.ts * DK, len, mt);
+      };
+      auto commit_w = [&]() {
+        rW.store(sW, LDK, mt);
+        rU.store(sU, LDU, mt);
+        if (mt < L::kG) sG[mt] = rG;
+      };
+      if (c0 < c1) {
+        fetch_w(c0);
+        fetch_k(c0);
+        commit_w();
+      }
+      lds_barrier();  // B1 of the first chunk
+      for (int n = c0; n < c1; ++n) {
+        const int64_t slot = (int64_t)row * N + n;
+        if (n + 1 < c1) fetch_w(n + 1);
+        lds_barrier();  // B2
+        rK.store(sK, LDK, mt);
+        if (p.save) unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
+        lds_barrier();  // B2'
+        if (n + 1 < c1) fetch_k(n + 1);
+        lds_barrier();  // B3
+        if (n + 1 < c1) commit_w();
+        lds_barrier();  // B1 of the next chunk
+      }
+      return;
+    }
+  } else if (wave >= 4) {
     // ---------------- movers ----------------
     const int mt = tid - 256;
     struct Tiles {
@@ -690,6 +741,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
                                 (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
       }
     }
+    if (L::SHARE) lds_barrier();  // B2': K has replaced W in the shared tile
     // S <- e^{G_last} S + K^T (D e^{G_last - G})
     if (GATE == LNX_GATE_SCALAR) {
       const float dec = __expf(gl);
@@ -731,8 +783,8 @@ template <typename T, int DK> struct OutSmem {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDK = DK + PAD;
   static constexpr int LDC = LNX_C + PAD;
-  static constexpr int BV = 64;
-  static constexpr size_t bytes = sizeof(T) * (64 * LDK + BV * LDK + 64 * LDC + BV * LDC) + sizeof(float) * 64;
+  static constexpr int BV = (sizeof(T) == 4 && DK > 128) ? 32 : 64;  // 4-byte inputs with dk = 256: LDS capacity
+  static constexpr size_t bytes = sizeof(T) * (64 * LDK + BV * LDK + 64 * LDC + 64 * LDC) + sizeof(float) * 64;  // Q, S^T, P, D
 };
 
 template <typename T, int DK, int GATE>
@@ -744,7 +796,7 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   T* sST = sQ + 64 * LDK;
   T* sP = sST + BV * LDK;
   T* sDT = sP + 64 * LDC;
-  float* sG = reinterpret_cast<float*>(sDT + BV * LDC);
+  float* sG = reinterpret_cast<float*>(sDT + 64 * LDC);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -782,7 +834,9 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
   lds_barrier();
 
-  const int wi = wave >> 1, wj = wave & 1;
+  // one 32x32 tile of the [64 x BV] outputs per wave (a 32-column slab has two: waves 0 and 1)
+  const int wi = (BV == 64) ? (wave >> 1) : wave, wj = (BV == 64) ? (wave & 1) : 0;
+  if (BV == 32 && wave >= 2) return;
   floatx16 acc[1][1];
   frag_zero(acc);
   mma_nt<T, 1, 1>(acc, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
@@ -869,7 +923,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(512), b2, st, p);
   if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
-    hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / 64)), dim3(256), b3, st, p);
+    hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / OutSmem<T, DK>::BV)), dim3(256), b3, st, p);
   }
   lnx_profile_mark(nullptr, st);
   return LNX_OK;
@@ -902,8 +956,6 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
   if (a->dk != 64 && a->dk != 128 && a->dk != 256)
     return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128, 256}, got %d", a->dk);
-  if (a->dk == 256 && a->dtype == LNX_F32)
-    return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take dk = 256 for 2-byte inputs only (the 4-byte tiles do not fit LDS)");
   if (a->dv <= 0 || a->dv % 64 != 0) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dv %% 64 == 0, got %d", a->dv);
   if (a->chunk != LNX_C) return lnx_set_error(LNX_ERR_SHAPE, "chunk length must be %d, got %d", LNX_C, a->chunk);
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
@@ -964,7 +1016,9 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
          : (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
                           : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
   else
-    rc = (a->dk == 128) ? launch_fwd_gate<float, 128>(a->gate, p, nstate, st) : launch_fwd_gate<float, 64>(a->gate, p, nstate, st);
+    rc = (a->dk == 256)   ? launch_fwd_gate<float, 256>(a->gate, p, nstate, st)
+         : (a->dk == 128) ? launch_fwd_gate<float, 128>(a->gate, p, nstate, st)
+                          : launch_fwd_gate<float, 64>(a->gate, p, nstate, st);
   if (rc != LNX_OK) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk forward launch: %s", hipGetErrorString(e));

@@ -1,7 +1,7 @@
 """Key head dimension 256 (the Gated DeltaNet presets of the reference: models.py:142-143, :369-370 use
 head_dim 256 with expand_v 2, i.e. dk = 256, dv = 512): chunk forward and backward for 2-byte inputs against
-the fp64 oracles, for every gate kind, ragged lengths, packed batches and token-first memory.  4-byte inputs
-with dk = 256 are refused.  Metric max|x - ref| / max|ref| <= 2e-2 (bf16 inputs, fp32 accumulation)."""
+the fp64 oracles, for every gate kind, ragged lengths, packed batches and token-first memory.
+Metric max|x - ref| / max|ref| <= 2e-2 (bf16 inputs, fp32 accumulation) or <= 1e-4 (fp32 inputs)."""
 import numpy as np
 import pytest
 import torch
@@ -74,12 +74,36 @@ def test_token_first_dk256():
     assert max_rel(o.float().cpu().numpy(), o_ref) < 2e-2 and max_rel(S.cpu().numpy(), S_ref) < 2e-2
 
 
-def test_fp32_dk256_is_refused():
-    import linearnexus_amd as la
-    x = make_inputs(85, 1, 1, 64, 256, 64)
-    t = lambda n: torch.from_numpy(x[n]).to(DEV)
-    with pytest.raises(RuntimeError, match="dk = 256"):
-        la.delta_rule_chunkwise(t("q"), t("k"), t("v"), t("beta"))
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("shape", [(1, 2, 200, 256, 128), (2, 1, 70, 256, 64), (1, 1, 128, 256, 512)])
+def test_fp32_dk256(gate, shape):
+    """4-byte inputs: K, Q and W of a chunk take turns in one LDS tile in the sequential kernels.  Tolerance 1e-4."""
+    B, H, T, dk, dv = shape
+    x = make_inputs(85, B, H, T, dk, dv, gate=gate, with_state=True, with_grad=True)
+    o_ref, S_ref = oracle_fwd(x, gate)
+    o, S = gpu_chunk_fwd(x, gate, torch.float32)
+    eo, eS = max_rel(o.cpu().numpy(), o_ref), max_rel(S.cpu().numpy(), S_ref)
+    assert eo < 1e-4 and eS < 1e-4, (eo, eS)
+    ref = delta_rule_adjoint(x["q"], x["k"], x["v"], x["beta"], x["dO"], x.get("g"), x["dS"], None, x["S0"], False)
+    check(gpu_grads(x, gate, torch.float32), ref, 1e-4)
+
+
+def test_fp32_dk256_packed():
+    H, T, dk, dv = 2, 300, 256, 128
+    x = make_inputs(86, 1, H, T, dk, dv, gate="scalar", with_grad=True)
+    cu = np.array([0, 64, 70, 200, 300], np.int32)
+    rng = np.random.default_rng(8)
+    x["S0"] = (rng.standard_normal((4, H, dk, dv)) * 0.02).astype(np.float32)
+    x["dS"] = (rng.standard_normal((4, H, dk, dv)) * 0.1).astype(np.float32)
+    parts = []
+    for s in range(4):
+        a, b = cu[s], cu[s + 1]
+        sl = lambda n: x[n][:, :, a:b]
+        parts.append(delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), sl("g"), x["dS"][s:s + 1], None,
+                                        x["S0"][s:s + 1], False))
+    ref = {n: np.concatenate([p[n] for p in parts], axis=2) for n in ("dq", "dk", "dv", "dbeta", "dg")}
+    ref["dS0"] = np.concatenate([p["dS0"] for p in parts], axis=0)
+    check(gpu_grads(x, "scalar", torch.float32, cu=cu), ref, 1e-4)
 
 
 def test_reference_preset_shape_against_token_kernel():
