@@ -353,6 +353,9 @@ class _ChunkScan(torch.autograd.Function):
         return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None
 
 
+_CHUNK_DK = (64, 128, 256)  # key head dimensions the chunk kernels are built for
+
+
 def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, need_mult16, cu_seqlens):
     if need_mult16 and chunk_size % 16 != 0:
         # gated_deltanet.py:318-320, kda.py:438-440
@@ -361,7 +364,23 @@ def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, 
         raise ValueError(f"chunk_size must be positive, got {chunk_size}")
     if scale is None:
         scale = q.shape[-1] ** -0.5
-    return _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+    dk, dv = q.shape[-1], v.shape[-1]
+    dkp = next((c for c in _CHUNK_DK if dk <= c), None)
+    dvp = -(-dv // 64) * 64
+    if dkp is None or q.dim() != 4 or (dkp, dvp) == (dk, dv):
+        return _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+    # Head dimensions between the kernels' sizes (the reference's own tests use dk = 8, 16, dv = 8, 32):
+    # zero channels are exact.  A zero key/query channel adds nothing to any <q,k>, <k,k> or |x|_2, the state rows
+    # and columns it would feed stay zero, and the padded value columns are independent of the others; autograd
+    # slices the gradients back.  `scale` was fixed above from the true dk.
+    pad = torch.nn.functional.pad
+    q, k, v = pad(q, (0, dkp - dk)), pad(k, (0, dkp - dk)), pad(v, (0, dvp - dv))
+    if g is not None and g.dim() == 4 and g.shape[-1] == dk:
+        g = pad(g, (0, dkp - dk))
+    if initial_state is not None:
+        initial_state = pad(initial_state, (0, dvp - dv, 0, dkp - dk))
+    o, sT = _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+    return o[..., :dv], sT[..., :dk, :dv]
 
 
 def delta_rule_chunkwise(q, k, v, beta, initial_state=None, chunk_size=64, scale=None, backend=None, *,
