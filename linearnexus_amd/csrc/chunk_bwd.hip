@@ -100,7 +100,9 @@ template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   // 4-byte inputs with dk = 256: K (read for dD), Q and W (read for the dS update) of a chunk take turns in one tile
   static constexpr bool SHARE = sizeof(T) == 4 && DK > 128;
-  static constexpr int nRow = SHARE ? 1 : 3;
+  // 2-byte inputs with dk = 256 and 64-column slabs: K (read for dD) and Q (read for the dS update) share a tile
+  static constexpr bool SHAREK = sizeof(T) == 2 && DK > 128 && BV == 64;
+  static constexpr int nRow = SHARE ? 1 : SHAREK ? 2 : 3;
   // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
   static constexpr size_t bytes = sizeof(T) * (nRow * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
 };
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   static_assert(DK >= 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
   T* sK = reinterpret_cast<T*>(smem);
-  T* sQ = L::SHARE ? sK : sK + L::kRow;
+  T* sQ = (L::SHARE || L::SHAREK) ? sK : sK + L::kRow;
   T* sW = L::SHARE ? sK : sQ + L::kRow;
   T* sdO = sK + L::nRow * L::kRow;
   T* sdDl = sdO + L::kSlab;
@@ -220,6 +222,83 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         lds_barrier();  // B2c
         lds_barrier();  // B3
         if (n - 1 >= c0) commit_k();
+        lds_barrier();  // B1 of the next chunk
+      }
+      return;
+    }
+  } else if constexpr (L::SHAREK) {
+    if (wave >= 4) {
+      // ---------------- movers, one tile shared by K and Q ----------------
+      // B1: K, W, P, dO of chunk n in LDS -> loads of those of chunk n-1, dS -> workspace;  B2: Q of chunk n -> the K
+      // tile, dD -> workspace;  B2': loads of Q of chunk n-1;  B3: tiles of chunk n-1 -> LDS.
+      const int mt = tid - 256;
+      typedef TileRegs<T, 64, BV> Slab;
+      TileRegs<T, 64, DK> rK, rQ, rW;
+      Slab rdO;
+      TileRegs<T, 64, 64> rP;
+      float os[Slab::IT], rG = 0.f;
+      const int64_t tsk = (int64_t)p.geom.ts * DK;
+      auto fetch_main = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        int tok0, len;
+        chunk_span(span, n, tok0, len);
+        const int64_t tbase = tok_index(p.geom, row, tok0);
+        if (GATE == LNX_GATE_VECTOR) rK.load(wsp<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else rK.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
+        rW.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+        rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
+        rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+        if (GATE == LNX_GATE_SCALAR && mt < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + mt];
+        if (GATE == LNX_GATE_VECTOR && mt < DK) rG = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+#pragma unroll
+        for (int it = 0; it < Slab::IT; ++it) {
+          const int r = min((mt + 256 * it) / Slab::VPR, 63);
+          os[it] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + r] : 0.f;
+        }
+      };
+      auto fetch_q = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        int tok0, len;
+        chunk_span(span, n, tok0, len);
+        if (GATE == LNX_GATE_VECTOR) rQ.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+        else rQ.load(reinterpret_cast<const T*>(p.q) + tok_index(p.geom, row, tok0) * DK, tsk, len, mt);
+      };
+      auto commit_main = [&]() {
+        rK.store(sK, LDK, mt);
+        rW.store(sW, LDK, mt);
+        rP.store(sP, LDC, mt);
+        rdO.store(sdOr, LDU, mt);
+#pragma unroll
+        for (int it = 0; it < Slab::IT; ++it) {
+          const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
+          typename Vec16<T>::V o = rdO.get(it, mt);
+          if (GATE != LNX_GATE_VECTOR) {  // dO rows scaled by scale e^{G_i}
+            const float f = (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(os[it]);
+#pragma unroll
+            for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * f);
+          }
+          if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
+        }
+        if (mt < L::kG) sG[mt] = rG;
+      };
+      if (c0 < c1) {
+        fetch_main(c1 - 1);
+        fetch_q(c1 - 1);
+        commit_main();
+      }
+      lds_barrier();  // B1 of the first chunk
+      for (int n = c1 - 1; n >= c0; --n) {
+        const int64_t slot = (int64_t)row * N + n;
+        if (n - 1 >= c0) fetch_main(n - 1);
+        if (GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
+        unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
+        lds_barrier();  // B2
+        rQ.store(sQ, LDK, mt);
+        unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+        lds_barrier();  // B2'
+        if (n - 1 >= c0) fetch_q(n - 1);
+        lds_barrier();  // B3
+        if (n - 1 >= c0) commit_main();
         lds_barrier();  // B1 of the next chunk
       }
       return;
@@ -399,13 +478,19 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) dS[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
     }
-    if (L::SHARE) lds_barrier();  // B2a: Q has replaced K in the shared tile
-    mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
-    if (L::SHARE) {
-      lds_barrier();  // B2b
-      lds_barrier();  // B2c: W has replaced Q
+    if (L::SHAREK) {  // W first: Q is still on its way into the tile it shares with K
+      mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
+      lds_barrier();  // B2'
+      mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+    } else {
+      if (L::SHARE) lds_barrier();  // B2a: Q has replaced K in the shared tile
+      mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+      if (L::SHARE) {
+        lds_barrier();  // B2b
+        lds_barrier();  // B2c: W has replaced Q
+      }
+      mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     }
-    mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     lds_barrier();  // B3
     if (n > c0) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
     lds_barrier();  // B1 of the next chunk
@@ -1024,8 +1109,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
-  constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
-  constexpr int WIDE = (DK > 128) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;  // dk = 256: only 32 columns fit LDS
+  constexpr bool can_narrow = DK >= 128 && sizeof(T) == 2;
+  constexpr int WIDE = 64, NARROW = can_narrow ? 32 : WIDE;  // 4-byte inputs with dk >= 128 get 32 columns from BScanCfg
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
   auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, NARROW> : bwd_scan_kernel<T, DK, GATE, WIDE>;
   const int bv = narrow ? BScanCfg<T, DK, NARROW>::BV : BScanCfg<T, DK, WIDE>::BV;

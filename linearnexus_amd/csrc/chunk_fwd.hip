@@ -488,8 +488,10 @@ template <typename T, int DK, int BVW = 64> struct ScanSmem {
   static constexpr int LDO = BV + 8;  // staging tile of 2-byte outputs (fp32 outputs go out as 128-byte row segments directly)
   // 4-byte inputs with dk = 256: W (read for D) and K (read for the state update) of a chunk take turns in one tile
   static constexpr bool SHARE = sizeof(T) == 4 && DK > 128;
+  // 2-byte inputs with dk = 256 and 64-column slabs: W (read for D) and Q (read for the outputs) take turns in one tile
+  static constexpr bool SHAREQ = sizeof(T) == 2 && DK > 128 && BV == 64;
   static constexpr int kW = 64 * LDK, kKT = SHARE ? 0 : 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
-  static constexpr int kQ = FUSE_OUT ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
+  static constexpr int kQ = (FUSE_OUT && !SHAREQ) ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
                                   (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (kG + 4);
@@ -512,8 +514,8 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   T* sU = sW + L::kW + L::kKT;         // U rows [token][v], replaced by D
   T* sST = sU + L::kU;
   T* sDT = sST + L::kST;
-  T* sQ = sDT + L::kDT;  // fused output only: Q rows (vector gate: scale Q e^G), P, output staging
-  T* sP = sQ + L::kQ;
+  T* sQ = L::SHAREQ ? sW : sDT + L::kDT;  // fused output only: Q rows (vector gate: scale Q e^G), P, output staging
+  T* sP = sDT + L::kDT + L::kQ;
   bf16_t* sO = reinterpret_cast<bf16_t*>(sP + L::kP);
   float* sG = reinterpret_cast<float*>(sO + (FUSE ? 64 * LDO : 0));
   int* sMeta = reinterpret_cast<int*>(sG + L::kG);  // first token and length of the chunk whose tiles are in LDS
@@ -577,6 +579,71 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         if (n + 1 < c1) fetch_k(n + 1);
         lds_barrier();  // B3
         if (n + 1 < c1) commit_w();
+        lds_barrier();  // B1 of the next chunk
+      }
+      return;
+    }
+  } else if constexpr (L::SHAREQ) {
+    if (wave >= 4) {
+      // ---------------- movers, one tile shared by W and Q ----------------
+      // B1: W, K, U, P of chunk n in LDS -> loads of those of chunk n+1;  B2: Q of chunk n -> the W tile, D ->
+      // workspace;  B2': loads of Q of chunk n+1;  B3: outputs -> global, tiles of chunk n+1 -> LDS.
+      const int mt = tid - 256;
+      TileRegs<T, 64, DK> rW, rK, rQ;
+      TileRegs<T, 64, BV> rU;
+      TileRegs<T, 64, 64> rP;
+      float rG = 0.f;
+      int ftok0 = 0, flen = 0;  // span of the chunk last fetched
+      const int64_t tsk = (int64_t)p.geom.ts * DK;
+      auto fetch_main = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        chunk_span(span, n, ftok0, flen);
+        rW.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+        if (GATE == LNX_GATE_VECTOR) rK.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else rK.load(reinterpret_cast<const T*>(p.k) + tok_index(p.geom, row, ftok0) * DK, tsk, flen, mt);
+        rU.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+        rP.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+        if (GATE == LNX_GATE_SCALAR && mt < 64) rG = ws_ptr<float>(p, p.off.G)[slot * 64 + mt];
+        if (GATE == LNX_GATE_VECTOR && mt < DK) rG = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+      };
+      auto fetch_q = [&](int n) {
+        const int64_t slot = (int64_t)row * N + n;
+        int tok0, len;
+        chunk_span(span, n, tok0, len);
+        if (GATE == LNX_GATE_VECTOR) rQ.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
+        else rQ.load(reinterpret_cast<const T*>(p.q) + tok_index(p.geom, row, tok0) * DK, tsk, len, mt);
+      };
+      auto commit_main = [&]() {
+        rW.store(sW, LDK, mt);
+        rK.store(sK, LDK, mt);
+        rU.store(sU, LDU, mt);
+        rP.store(sP, LDC, mt);
+        if (mt < L::kG) sG[mt] = rG;
+        if (mt == 0) {
+          sMeta[0] = ftok0;
+          sMeta[1] = flen;
+        }
+      };
+      if (c0 < c1) {
+        fetch_main(c0);
+        fetch_q(c0);
+        commit_main();
+      }
+      lds_barrier();  // B1 of the first chunk
+      for (int n = c0; n < c1; ++n) {
+        const int64_t slot = (int64_t)row * N + n;
+        const int tok0 = ftok0, len = flen;
+        if (n + 1 < c1) fetch_main(n + 1);
+        lds_barrier();  // B2
+        rQ.store(sQ, LDK, mt);
+        if (p.save) unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
+        lds_barrier();  // B2'
+        if (n + 1 < c1) fetch_q(n + 1);
+        lds_barrier();  // B3
+        if (p.o_dtype == LNX_BF16)
+          unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
+                                       (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
+        if (n + 1 < c1) commit_main();
         lds_barrier();  // B1 of the next chunk
       }
       return;
@@ -722,45 +789,57 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
     lds_barrier();  // B2
 
-    if (FUSE && has_tile) {
-      // o = scale e^G (Q S) + P D for this slab
-      floatx16 o[1][1];
-      frag_zero(o);
-      mma_nt<T, 1, 1>(o, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
-      if (GATE != LNX_GATE_VECTOR) {
+    auto outputs = [&]() {
+      if (FUSE && has_tile) {
+        // o = scale e^G (Q S) + P D for this slab
+        floatx16 o[1][1];
+        frag_zero(o);
+        mma_nt<T, 1, 1>(o, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+        if (GATE != LNX_GATE_VECTOR) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+          for (int e = 0; e < 16; ++e)
+            o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+        }
+        mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
+        if (p.o_dtype == LNX_BF16) {
+          frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
+        } else {
+          const int tok0 = sMeta[0], len = sMeta[1];
+          frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + (tok_index(p.geom, row, tok0) + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj,
+                                  (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
+        }
       }
-      mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
-      if (p.o_dtype == LNX_BF16) {
-        frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
-      } else {
-        const int tok0 = sMeta[0], len = sMeta[1];
-        frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + (tok_index(p.geom, row, tok0) + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj,
-                                (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
+    };
+    auto update = [&]() {
+      // S <- e^{G_last} S + K^T (D e^{G_last - G})
+      if (GATE == LNX_GATE_SCALAR) {
+        const float dec = __expf(gl);
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) S[i][j][e] *= dec;
       }
+      if (GATE == LNX_GATE_VECTOR) {  // per state row (key channel)
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) S[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
+      }
+      mma_x<T, RT, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
+    };
+    if (L::SHAREQ) {
+      update();
+      lds_barrier();  // B2': Q has replaced W in the shared tile
+      outputs();
+    } else {
+      outputs();
+      if (L::SHARE) lds_barrier();  // B2': K has replaced W in the shared tile
+      update();
     }
-    if (L::SHARE) lds_barrier();  // B2': K has replaced W in the shared tile
-    // S <- e^{G_last} S + K^T (D e^{G_last - G})
-    if (GATE == LNX_GATE_SCALAR) {
-      const float dec = __expf(gl);
-#pragma unroll
-      for (int i = 0; i < RT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) S[i][j][e] *= dec;
-    }
-    if (GATE == LNX_GATE_VECTOR) {  // per state row (key channel)
-#pragma unroll
-      for (int i = 0; i < RT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) S[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
-    }
-    mma_x<T, RT, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
     lds_barrier();  // B3
     if (n + 1 < c1) frag_store_t<T, RT, NT>(S, sST + scol * LDK + srow, LDK, lane);
     lds_barrier();  // B1 of the next chunk
@@ -902,10 +981,10 @@ template <typename T, int DK, int GATE>
 int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
   auto k1 = PrepSelect<T, DK, GATE>::kernel();
-  // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs); always for dk = 256,
-  // whose tiles leave no room in LDS for a wider slab
-  constexpr bool can_narrow = DK == 128 && sizeof(T) == 2;
-  constexpr int WIDE = (DK > 128) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;
+  // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs); always for 4-byte inputs
+  // with dk = 256, whose tiles leave no room in LDS for a wider slab
+  constexpr bool can_narrow = DK >= 128 && sizeof(T) == 2;
+  constexpr int WIDE = (DK > 128 && sizeof(T) == 4) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
   auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, NARROW> : chunk_scan_kernel<T, DK, GATE, WIDE>;
   auto k3 = chunk_output_kernel<T, DK, GATE>;
