@@ -173,8 +173,8 @@ int lnx_dplr_step(const lnx_dplr_args* a, void* hip_stream);
  * RMSNorm with an optional sigmoid gate over the rows of [rows, d] matrices, the output epilogue of the reference's
  * blocks: y = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate).  Replaces FusedRMSNormGated.__call__
  * (linearnexus/modules/linear_attn/kda.py:664-700) and o_norm(o) * sigmoid(g_out) (gated_deltanet.py:854-862).
- * x, gate, y, dy, dx, d_gate in `dtype`; weight, d_weight [d] fp32; gate NULL = no gate; d a multiple of 16 bytes
- * of elements with 4..64 such vectors per row.  d_weight (may be NULL) is summed without atomics through partial rows
+ * x, gate, y, dy, dx, d_gate in `dtype`; weight, d_weight [d] fp32; gate NULL = no gate; d a whole number of
+ * 16-byte vectors, at most 256 of them (rows of 4, 8, 16, 32 or 64 vectors take the faster kernels).  d_weight (may be NULL) is summed without atomics through partial rows
  * in a caller-owned workspace of lnx_rmsnorm_gated_bwd_workspace_bytes bytes.
  */
 int lnx_rmsnorm_gated_fwd(const void* x, const void* gate, const float* weight, void* y, int64_t rows, int32_t d,

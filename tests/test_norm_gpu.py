@@ -21,11 +21,10 @@ def _t(a, dt=None, grad=False):
 
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("gated", [False, True])
-@pytest.mark.parametrize("shape", [(2, 7, 4, 128), (1, 33, 2, 64), (5, 256), (1, 1, 1, 32), (3, 100, 256), (1000, 16)])
+@pytest.mark.parametrize("shape", [(2, 7, 4, 128), (1, 33, 2, 64), (5, 256), (1, 1, 1, 32), (3, 100, 256), (1000, 16),
+                                   (2, 9, 3, 512), (3, 11, 80), (70, 1024), (5, 40), (2, 3, 200)])
 def test_forward_backward_match_oracle(shape, gated, bf16):
     import linearnexus_amd as la
-    if shape[-1] == 16 and bf16:
-        pytest.skip("16 bf16 elements are two 16-byte vectors: below the kernels' four-vector minimum")
     r = np.random.default_rng(91)
     rnd = (lambda a: to_bf16_grid(a.astype(np.float32))) if bf16 else (lambda a: a.astype(np.float32))
     x, g, dy = (rnd(r.standard_normal(shape)) for _ in range(3))
@@ -49,9 +48,11 @@ def test_forward_backward_match_oracle(shape, gated, bf16):
 
 def test_errors_and_empty():
     import linearnexus_amd as la
-    w = torch.ones(24, device=DEV)
+    w = torch.ones(22, device=DEV)
     with pytest.raises(RuntimeError):
-        la.rmsnorm_gated(torch.randn(4, 24, device=DEV), None, w)  # 24 floats = 6 vectors: not a supported row length
+        la.rmsnorm_gated(torch.randn(4, 22, device=DEV), None, w)  # 22 floats: no whole number of 16-byte vectors
+    with pytest.raises(RuntimeError):
+        la.rmsnorm_gated(torch.randn(2, 2048, device=DEV), None, torch.ones(2048, device=DEV))  # 512 vectors: too wide
     with pytest.raises(RuntimeError):
         la.rmsnorm_gated(torch.randn(4, 32), None, torch.ones(32))
     with pytest.raises(RuntimeError):
