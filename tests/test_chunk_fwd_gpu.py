@@ -142,6 +142,6 @@ def test_chunk_equals_recurrent_kernel_at_full_config2_size():
 def test_unsupported_dims_raise_runtime_error():
     # same error type as the reference's accelerated path (kernels/pallas/delta_rule.py:108-115)
     import linearnexus_amd as la
-    q = torch.randn(1, 1, 64, 16, device=DEV)
+    q = torch.randn(1, 1, 64, 272, device=DEV)  # key heads wider than 256 (narrower ones are embedded with zero channels)
     with pytest.raises(RuntimeError):
         la.delta_rule_chunkwise(q, q, torch.randn(1, 1, 64, 64, device=DEV), torch.ones(1, 1, 64, device=DEV))

@@ -96,7 +96,8 @@ def test_orthonormal_keys_closed_form_on_gpu():
 
 @pytest.mark.parametrize("gate", ["none", "scalar", "vector"])
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("shape", [(3, 4, 128, 128), (2, 2, 64, 64), (2, 4, 16, 32), (2, 4, 8, 8), (1, 2, 32, 200)])
+@pytest.mark.parametrize("shape", [(3, 4, 128, 128), (2, 2, 64, 64), (2, 4, 16, 32), (2, 4, 8, 8), (1, 2, 32, 200),
+                                   (2, 3, 256, 512)])
 def test_decode_step_matches_oracle(gate, bf16, shape):
     import linearnexus_amd as la
     B, H, dk, dv = shape
