@@ -96,16 +96,22 @@ CHUNK_CONFIGS = {
     "deltanet_fp32": ("delta32", 2, 4, 512, 64, 0, False, False),     # configuration 1 (forward only)
     # head shape of the reference's Gated DeltaNet presets (models.py:142-143: head_dim 256, expand_v 2), 2048 wide
     "gdn_dk256": ("gated", 8, 8, 4096, (256, 512), 0, False, True),
+    # fp32 inputs (the reference's models run fp32 unless told otherwise): configuration 2's shape and the presets'
+    "gdn_chunk_fp32": ("gated32", 8, 16, 4096, 128, 0, False, True),
+    "gdn_dk256_fp32": ("gated32", 8, 8, 4096, (256, 512), 0, False, True),
 }
 
 
 def bench_chunk(args, torch, la, _lib, name):
     variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
-    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6}[name]
+    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
+            "gdn_chunk_fp32": 2, "gdn_dk256_fp32": 6}[name]
+    fp32 = variant.endswith("32")
+    variant = variant[:-2] if fp32 else variant
     d, dv = d if isinstance(d, tuple) else (d, d)
     x = make_gdn_inputs(torch, B, H, T, d, seed, dev, dv)
-    dt = torch.float32 if variant == "delta32" else torch.bfloat16
+    dt = torch.float32 if fp32 else torch.bfloat16
     q, k, v, dO = (x[n].to(dt) for n in ("q", "k", "v", "dO"))
     beta, g = x["beta"], x["g"]
     gen = torch.Generator(device="cpu").manual_seed(seed + 100)
@@ -178,13 +184,13 @@ def bench_chunk(args, torch, la, _lib, name):
         fl["bwd_scan"] += fl.pop("bwd_local")
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
-    peak = PEAK_FP32_MFMA if variant == "delta32" else PEAK_BF16
+    peak = PEAK_FP32_MFMA if fp32 else PEAK_BF16
     total_fl = (3 if backward else 1) * (2 * C * C * (3 * d + 2 * dv) + 6 * C * d * dv) * nchunks
     out = {
         "metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
         "value": B * T / dtm, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dtm * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if variant == "delta32" else "bf16", "data": "synthetic",
+        "dtype": "f32" if fp32 else "bf16", "data": "synthetic",
         "config": {"workload": name + ("_fwd_bwd" if backward else "_fwd"), "variant": variant, "B": B, "H": H, "T": T,
                    "dk": d, "dv": dv, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
                    "use_qk_l2norm": False, "inputs": "q,k pre-normalised; fp32 beta/g"},
