@@ -325,16 +325,18 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(to_f32(sRow[i * LDC + c]) * fa, to_f32(sK[j * LDC + c]) * fb, acc[u], 0, 0, 0);
       }
     }
-    {  // diagonal blocks: wave = block; lane = (pair of rows rp and 15 - rp, eighth of the half's channels);
-       // the two rows together have 17 columns j <= i
-      const int rp = lane & 7, ce = lane >> 3, r0 = 16 * wave;
-#pragma unroll 1
-      for (int t = 0; t < 17; ++t) {
+    {  // diagonal blocks: wave = block; lane = (row slot, quarter q4 of the half's channels).  Rows rp and 15 - rp
+       // together have 17 columns j <= i; the two slots of a row pair take nine and eight of them.  The quarters are
+       // summed inside the quad, so the only cross-lane traffic is two DPP permutes per value.
+      const int q4 = lane & 3, slot_ = lane >> 2, rp = slot_ & 7, t0 = (slot_ >> 3) * 9, r0 = 16 * wave;
+#pragma unroll 3
+      for (int u = 0; u < 9; ++u) {
+        const int t = min(t0 + u, 16);  // the second slot's ninth pass repeats its eighth and is dropped below
         const bool first = t <= rp;
         const int i = r0 + (first ? rp : 15 - rp), j = r0 + (first ? t : t - rp - 1);
         float x = 0.f, pp = 0.f;
 #pragma unroll
-        for (int c = 8 * ce; c < 8 * ce + 8; c += 4) {
+        for (int c = 16 * q4; c < 16 * q4 + 16; c += 4) {
           const floatx4 ki = load4(sK + i * LDC + c), qi = load4(sQ + i * LDC + c), gi = load4(sG + i * LDF + c);
           const floatx4 kj = load4(sK + j * LDC + c), gj = load4(sG + j * LDF + c);
 #pragma unroll
@@ -344,12 +346,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
             pp += qi[e] * ee;
           }
         }
-#pragma unroll
-        for (int m = 8; m < 64; m <<= 1) {
-          x += __shfl_xor(x, m, LNX_WAVE);
-          pp += __shfl_xor(pp, m, LNX_WAVE);
-        }
-        if (ce == 0) {  // the same lane owns (i, j) in every half
+        x = quad_sum(x);
+        pp = quad_sum(pp);
+        if (q4 == 0 && t0 + u < 17) {  // the same lane owns (i, j) in every half
           sA[i * LNX_LDA + j] += x;
           sT[i * LNX_LDA + j] += pp;
         }

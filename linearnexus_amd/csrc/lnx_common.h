@@ -58,6 +58,13 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 // Sum over all 64 lanes; every lane gets the total.
+// Sum over the four lanes of a quad (lanes 4q .. 4q+3), in every lane: two DPP quad permutes, no LDS crossbar.
+__device__ __forceinline__ float quad_sum(float x) {
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));  // lanes [1,0,3,2]
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));  // lanes [2,3,0,1]
+  return x;
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, LNX_WAVE);
