@@ -14,6 +14,8 @@
 // (delta_net.py:296-330 without a gate, kda.py:569-648 with a vector gate); E_ij =
 // exp(G_i - G_j) with G the cumulative log-decay inside the chunk.
 
+#include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "chunk_common.h"
@@ -32,6 +34,7 @@ struct FwdParams {
   void* o;
   int dv, o_dtype;
   int save;  // write the per-chunk tensors the backward pass (or the separate output kernel) reads
+  int out_spw;  // chunk_output: value slabs per workgroup
   float scale;
   char* ws;
   ChunkWs off;
@@ -878,17 +881,27 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
+  // one workgroup = one chunk and out_spw consecutive value slabs: Q and P are staged once for all of them
+  const int nslab = p.dv / BV, nparts = (nslab + p.out_spw - 1) / p.out_spw;
   int64_t slot;
   int part;
-  if (!xcd_slot_part((int64_t)p.geom.rows * N, p.dv / BV, slot, part)) return;
+  if (!xcd_slot_part((int64_t)p.geom.rows * N, nparts, slot, part)) return;
   const int row = (int)(slot / N), n = (int)(slot % N);
-  const int v0 = part * BV;
+  const int s0 = part * p.out_spw, s1 = min(nslab, s0 + p.out_spw);
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = tok_index(p.geom, row, tok0);
   const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;
 
+  TileRegs<T, BV, DK> rS;   // S_n^T slab [v][dk]
+  TileRegs<T, 64, BV> rD;   // D slab [token][v]
+  auto fetch = [&](int s_) {
+    const int v0 = s_ * BV;
+    rS.load(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, tid);
+    rD.load(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);
+  };
+  fetch(s0);
   if (GATE == LNX_GATE_VECTOR) {
     constexpr int VN = Vec16<T>::N;
     const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
@@ -906,29 +919,36 @@ __global__ __launch_bounds__(256) void chunk_output_kernel(FwdParams p) {
   } else {
     stage_tile<T, 64, DK>(sQ, LDK, reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, len, tid);
   }
-  stage_tile<T, BV, DK>(sST, LDK, ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, BV, tid);
   stage_tile<T, 64, 64>(sP, LDC, ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
-  stage_tile<T, 64, BV>(sDT, LDC, ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, 64, tid);  // D rows [token][v]
   if (tid < 64) sG[tid] = (GATE == LNX_GATE_SCALAR) ? ws_ptr<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
-  lds_barrier();
 
   // one 32x32 tile of the [64 x BV] outputs per wave (a 32-column slab has two: waves 0 and 1)
   const int wi = (BV == 64) ? (wave >> 1) : wave, wj = (BV == 64) ? (wave & 1) : 0;
-  if (BV == 32 && wave >= 2) return;
-  floatx16 acc[1][1];
-  frag_zero(acc);
-  mma_nt<T, 1, 1>(acc, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+  const bool has_tile = BV == 64 || wave < 2;
+#pragma unroll 1
+  for (int s_ = s0; s_ < s1; ++s_) {
+    lds_barrier();  // the previous slab's tiles have been read
+    rS.store(sST, LDK, tid);
+    rD.store(sDT, LDC, tid);
+    lds_barrier();
+    if (s_ + 1 < s1) fetch(s_ + 1);
+    if (has_tile) {
+      floatx16 acc[1][1];
+      frag_zero(acc);
+      mma_nt<T, 1, 1>(acc, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const float gm = (GATE == LNX_GATE_VECTOR) ? 1.f : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
-    acc[0][0][e] *= gm;
+      for (int e = 0; e < 16; ++e) {
+        const float gm = (GATE == LNX_GATE_VECTOR) ? 1.f : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+        acc[0][0][e] *= gm;
+      }
+      mma_x<T, 1, 1, false, true>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj, LDC, 64, lane);
+      const int64_t obase = (tbase + (int64_t)32 * wi * p.geom.ts) * p.dv + s_ * BV + 32 * wj;
+      if (p.o_dtype == LNX_BF16)
+        frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, tsv, lane, len - 32 * wi);
+      else
+        frag_store<float, 1, 1>(acc, reinterpret_cast<float*>(p.o) + obase, tsv, lane, len - 32 * wi);
+    }
   }
-  mma_x<T, 1, 1, false, true>(acc, sP + 32 * wi * LDC, LDC, sDT + 32 * wj, LDC, 64, lane);
-  const int64_t obase = (tbase + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj;
-  if (p.o_dtype == LNX_BF16)
-    frag_store<bf16_t, 1, 1>(acc, reinterpret_cast<bf16_t*>(p.o) + obase, tsv, lane, len - 32 * wi);
-  else
-    frag_store<float, 1, 1>(acc, reinterpret_cast<float*>(p.o) + obase, tsv, lane, len - 32 * wi);
 }
 
 // state-only path for T == 0: final = initial (or zeros)
@@ -1001,7 +1021,12 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(512), b2, st, p);
   if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
-    hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, p.dv / OutSmem<T, DK>::BV)), dim3(256), b3, st, p);
+    // value slabs per workgroup: as many as leave about two thousand workgroups (LNX_OUT_SLABS overrides, for tests)
+    const int nslab = p.dv / OutSmem<T, DK>::BV;
+    FwdParams po = p;
+    po.out_spw = (int)std::max<int64_t>(1, std::min<int64_t>(nslab, slots * nslab / 2048));
+    if (const char* e = getenv("LNX_OUT_SLABS")) po.out_spw = std::max(1, std::min(nslab, atoi(e)));
+    hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, (nslab + po.out_spw - 1) / po.out_spw)), dim3(256), b3, st, po);
   }
   lnx_profile_mark(nullptr, st);
   return LNX_OK;
@@ -1088,6 +1113,7 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   p.sT_out = a->final_state; p.o = a->o; p.dv = a->dv; p.o_dtype = a->o_dtype; p.scale = a->scale;
   // 4-byte inputs form the outputs in a separate kernel that reads the state and D back
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
+  p.out_spw = 1;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)

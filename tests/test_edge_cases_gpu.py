@@ -170,6 +170,19 @@ def test_both_slab_widths_of_the_sequential_kernels(gate, slab, monkeypatch):
     check(gpu_grads(xb, gate, dt), ref, 2e-2)
 
 
+@pytest.mark.parametrize("spw", ["1", "3", "8"])
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("dk,dv", [(128, 320), (256, 160), (64, 192)])
+def test_output_kernel_slabs_per_workgroup(gate, spw, dk, dv, monkeypatch):
+    """4-byte inputs form the outputs in a kernel of their own, which takes several value slabs per workgroup at
+    large shapes (Q and P staged once); LNX_OUT_SLABS forces the count, here with a ragged last group."""
+    monkeypatch.setenv("LNX_OUT_SLABS", spw)
+    x = make_inputs(68, 1, 2, 150, dk, dv, gate=gate, with_state=True)
+    o_ref, S_ref = oracle_fwd(x, gate)
+    o, S = gpu_chunk_fwd(x, gate, torch.float32)
+    assert max_rel(o.cpu().numpy(), o_ref) < 1e-4 and max_rel(S.cpu().numpy(), S_ref) < 1e-4
+
+
 def _tf(x):
     """The same logical [B, H, T, ...] tensor on [B, T, H, ...] memory."""
     return x.transpose(1, 2).contiguous().transpose(1, 2)
