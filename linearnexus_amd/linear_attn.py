@@ -57,6 +57,20 @@ def _f32(t: Tensor) -> Tensor:
     return t.to(torch.float32).contiguous()
 
 
+def _promote(q: Tensor, k: Tensor, v: Tensor):
+    """The reference up-casts q, k, v to float32 whatever they are and returns the output in q's dtype
+    (delta_net.py:170-179, :213; gated_deltanet.py:167-175, :229).  The kernels take one dtype, float32 or bfloat16:
+    anything else -- mixed dtypes (the DeltaNet block normalises q, k in float32 next to a bf16 v,
+    delta_net.py:566-575), float16, float64 -- is computed in float32 and the output cast back to q's dtype.
+    Returns (q, k, v, dtype to cast the output to or None)."""
+    ts = (q, k, v)
+    if not all(isinstance(t, torch.Tensor) and t.is_floating_point() for t in ts):
+        return q, k, v, None  # _check_inputs reports it
+    if q.dtype == k.dtype == v.dtype and q.dtype in _DT:
+        return q, k, v, None
+    return q.to(torch.float32), k.to(torch.float32), v.to(torch.float32), q.dtype
+
+
 # Memory layout of the token tensors.  The ops take the reference's head-first [B, H, T, .] shapes; a caller
 # whose data lives token-first -- [B, T, H, .], what the reference's blocks hold before they transpose
 # (delta_net.py:645-647) -- passes ``x.transpose(1, 2)`` views, and the kernels then read and write that
@@ -151,6 +165,10 @@ class KDAState(_ScanState):
 # --------------------------------------------------------------------------------------
 
 def _step(q, k, v, g, beta, state, scale, l2norm, o_dtype_from_state, inplace):
+    q, k, v, back = _promote(q, k, v)
+    if back is not None:
+        o, s_out = _step(q, k, v, g, beta, state, scale, l2norm, o_dtype_from_state, inplace)
+        return (o if o_dtype_from_state else o.to(back)), s_out
     dt = _check_inputs(q, k, v)
     if q.dim() != 3:
         raise RuntimeError(f"step ops take [B, H, d] vectors, got q {tuple(q.shape)}")
@@ -224,6 +242,10 @@ def _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens):
 
 
 def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):
+    q, k, v, back = _promote(q, k, v)
+    if back is not None:
+        o, sT = _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens)
+        return o.to(back), sT
     dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
     if scale is None:
         scale = dk ** -0.5
@@ -364,6 +386,10 @@ def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, 
         raise ValueError(f"chunk_size must be positive, got {chunk_size}")
     if scale is None:
         scale = q.shape[-1] ** -0.5
+    q, k, v, back = _promote(q, k, v)
+    if back is not None:  # computed in float32; o_dtype is what the caller gets
+        o, sT = _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, torch.float32, need_mult16, cu_seqlens)
+        return o.to(o_dtype), sT
     dk, dv = q.shape[-1], v.shape[-1]
     dkp = next((c for c in _CHUNK_DK if dk <= c), None)
     dvp = -(-dv // 64) * 64

@@ -8,7 +8,7 @@ import torch
 
 from oracle import recurrent as rc
 from oracle.adjoint import delta_rule_adjoint
-from oracle.inputs import make_inputs
+from oracle.inputs import make_inputs, to_bf16_grid
 from conftest import max_rel
 from test_chunk_bwd_gpu import gpu_grads, check, _prep as _prep_bwd
 from test_chunk_fwd_gpu import gpu_chunk_fwd, oracle_fwd, _prep
@@ -240,3 +240,39 @@ def test_token_first_memory_is_used_in_place(gate, bf16, packed):
     o1, S1, _ = run(lambda t: t, False, False)
     o2, S2, _ = run(_tf, False, False)
     assert torch.equal(o1, o2) and torch.equal(S1, S2) and o2.transpose(1, 2).is_contiguous()
+
+
+@pytest.mark.parametrize("kind", ["mixed", "float16", "float64"])
+def test_other_input_dtypes_are_computed_in_float32(kind):
+    """The reference up-casts q, k, v to float32 whatever they are and returns o in q's dtype (delta_net.py:170-179,
+    :213).  Its DeltaNet block hands float32 q, k (normalised in float32, delta_net.py:566-575) next to a v in the model
+    dtype; float16 and float64 inputs go the same way.  Chunk (with gradients), token scan and decode step."""
+    import linearnexus_amd as la
+    x = make_inputs(69, 1, 2, 100, 64, 64, gate="scalar", with_state=True, with_grad=True)
+    if kind == "mixed":
+        x["v"] = to_bf16_grid(x["v"])
+        dts = (torch.float32, torch.float32, torch.bfloat16)
+    elif kind == "float16":
+        for n in ("q", "k", "v"):
+            x[n] = x[n].astype(np.float16).astype(np.float32)
+        dts = (torch.float16,) * 3
+    else:
+        dts = (torch.float64,) * 3
+    q, k, v = (torch.from_numpy(x[n]).to(DEV).to(dt).requires_grad_(True) for n, dt in zip(("q", "k", "v"), dts))
+    g, beta, s0 = (torch.from_numpy(x[n]).to(DEV) for n in ("g", "beta", "S0"))
+    o_ref, S_ref = oracle_fwd(x, "scalar")
+    tol = 2e-3 if kind == "float16" else 1e-4  # o is rounded to q's dtype on the way out
+    o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, s0, 64, False)
+    assert o.dtype == dts[0] and S.dtype == torch.float32
+    assert max_rel(o.detach().float().cpu().numpy(), o_ref) < tol and max_rel(S.detach().cpu().numpy(), S_ref) < 1e-4
+    (o.float() * torch.from_numpy(x["dO"]).to(DEV)).sum().backward()
+    ref = delta_rule_adjoint(x["q"], x["k"], x["v"], x["beta"], x["dO"], x["g"], None, None, x["S0"], False)
+    assert q.grad.dtype == dts[0] and v.grad.dtype == dts[2]
+    gtol = 2e-2 if kind != "float64" else 1e-4  # gradients come back rounded to the leaves' dtypes
+    for n, t in (("dq", q), ("dk", k), ("dv", v)):
+        assert max_rel(t.grad.float().cpu().numpy(), ref[n]) < gtol, n
+    o2, S2 = la.gated_delta_rule_recurrent(q.detach(), k.detach(), v.detach(), g, beta, None, s0, False)
+    assert o2.dtype == dts[0] and max_rel(o2.float().cpu().numpy(), o_ref) < tol and max_rel(S2.cpu().numpy(), S_ref) < 1e-4
+    o3, S3 = la.gated_delta_rule_step(q.detach()[:, :, 0], k.detach()[:, :, 0], v.detach()[:, :, 0], g[:, :, 0], beta[:, :, 0], s0,
+                                      use_qk_l2norm=False)
+    assert o3.dtype == dts[0] and max_rel(o3.float().cpu().numpy(), o_ref[:, :, 0]) < tol
