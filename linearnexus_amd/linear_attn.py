@@ -135,29 +135,50 @@ def _base_args(B, H, T, dk, dv, dtype, o_dtype, gate, l2norm, scale) -> ScanArgs
 # --------------------------------------------------------------------------------------
 
 @dataclass
-class _ScanState:
+class DeltaNetState:
+    """Cache for DeltaNet generation (delta_net.py:81-118): ``S [batch, heads, key_dim, value_dim]`` float32 and the
+    conv cache ``[batch, kernel-1, channels]`` of the block's one convolution over the concatenated q, k, v."""
     S: Tensor
     conv_state: Optional[Tensor] = None
 
     @classmethod
-    def zeros(cls, batch_size, num_heads, key_dim, value_dim, conv_channels=None, conv_size=4, device="cuda"):
+    def zeros(cls, batch_size, num_heads, key_dim, value_dim, conv_channels=None, conv_size=4, *, device="cuda"):
         S = torch.zeros(batch_size, num_heads, key_dim, value_dim, dtype=torch.float32, device=device)
-        conv = None
+        conv_state = None
         if conv_channels is not None:
-            conv = torch.zeros(batch_size, conv_size - 1, conv_channels, dtype=torch.float32, device=device)
-        return cls(S=S, conv_state=conv)
+            conv_state = torch.zeros(batch_size, conv_size - 1, conv_channels, dtype=torch.float32, device=device)
+        return cls(S=S, conv_state=conv_state)
 
 
-class DeltaNetState(_ScanState):
-    pass
+@dataclass
+class _GatedState:
+    """``S [batch, num_v_heads, key_dim_per_head, value_dim_per_head]`` float32 and one conv cache each for q, k
+    (``[batch, kernel-1, key_dim_total]``) and v (``[batch, kernel-1, value_dim]``)."""
+    S: Tensor
+    conv_state_q: Optional[Tensor] = None
+    conv_state_k: Optional[Tensor] = None
+    conv_state_v: Optional[Tensor] = None
+
+    @classmethod
+    def zeros(cls, batch_size, num_v_heads, key_dim_per_head, value_dim_per_head, key_dim_total=None, value_dim=None,
+              conv_size=4, use_conv=True, *, device="cuda"):
+        z = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device=device)
+        state = cls(S=z(batch_size, num_v_heads, key_dim_per_head, value_dim_per_head))
+        if use_conv and key_dim_total is not None and value_dim is not None:
+            state.conv_state_q = z(batch_size, conv_size - 1, key_dim_total)
+            state.conv_state_k = z(batch_size, conv_size - 1, key_dim_total)
+            state.conv_state_v = z(batch_size, conv_size - 1, value_dim)
+        return state
 
 
-class GatedDeltaNetState(_ScanState):
-    pass
+@dataclass
+class GatedDeltaNetState(_GatedState):
+    """Cache for Gated DeltaNet generation (gated_deltanet.py:72-128)."""
 
 
-class KDAState(_ScanState):
-    pass
+@dataclass
+class KDAState(_GatedState):
+    """Cache for KDA generation (kda.py:57-113)."""
 
 
 # --------------------------------------------------------------------------------------

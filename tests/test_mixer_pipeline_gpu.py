@@ -153,3 +153,40 @@ def test_kda_mixer_forward_and_backward_fp32(shape):
     errs = {"y": rel(y, y_ref), "S": rel(S, S_ref), **{"d" + n: rel(g[n], g_ref[n]) for n in g_ref}}
     bad = {n: e for n, e in errs.items() if not e < 1e-4}
     assert not bad, (bad, errs)
+
+
+def test_prefill_then_token_by_token_decode_equals_whole_sequence():
+    """Generation the way the reference's block runs it (gated_deltanet.py:756-779, :829-841, :868-876): the prompt goes
+    through the chunk path once and leaves a GatedDeltaNetState (scan state + the three conv caches); every further
+    token is one conv step on the caches and one gated_delta_rule_step.  The outputs must equal the whole sequence
+    through the chunk path (the step-by-step == whole-sequence property of tests/test_comprehensive.py:57-83)."""
+    import linearnexus_amd as la
+    B, T, H, dk, dv, K, T0 = 2, 90, 2, 64, 128, 4, 70
+    x = {n: torch.from_numpy(a).to(DEV) for n, a in _inputs(98, B, T, H, dk, dv, K).items()}
+
+    def mixer(sl, state):
+        q, cq = la.depthwise_conv1d_causal(x["q"][:, sl], x["wq"], None, cache=state.conv_state_q, activation="silu")
+        k, ck = la.depthwise_conv1d_causal(x["k"][:, sl], x["wk"], None, cache=state.conv_state_k, activation="silu")
+        v, cv = la.depthwise_conv1d_causal(x["v"][:, sl], x["wv"], None, cache=state.conv_state_v, activation="silu")
+        n = q.shape[1]
+        q, k, v = (t.view(B, n, H, -1).transpose(1, 2) for t in (q, k, v))
+        beta = torch.sigmoid(x["b"][:, sl]).transpose(1, 2)
+        g = (-torch.exp(x["A_log"]) * torch.nn.functional.softplus(x["a"][:, sl] + x["dt_bias"])).transpose(1, 2)
+        if n == 1:
+            o, S = la.gated_delta_rule_step(q[:, :, 0], k[:, :, 0], v[:, :, 0], g[:, :, 0], beta[:, :, 0], state.S)
+            o = o[:, :, None]
+        else:
+            o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, state.S, 64, True)
+        y = la.rmsnorm_gated(o.transpose(1, 2), x["gate"][:, sl], x["norm_w"])
+        return y, la.GatedDeltaNetState(S=S, conv_state_q=cq, conv_state_k=ck, conv_state_v=cv)
+
+    zero = lambda: la.GatedDeltaNetState.zeros(B, H, dk, dv, key_dim_total=H * dk, value_dim=H * dv, conv_size=K)
+    y_full, s_full = mixer(slice(0, T), zero())
+    y, state = mixer(slice(0, T0), zero())
+    assert (y - y_full[:, :T0]).abs().max() <= 1e-4 * y_full.abs().max()
+    for t in range(T0, T):
+        y, state = mixer(slice(t, t + 1), state)
+        assert (y[:, 0] - y_full[:, t]).abs().max() <= 1e-4 * y_full.abs().max(), t
+    assert (state.S - s_full.S).abs().max() <= 1e-4 * s_full.S.abs().max()
+    for n in ("conv_state_q", "conv_state_k", "conv_state_v"):
+        assert torch.equal(getattr(state, n), getattr(s_full, n))

@@ -1,0 +1,36 @@
+"""The generation caches mirror the reference's dataclasses field for field and argument for argument
+(delta_net.py:81-118, gated_deltanet.py:72-128, kda.py:57-113), so a caller's ``State.zeros(...)`` lines keep working."""
+import dataclasses
+import inspect
+
+import pytest
+import torch
+
+import linearnexus_amd as la
+
+
+def test_deltanet_state():
+    assert [f.name for f in dataclasses.fields(la.DeltaNetState)] == ["S", "conv_state"]
+    names = list(inspect.signature(la.DeltaNetState.zeros).parameters)
+    assert names[:6] == ["batch_size", "num_heads", "key_dim", "value_dim", "conv_channels", "conv_size"]
+    s = la.DeltaNetState.zeros(2, 3, 16, 32, device="cpu")
+    assert tuple(s.S.shape) == (2, 3, 16, 32) and s.S.dtype == torch.float32 and s.conv_state is None
+    assert not s.S.any()
+    s = la.DeltaNetState.zeros(2, 3, 16, 32, conv_channels=3 * (16 + 16 + 32), conv_size=4, device="cpu")
+    assert tuple(s.conv_state.shape) == (2, 3, 192)
+
+
+@pytest.mark.parametrize("cls", [la.GatedDeltaNetState, la.KDAState])
+def test_gated_and_kda_states(cls):
+    assert [f.name for f in dataclasses.fields(cls)] == ["S", "conv_state_q", "conv_state_k", "conv_state_v"]
+    names = list(inspect.signature(cls.zeros).parameters)
+    assert names[:8] == ["batch_size", "num_v_heads", "key_dim_per_head", "value_dim_per_head", "key_dim_total",
+                         "value_dim", "conv_size", "use_conv"]
+    s = cls.zeros(2, 4, 256, 512, device="cpu")
+    assert isinstance(s, cls) and tuple(s.S.shape) == (2, 4, 256, 512) and s.S.dtype == torch.float32
+    assert s.conv_state_q is None and s.conv_state_k is None and s.conv_state_v is None
+    s = cls.zeros(2, 4, 256, 512, key_dim_total=1024, value_dim=2048, conv_size=4, device="cpu")
+    assert tuple(s.conv_state_q.shape) == (2, 3, 1024) and tuple(s.conv_state_k.shape) == (2, 3, 1024)
+    assert tuple(s.conv_state_v.shape) == (2, 3, 2048)
+    s = cls.zeros(2, 4, 256, 512, key_dim_total=1024, value_dim=2048, use_conv=False, device="cpu")
+    assert s.conv_state_q is None
