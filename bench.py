@@ -36,6 +36,10 @@ TRAFFIC = {
     ("gdn_chunk", "chunk_prepare"): 892791394, ("gdn_chunk", "chunk_scan"): 1151619330,
     ("gdn_chunk", "bwd_scan"): 1019418003, ("gdn_chunk", "bwd_dqk"): 1617145429,
     ("gdn_chunk", "bwd_wy"): 1084088355, ("decode", "decode_step"): 1083426478,
+    ("gdn_dk256", "chunk_prepare"): 1144179908, ("gdn_dk256", "chunk_scan"): 2350101812,
+    ("gdn_dk256", "bwd_scan"): 2082675160, ("gdn_dk256", "bwd_dqk"): 3686681985, ("gdn_dk256", "bwd_wy"): 1381163915,
+    ("kda_chunk", "chunk_prepare"): 2082771134, ("kda_chunk", "chunk_scan"): 1287886410,
+    ("kda_chunk", "bwd_scan"): 1019391118, ("kda_chunk", "bwd_dqk"): 2732077910, ("kda_chunk", "bwd_wy"): 2664907117,
 }
 
 
