@@ -8,6 +8,8 @@ Metric max|x - ref| / max|ref| <= 1e-4 (fp32) or 2e-2 (bf16 activations).  In bf
 gradients, sums of B*T signed terms, are measured against the sum of the terms' magnitudes, at 5e-2: the error of
 dg_t, a reverse cumulative sum inside each chunk, is shared by the tokens before t and does not average out over the
 sum (the fp32 run of the same pipeline pins the algebra at 1e-4)."""
+import dataclasses
+
 import numpy as np
 import pytest
 import torch
@@ -190,3 +192,51 @@ def test_prefill_then_token_by_token_decode_equals_whole_sequence():
     assert (state.S - s_full.S).abs().max() <= 1e-4 * s_full.S.abs().max()
     for n in ("conv_state_q", "conv_state_k", "conv_state_v"):
         assert torch.equal(getattr(state, n), getattr(s_full, n))
+
+
+def test_whole_mixer_decode_step_replayed_from_one_graph():
+    """Serving: one token of the whole mixer (three conv steps on their caches, gates, the decode step on the state
+    in place, gated RMSNorm) captured once in a HIP graph; every replay on new token inputs must equal the eager
+    step bit for bit, with eager work and synchronisations between the replays."""
+    import linearnexus_amd as la
+    B, T, H, dk, dv, K = 4, 12, 3, 256, 512, 4
+    x = {n: torch.from_numpy(a).to(DEV) for n, a in _inputs(99, B, T, H, dk, dv, K).items()}
+
+    def new_state():
+        return la.GatedDeltaNetState.zeros(B, H, dk, dv, key_dim_total=H * dk, value_dim=H * dv, conv_size=K)
+
+    def step(tok, st):  # tok: dict of [B, 1, ...] inputs of one token; the state is updated in place
+        q, _ = la.depthwise_conv1d_causal(tok["q"], x["wq"], None, cache=st.conv_state_q, activation="silu", inplace_cache=True)
+        k, _ = la.depthwise_conv1d_causal(tok["k"], x["wk"], None, cache=st.conv_state_k, activation="silu", inplace_cache=True)
+        v, _ = la.depthwise_conv1d_causal(tok["v"], x["wv"], None, cache=st.conv_state_v, activation="silu", inplace_cache=True)
+        beta = torch.sigmoid(tok["b"][:, 0])
+        g = -torch.exp(x["A_log"]) * torch.nn.functional.softplus(tok["a"][:, 0] + x["dt_bias"])
+        o, _ = la.gated_delta_rule_step(q.view(B, H, dk), k.view(B, H, dk), v.view(B, H, dv), g, beta, st.S, inplace=True)
+        return la.rmsnorm_gated(o, tok["gate"][:, 0], x["norm_w"])
+
+    names = ("q", "k", "v", "a", "b", "gate")
+    token = lambda t: {n: x[n][:, t:t + 1].contiguous() for n in names}
+    eager_state, graph_state = new_state(), new_state()
+    static = {n: torch.zeros_like(v_) for n, v_ in token(0).items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(static, new_state())  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph):
+        y_static = step(static, graph_state)
+    for f in dataclasses.fields(graph_state):  # the capture itself ran nothing: start from zeros
+        getattr(graph_state, f.name).zero_()
+    for t in range(T):
+        for n in names:
+            static[n].copy_(token(t)[n])
+        graph.replay()
+        y_graph = y_static.clone()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            y_eager = step(token(t), eager_state)  # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_eager), t
+        for f in dataclasses.fields(graph_state):
+            assert torch.equal(getattr(graph_state, f.name), getattr(eager_state, f.name)), (t, f.name)
