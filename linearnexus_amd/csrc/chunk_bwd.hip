@@ -515,17 +515,22 @@ template <typename T, int DK, int GATE> struct DqkCfg {
   static constexpr int PAD = Mma<T>::PAD;
   static constexpr int LDC = LNX_C + PAD, LDF = 64 + 4;
   static constexpr int kTile = 64 * LDC;
-  // loop phase: dO, D, dD, S_n, dS_n tiles; scalar epilogue: dPe, dPe^T, K^T, Q^T + one staging tile
-  static constexpr size_t loop_bytes = sizeof(T) * 5 * kTile;
+  // loop phase: dO, D, dD slabs [64][SV] and S_n, dS_n slabs [SV][64], five tiles of kLoop elements
+  static constexpr int SV = 32, LDSV = SV + PAD;
+  static constexpr int kLoop = (64 * LDSV > SV * LDC) ? 64 * LDSV : SV * LDC;
+  static constexpr size_t loop_bytes = sizeof(T) * 5 * kLoop;
+  // scalar epilogue: dPe, K rows, Q rows and one staging tile (dW, then dk), four [64][64] tiles
+  static constexpr size_t scalar_bytes = sizeof(T) * 4 * kTile;
   // vector epilogue: alpha, out (fp32 [64][LDF]) and K, Q rows, plus dP in fp32
   static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * 2 * kTile;
-  static constexpr size_t big = (GATE == LNX_GATE_VECTOR && vec_bytes > loop_bytes) ? vec_bytes : loop_bytes;
+  static constexpr size_t epi_bytes = (GATE == LNX_GATE_VECTOR) ? vec_bytes : scalar_bytes;
+  static constexpr size_t big = epi_bytes > loop_bytes ? epi_bytes : loop_bytes;
   static constexpr int kSmall = 64 * 4 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0);  // floats
   static constexpr size_t bytes = sizeof(float) * kSmall + big;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3 : 1)) void bwd_dqk_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 ? 3 : 2)) void bwd_dqk_kernel(BwdParams p) {
   typedef DqkCfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF;
   extern __shared__ __align__(16) char smem[];
@@ -534,10 +539,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
   float* sMisc = sSS + 64;  // [0] = sum_j r_j <dKr_j, k_j>, [1] = <dS_n, S_n>
   float* sR = sMisc + 64;   // vector gate only: dP [64][LNX_LDA]
   T* sdO = reinterpret_cast<T*>(sMisc + 64 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0));
-  T* sD = sdO + L::kTile;
-  T* sdD = sD + L::kTile;
-  T* sSn = sdD + L::kTile;
-  T* sdSn = sSn + L::kTile;
+  T* sD = sdO + L::kLoop;
+  T* sdD = sD + L::kLoop;
+  T* sSn = sdD + L::kLoop;
+  T* sdSn = sSn + L::kLoop;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -557,7 +562,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
 
   // dv is consumed in slabs of SV columns; narrow slabs keep the prefetch registers few enough
   // for three waves per SIMD
-  constexpr int SV = 32, LDS_ = SV + Mma<T>::PAD;
+  constexpr int SV = L::SV, LDS_ = L::LDSV;
   TileRegs<T, 64, SV> rdO, rD, rdD;
   TileRegs<T, SV, 64> rSn, rdSn;  // S_n and dS_n slabs stay [v][c]: contracted along their rows
   auto fetch = [&](int v0) {
@@ -688,11 +693,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 && GATE != LNX_GATE_VECTOR ? 3
     }
   } else {
     // ---- scalar / no gate ----
-    T* sPe = sdO;     // scale E dP   [i][j]
-    T* sOut2 = sD;    // staging for dk
-    T* sKr = sdD;     // K rows of this half [token][c]
-    T* sQr = sSn;     // Q rows
-    T* sOut = sdSn;
+    T* sPe = sdO;                 // scale E dP   [i][j]
+    T* sKr = sPe + L::kTile;      // K rows of this half [token][c]
+    T* sQr = sKr + L::kTile;      // Q rows
+    T* sOut = sQr + L::kTile;     // staging for dW ...
+    T* sOut2 = sOut;              // ... and, once dW has left, for dk
     TileRegs<T, 64, 64> rKT, rQT;
     rKT.load(kg, tsk, len, tid);
     rQT.load(qg, tsk, len, tid);
