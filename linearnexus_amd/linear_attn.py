@@ -57,6 +57,13 @@ def _f32(t: Tensor) -> Tensor:
     return t.to(torch.float32).contiguous()
 
 
+def _wants_grad(*tensors) -> bool:
+    """The reference's token-by-token ops are differentiable like everything in JAX, and its blocks call them while
+    training (sequences of at most 32 tokens, gated_deltanet.py:836-846).  The token kernels have no backward pass;
+    when a gradient is wanted the same function is computed by the chunk kernels, which have one."""
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 def _promote(q: Tensor, k: Tensor, v: Tensor):
     """The reference up-casts q, k, v to float32 whatever they are and returns the output in q's dtype
     (delta_net.py:170-179, :213; gated_deltanet.py:167-175, :229).  The kernels take one dtype, float32 or bfloat16:
@@ -193,6 +200,13 @@ def _step(q, k, v, g, beta, state, scale, l2norm, o_dtype_from_state, inplace):
     dt = _check_inputs(q, k, v)
     if q.dim() != 3:
         raise RuntimeError(f"step ops take [B, H, d] vectors, got q {tuple(q.shape)}")
+    if _wants_grad(q, k, v, g, beta, state):
+        if inplace:
+            raise RuntimeError("inplace=True overwrites the state a backward pass would need")
+        o, s_out = _chunk(q[:, :, None], k[:, :, None], v[:, :, None], None if g is None else g[:, :, None],
+                          _squeeze_beta(beta, 3)[:, :, None], scale, state, CHUNK, l2norm,
+                          torch.float32 if o_dtype_from_state else q.dtype, False, None)
+        return o[:, :, 0], s_out
     B, H, dk = q.shape
     dv = v.shape[-1]
     beta = _squeeze_beta(beta, 3)
@@ -267,6 +281,8 @@ def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):
     if back is not None:
         o, sT = _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens)
         return o.to(back), sT
+    if _wants_grad(q, k, v, g, beta, initial_state):
+        return _chunk(q, k, v, g, beta, scale, initial_state, CHUNK, l2norm, q.dtype, False, cu_seqlens)
     dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
     if scale is None:
         scale = dk ** -0.5
