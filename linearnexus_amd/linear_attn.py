@@ -324,7 +324,14 @@ def kda_recurrent(q, k, v, g, beta, scale=None, initial_state=None, use_qk_l2nor
 # --------------------------------------------------------------------------------------
 
 def l2norm_rows(x: Tensor) -> Tensor:
-    """``x / (|x|_2 + 1e-6)`` over the last dimension, in x's dtype (gated_deltanet.py:273-275)."""
+    """``x / (|x|_2 + 1e-6)`` over the last dimension, in x's dtype (gated_deltanet.py:273-275; what the DeltaNet
+    block applies to q and k before the op, delta_net.py:566-575).  Differentiable."""
+    if _wants_grad(x):
+        return _L2Norm.apply(x)
+    return _l2norm_rows_fwd(x)
+
+
+def _l2norm_rows_fwd(x: Tensor) -> Tensor:
     x, back = _dense(x)
     y = torch.empty_like(x)
     d = x.shape[-1]
@@ -343,6 +350,18 @@ def _l2norm_rows_bwd(x: Tensor, dy: Tensor) -> Tensor:
     return back(dx)
 
 
+class _L2Norm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return _l2norm_rows_fwd(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        return _l2norm_rows_bwd(x, dy.to(x.dtype))
+
+
 class _ChunkScan(torch.autograd.Function):
     """Pairs lnx_chunk_fwd with lnx_chunk_bwd (the role ``jax.custom_vjp`` plays for a JAX caller)."""
 
@@ -353,8 +372,8 @@ class _ChunkScan(torch.autograd.Function):
         q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
         # the reference's chunk path normalises in the input dtype before anything else
         # (gated_deltanet.py:273-275, kda.py:379-381)
-        qn = l2norm_rows(q_in) if l2norm else q_in
-        kn = l2norm_rows(k_in) if l2norm else k_in
+        qn = _l2norm_rows_fwd(q_in) if l2norm else q_in
+        kn = _l2norm_rows_fwd(k_in) if l2norm else k_in
         v = _as_layout(v, tf)
         beta_f = _as_layout(beta.to(torch.float32), tf)
         g_f = None if g is None else _as_layout(g.to(torch.float32), tf)

@@ -22,6 +22,10 @@ Tensor = torch.Tensor
 
 def _args(q, k, v, a, b, gk, lead_dims):
     dt = _check_inputs(q, k, v)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v, a, b, gk)):
+        # no silent loss of gradients: the rule has a forward (decode / prefill) kernel only
+        raise RuntimeError("the DPLR delta rule has no backward pass here: call it under torch.no_grad() or on "
+                           "detached tensors")
     if q.dim() != lead_dims + 1:
         raise RuntimeError(f"expected {lead_dims + 1}-dimensional q, got {tuple(q.shape)}")
     for name, t in (("a", a), ("b", b), ("gk", gk)):

@@ -108,3 +108,11 @@ def test_errors_and_empty():
     h0 = torch.randn(1, 2, 16, 16, device=DEV)
     o, h = la.dplr_delta_rule_recurrent(e, e, e, e, e, e, initial_state=h0)
     assert o.shape == (1, 2, 0, 16) and torch.equal(h, h0)
+
+
+def test_wanted_gradient_is_refused_loudly():
+    import linearnexus_amd as la
+    t = lambda *s: torch.randn(*s, device="cuda")
+    q = t(1, 2, 8, 64).requires_grad_(True)
+    with pytest.raises(RuntimeError, match="no backward pass"):
+        la.dplr_delta_rule_recurrent(q, t(1, 2, 8, 64), t(1, 2, 8, 64), t(1, 2, 8, 64), t(1, 2, 8, 64), -t(1, 2, 8, 64).abs())

@@ -169,3 +169,7 @@ def test_l2norm_rows_fwd_bwd(rows, d, bf16):
     dx = _l2norm_rows_bwd(x.detach().to(dt), dy.to(dt))
     assert y.shape == (rows, d) and y.dtype == dt
     assert torch.allclose(y.float(), y_ref, atol=tol) and torch.allclose(dx.float(), x.grad, atol=tol * 4)
+    if rows:  # and through autograd on the public op
+        xa = x.detach().to(dt).requires_grad_(True)
+        la.l2norm_rows(xa).backward(dy.to(dt))
+        assert torch.equal(xa.grad, dx)
