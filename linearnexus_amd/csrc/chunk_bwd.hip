@@ -781,13 +781,14 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   static constexpr size_t vec_bytes = sizeof(float) * 2 * 64 * LDF + sizeof(T) * kTile;
   static_assert(GATE != LNX_GATE_VECTOR || vec_bytes <= sizeof(T) * 5 * kTile, "epilogue tiles overlay the loop tiles");
   // tiles: Tm^T, dW/dD slab, dB slab, K/V slab, and the W/U slab (vector gate) or all K slabs but the last kept
-  // for the epilogue (other gates)
-  static constexpr int ntile = (GATE == LNX_GATE_VECTOR) ? 5 : 4 + (DK / 64 - 1);
+  // for the epilogue (other gates; 4-byte inputs with dk <= 128 read K again instead, so that two workgroups fit a CU)
+  static constexpr bool KEEP_K = GATE != LNX_GATE_VECTOR && (sizeof(T) == 2 || DK > 128);
+  static constexpr int ntile = (GATE == LNX_GATE_VECTOR) ? 5 : KEEP_K ? 4 + (DK / 64 - 1) : 4;
   static constexpr size_t bytes = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || DK > 128 ? 2 : 3) : 1)) void bwd_wy2_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || DK > 128 ? 2 : 3) : (GATE == LNX_GATE_VECTOR || DK > 128 ? 1 : 2))) void bwd_wy2_kernel(BwdParams p) {
   typedef Wy2Cfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
@@ -819,7 +820,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   const int wi = wave >> 1, wj = wave & 1;
   // V slabs first, K slabs last: without a per-channel gate the K slabs then stay in LDS for the epilogue
   const int nvs = p.dv / 64, nslab = NKS + nvs;
-  constexpr bool KEEP_K = GATE != LNX_GATE_VECTOR;
+  constexpr bool KEEP_K = L::KEEP_K;
+  constexpr bool RESTAGE = GATE != LNX_GATE_VECTOR && !KEEP_K;  // K slabs staged again in the epilogue
 
   // dA needs M = dBw W^T + dBu U^T.  With a per-channel gate W and U are read back from the workspace.  Otherwise
   // W = Tm diag(beta e^G) K and U = Tm diag(beta) V give M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T with
@@ -840,6 +842,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
     }
   };
   floatx16 aBw[NKS][1][1], aM[1][1], aZu[1][1];  // aM doubles as Zw inside the loop
+  floatx16 aX[1][1];                             // X = K K^T: summed in the loop when the K slabs are not kept
+  frag_zero(aX);
 #pragma unroll
   for (int s_ = 0; s_ < NKS; ++s_) frag_zero(aBw[s_]);
   frag_zero(aM);
@@ -883,6 +887,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
     if (LOAD_WU) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sWU + 32 * wj * LDC, LDC, 64, lane);
     else if (is_k) mma_nt<T, 1, 1>(aM, sdBt + 32 * wi * LDC, LDC, sKc + 32 * wj * LDC, LDC, 64, lane);
     else mma_nt<T, 1, 1>(aZu, sdBt + 32 * wi * LDC, LDC, sKc + 32 * wj * LDC, LDC, 64, lane);
+    if (RESTAGE && is_k && !(wi == 0 && wj == 1))
+      mma_nt<T, 1, 1>(aX, sKc + 32 * wi * LDC, LDC, sKc + 32 * wj * LDC, LDC, 64, lane);
     if (GATE != LNX_GATE_VECTOR || !is_k) {  // <dB row, k row> / <dB row, v row>; thread = (row, quarter of the slab)
       const int r = tid >> 2, q0 = (tid & 3) * 16;
       float t = 0.f;
@@ -1021,7 +1027,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   // The K slabs are still in LDS (the last one in the slab tile, the others in tiles of their own); the partial dk of
   // bwd_dqk is fetched one slab at a time.
   TileRegs<T, 64, 64> rdk;
-  auto k_tile = [&](int u) -> const T* { return (u + 1 < NKS) ? sK0 + u * L::kTile : sKs; };
+  auto k_tile = [&](int u) -> const T* { return (KEEP_K && u + 1 < NKS) ? sK0 + u * L::kTile : sKs; };
   lds_barrier();  // loop tiles dead
   {  // M = (Zw diag(beta e^G) + Zu diag(beta)) Tm^T
     floatx16 z[1][1];
@@ -1037,9 +1043,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   }
   T* sYa = sIn;   // beta dA E (strictly lower); its transpose is read through the same tile
   {
-    floatx16 aX[1][1], y[1][1];
-    frag_zero(aX);
-    if (!(wi == 0 && wj == 1)) {
+    floatx16 y[1][1];
+    if (!RESTAGE && !(wi == 0 && wj == 1)) {
 #pragma unroll
       for (int u = 0; u < NKS; ++u) {
         const T* sKT = k_tile(u);
@@ -1066,6 +1071,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   for (int u = 0; u < NKS; ++u) {
     const T* sKT = k_tile(u);
     rdk.load(reinterpret_cast<const T*>(p.dk) + tbase * DK + 64 * u, tsk, len, tid);  // partial dk of bwd_dqk
+    if (RESTAGE) {
+      if (u > 0) lds_barrier();  // the previous slab's K tile has been read
+      stage_tile<T, 64, 64>(sKs, LDC, kg + 64 * u, tsk, len, tid);
+      lds_barrier();
+    }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane);
