@@ -572,6 +572,9 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
     rdSn.load(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
   };
+  // per-channel gate: K, Q rows and the cumulative gate of this half for the epilogue, fetched during the last slab
+  TileRegs<T, 64, (GATE == LNX_GATE_VECTOR ? 64 : 8)> rk, rq;
+  TileRegs<float, 64, (GATE == LNX_GATE_VECTOR ? 64 : 4)> rGe;
   floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
   frag_zero(aP);
   frag_zero(aQ);
@@ -593,6 +596,11 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     rdSn.store(sdSn, LDC, tid);
     lds_barrier();
     if (v0 + SV < p.dv) fetch(v0 + SV);
+    else if (GATE == LNX_GATE_VECTOR) {  // last slab: the epilogue's K, Q and gate tiles instead
+      rk.load(kg, tsk, len, tid);
+      rq.load(qg, tsk, len, tid);
+      rGe.load(wsp<float>(p, p.off.G) + slot * 64 * DK + ch0, DK, 64, tid);
+    }
     mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDS_, LDS_, sD + 32 * wj * LDS_, LDS_, SV, lane);
     mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
     mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
@@ -624,9 +632,6 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     T* sQr = sKr + L::kTile;
     const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK + ch0;
     float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK + ch0;
-    TileRegs<T, 64, 64> rk, rq;
-    rk.load(kg, tsk, len, tid);
-    rq.load(qg, tsk, len, tid);
     // dW half through sOut (fp32) -> global
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -636,10 +641,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     }
     rk.store(sKr, LDC, tid);
     rq.store(sQr, LDC, tid);
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int r = idx >> 4, c = (idx & 15) * 4;
-      store4(sAl + r * LDF + c, load4(Gg + r * DK + c));
-    }
+    rGe.store(sAl, LDF, tid);
     lds_barrier();
     {
       T* dWg = wsp<T>(p, p.off.dW) + slot * 64 * DK + ch0;
@@ -653,7 +655,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-      sOut[r * LDF + c] = aQ[0][0][e] * p.scale * __expf(Gg[r * DK + c]);
+      sOut[r * LDF + c] = aQ[0][0][e] * p.scale * __expf(sAl[r * LDF + c]);
     }
     lds_barrier();
     pair_row<T, 64, false>(sOut, sR, sAl, LDF, sKr, LDC, p.scale, tid);
@@ -670,13 +672,13 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-      sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(Gg[63 * DK + c] - Gg[r * DK + c], 0.f));
+      sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(sAl[63 * LDF + c] - sAl[r * LDF + c], 0.f));
     }
     lds_barrier();
     float dgc = 0.f;
     if (tid < 64) {
       for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDC + tid]);
-      dgc += __expf(Gg[63 * DK + tid]) * sSS[tid];
+      dgc += __expf(sAl[63 * LDF + tid]) * sSS[tid];
       sSS[tid] = dgc;  // chunk-end gate term, added to row 63 below
     }
     lds_barrier();
