@@ -958,9 +958,11 @@ __global__ void copy_state_kernel(const float* src, float* dst, int64_t n) {
 }
 
 // packed batches: slot table [N][2] = (token0, len), then seq_chunk0[nseq + 1], then the sequence
-// indices by decreasing length (ties by index).  One workgroup.
+// indices by decreasing length (ties by index).  One workgroup: the first chunk slot of every sequence by a serial
+// prefix over the (few) sequences, then all threads fill the slots, each finding its sequence by bisection.
 __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* tab) {
-  int32_t* order = tab + 2 * N + nseq + 1;
+  int32_t* chunk0 = tab + 2 * N;
+  int32_t* order = chunk0 + nseq + 1;
   for (int s = threadIdx.x; s < nseq; s += blockDim.x) {
     const int ls = cu[s + 1] - cu[s];
     int rank = 0;
@@ -970,20 +972,32 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* 
     }
     order[rank] = s;
   }
-  if (threadIdx.x != 0) return;
-  int c = 0;
-  for (int s = 0; s < nseq; ++s) {
-    tab[2 * N + s] = c;
-    for (int t = cu[s]; t < cu[s + 1] && c < N; t += LNX_C) {
-      tab[2 * c] = t;
-      tab[2 * c + 1] = min(LNX_C, cu[s + 1] - t);
-      ++c;
+  if (threadIdx.x == 0) {
+    int c = 0;
+    for (int s = 0; s < nseq; ++s) {
+      chunk0[s] = min(c, N);
+      c += (cu[s + 1] - cu[s] + LNX_C - 1) / LNX_C;
     }
+    chunk0[nseq] = min(c, N);
   }
-  tab[2 * N + nseq] = c;
-  for (; c < N; ++c) {
-    tab[2 * c] = 0;
-    tab[2 * c + 1] = 0;
+  __threadfence_block();
+  __syncthreads();  // chunk0 is read back from global memory by the other threads
+  const int total = chunk0[nseq];
+  for (int c = threadIdx.x; c < N; c += blockDim.x) {
+    int t0 = 0, len = 0;
+    if (c < total) {
+      int lo = 0, hi = nseq - 1;  // last sequence whose first slot is <= c (empty sequences share a first slot)
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (chunk0[mid] <= c) lo = mid; else hi = mid - 1;
+      }
+      // skip forward over empty sequences that start at the same slot: the slot belongs to the one with tokens
+      while (lo + 1 < nseq && chunk0[lo + 1] <= c) ++lo;
+      t0 = cu[lo] + (c - chunk0[lo]) * LNX_C;
+      len = min(LNX_C, cu[lo + 1] - t0);
+    }
+    tab[2 * c] = t0;
+    tab[2 * c + 1] = len;
   }
 }
 
