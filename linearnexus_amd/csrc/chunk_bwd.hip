@@ -630,7 +630,6 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     float* sOut = sAl + 64 * LDF;                    // [64][LDF]
     T* sKr = reinterpret_cast<T*>(sOut + 64 * LDF);  // K rows [64][LDC] (this half's channels)
     T* sQr = sKr + L::kTile;
-    const float* Gg = wsp<float>(p, p.off.G) + slot * 64 * DK + ch0;
     float* dGg = wsp<float>(p, p.off.dG) + slot * 64 * DK + ch0;
     // dW half through sOut (fp32) -> global
 #pragma unroll
