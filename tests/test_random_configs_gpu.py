@@ -28,6 +28,20 @@ def _cases():
         T = int(r.integers(1, 330))
         nseq = int(r.integers(1, 5)) if packed else 0
         out.append((i, gate, bf16, B, H, T, dk, dv, nseq, bool(r.integers(2)), bool(r.integers(2))))
+    # a second list (its own generator, so the first keeps its cases): the wide key heads of the reference's presets,
+    # head sizes between the kernels' sizes, either dtype
+    r = np.random.default_rng(2025)
+    for i in range(36, 60):
+        gate = ("none", "scalar", "vector")[i % 3]
+        bf16 = bool(r.integers(2))
+        dk = int(r.choice([256, 256, 96, 200, 16]))
+        dv = int(r.choice([64, 128, 512, 80, 32] if bf16 or dk < 256 else [64, 128, 80]))
+        H = int(r.integers(1, 3))
+        packed = bool(r.integers(3) == 0)
+        B = 1 if packed else int(r.integers(1, 3))
+        T = int(r.integers(1, 200))
+        nseq = int(r.integers(1, 5)) if packed else 0
+        out.append((i, gate, bf16, B, H, T, dk, dv, nseq, bool(r.integers(2)), bool(r.integers(2))))
     return out
 
 
