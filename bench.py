@@ -428,12 +428,47 @@ def bench_decode_graph(torch, steps):
     return res
 
 
+def bench_prefill_long(torch, la, steps):
+    """Forward only (prefill) of single long prompts, Gated DeltaNet bf16: one sequential chain per (head, value slab)
+    against the segments-in-parallel form the ops pick for few long sequences (LNX_PREFILL_SEGMENTS=1 disables it)."""
+    import os
+    res = []
+    for H, T, dk, dv in ((4, 65536, 128, 128), (16, 131072, 128, 128), (4, 32768, 256, 512)):
+        gen = torch.Generator(device="cpu").manual_seed(7)
+        rn = lambda *s_: torch.randn(*s_, generator=gen, dtype=torch.float32)
+        nrm = lambda x: x / (x.norm(dim=-1, keepdim=True) + 1e-6)
+        q, k = nrm(rn(1, H, T, dk)).to("cuda:0").bfloat16(), nrm(rn(1, H, T, dk)).to("cuda:0").bfloat16()
+        v = rn(1, H, T, dv).to("cuda:0").bfloat16()
+        beta = torch.sigmoid(rn(1, H, T)).to("cuda:0")
+        g = (-torch.nn.functional.softplus(rn(1, H, T)) * 0.1).to("cuda:0")
+        ms = {}
+        for name, env in (("one_chain", "1"), ("segmented", None)):
+            if env is None:
+                os.environ.pop("LNX_PREFILL_SEGMENTS", None)
+            else:
+                os.environ["LNX_PREFILL_SEGMENTS"] = env
+            with torch.no_grad():
+                for _ in range(2):
+                    la.gated_delta_rule_chunkwise(q, k, v, g, beta, use_qk_l2norm=False)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    la.gated_delta_rule_chunkwise(q, k, v, g, beta, use_qk_l2norm=False)
+                torch.cuda.synchronize()
+            ms[name] = (time.perf_counter() - t0) / steps * 1e3
+        os.environ.pop("LNX_PREFILL_SEGMENTS", None)
+        res.append({"B": 1, "H": H, "T": T, "dk": dk, "dv": dv, "one_chain_ms": ms["one_chain"],
+                    "segmented_ms": ms["segmented"], "tokens_per_s": T / (ms["segmented"] * 1e-3)})
+        del q, k, v, beta, g
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated", "kda_gate"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated", "kda_gate", "prefill_long"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
@@ -454,6 +489,14 @@ def main():
 
     if args.workload == "kda_gate":
         print(json.dumps(bench_kda_gate(torch, la, _lib, args.steps, args.warmup)))
+        return
+    if args.workload == "prefill_long":
+        res = bench_prefill_long(torch, la, min(args.steps, 10))
+        print(json.dumps({"metric": "single long prompt, forward only: tokens/s", "value": res[0]["tokens_per_s"],
+                          "unit": "tokens/s", "n_gpus": 1, "steps": min(args.steps, 10), "warmup": 2,
+                          "ms_per_step": res[0]["segmented_ms"], "higher_is_better": True, "vs_baseline": None,
+                          "dtype": "bf16", "data": "synthetic", "config": {"workload": "gated_deltanet_prefill_long"},
+                          "cases": res}))
         return
     if args.workload == "rmsnorm_gated":
         print(json.dumps(bench_rmsnorm_gated(torch, la, _lib, args.steps, args.warmup)))
