@@ -77,6 +77,12 @@ typedef struct lnx_scan_args {
 
   void* workspace;
   uint64_t workspace_bytes;
+
+  int32_t value_cols;           /* lnx_chunk_fwd with forward_only (ABI version 4): v holds only the first value_cols
+                                   of the dv value columns (its rows are value_cols long); the others are zero and
+                                   are not read.  0 = all dv.  With forward_only, o may also be NULL: only the final
+                                   states are wanted.  (Transition matrices of sequence segments: value columns
+                                   [v | 0], initial states [0 | I].) */
 } lnx_scan_args;
 
 /* Library identification; also the symbol a loader probes first. */

@@ -36,6 +36,7 @@ class ScanArgs(C.Structure):
         ("d_o", C.c_void_p), ("d_final_state", C.c_void_p), ("d_q", C.c_void_p), ("d_k", C.c_void_p),
         ("d_v", C.c_void_p), ("d_beta", C.c_void_p), ("d_g", C.c_void_p), ("d_initial_state", C.c_void_p),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
+        ("value_cols", C.c_int32),
     ]
 
 

@@ -35,6 +35,7 @@ struct FwdParams {
   int dv, o_dtype;
   int save;  // write the per-chunk tensors the backward pass (or the separate output kernel) reads
   int out_spw;  // chunk_output: value slabs per workgroup
+  int vcols;    // leading value columns present in v (its row length); the rest of the dv columns are zero
   float scale;
   char* ws;
   ChunkWs off;
@@ -102,10 +103,10 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = tok_index(p.geom, row, tok0);
-  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;  // row strides of the token tiles
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.vcols;  // row strides of the token tiles
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
-  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.vcols;
   const int wi = wave >> 1, wj = wave & 1;
 
   TileRegs<T, 64, 64> rK, rQ;
@@ -142,7 +143,8 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   TileRegs<T, 64, 64> rIn;
   auto fetch = [&](int s_) {
     if (s_ < NKS) rIn.load(kg + 64 * s_, tsk, len, tid);
-    else rIn.load(vg + 64 * (s_ - NKS), tsv, len, tid);
+    else if (64 * (s_ - NKS) < p.vcols) rIn.load(vg + 64 * (s_ - NKS), tsv, len, tid);
+    else rIn.zero();  // value columns that v does not hold
   };
   fetch(0);
   lds_barrier();  // slab tiles dead
@@ -244,10 +246,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = tok_index(p.geom, row, tok0);
-  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;  // row strides of the token tiles
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.vcols;  // row strides of the token tiles
   const T* qg = reinterpret_cast<const T*>(p.q) + tbase * DK;
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
-  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
+  const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.vcols;
   float* Gg = ws_ptr<float>(p, p.off.G) + slot * 64 * DK;
   const int l16 = lane & 15, kq = lane >> 4;
 
@@ -425,7 +427,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         for (int j = 0; j < VN / 4; ++j) rGs[it][j] = load4(Gg + r * DK + 64 * s_ + c + 4 * j);
       }
     } else {
-      rIn.load(vg + 64 * (s_ - NH), tsv, len, tid);
+      if (64 * (s_ - NH) < p.vcols) rIn.load(vg + 64 * (s_ - NH), tsv, len, tid);
+      else rIn.zero();  // value columns that v does not hold
     }
   };
   __syncthreads();  // G is read back from the workspace by other threads than wrote it: global memory must be ordered too
@@ -642,7 +645,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         lds_barrier();  // B2'
         if (n + 1 < c1) fetch_q(n + 1);
         lds_barrier();  // B3
-        if (p.o_dtype == LNX_BF16)
+        if (p.o_dtype == LNX_BF16 && p.o)
           unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
                                        (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
         if (n + 1 < c1) commit_main();
@@ -712,7 +715,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       lds_barrier();  // B3
       // the output rows first: the next fetch recycles the registers these stores read, which the compiler
       // protects with a wait for the stores -- the tile commits in between give them time to complete
-      if (FUSE && p.o_dtype == LNX_BF16)
+      if (FUSE && p.o_dtype == LNX_BF16 && p.o)
         unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
                                      (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
       if (STEADY || n + 1 < c1) commit_rest(nxt);
@@ -805,7 +808,7 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
         if (p.o_dtype == LNX_BF16) {
           frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
-        } else {
+        } else if (p.o) {
           const int tok0 = sMeta[0], len = sMeta[1];
           frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + (tok_index(p.geom, row, tok0) + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj,
                                   (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
@@ -1033,7 +1036,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   hipLaunchKernelGGL(k1, dim3((unsigned)slots), dim3(256), b1, st, p);
   lnx_profile_mark("chunk_scan", st);
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(512), b2, st, p);
-  if (!ScanSmem<T, DK>::FUSE_OUT) {  // otherwise the scan has written the outputs
+  if (!ScanSmem<T, DK>::FUSE_OUT && p.o) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
     // value slabs per workgroup: as many as leave about two thousand workgroups (LNX_OUT_SLABS overrides, for tests)
     const int nslab = p.dv / OutSmem<T, DK>::BV;
@@ -1064,8 +1067,10 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   // tensors without elements (no batch rows, or no tokens) may come with null pointers
   const bool tokens = a->B > 0 && a->T > 0;
   if (tokens && (!a->q || !a->k || !a->v || !a->beta)) return lnx_set_error(LNX_ERR_NULL, "q, k, v and beta are required");
-  if (!backward && ((tokens && !a->o) || (a->B > 0 && !a->final_state)))
-    return lnx_set_error(LNX_ERR_NULL, "o and final_state are required");
+  if (!backward && ((tokens && !a->o && !a->forward_only) || (a->B > 0 && !a->final_state)))
+    return lnx_set_error(LNX_ERR_NULL, "o (unless forward_only) and final_state are required");
+  if (a->value_cols != 0 && (backward || !a->forward_only || a->value_cols < 0 || a->value_cols > a->dv || a->value_cols % 64 != 0))
+    return lnx_set_error(LNX_ERR_SHAPE, "value_cols = %d needs forward_only and a multiple of 64 up to dv = %d", a->value_cols, a->dv);
   if (backward && tokens && (!a->d_o || !a->d_q || !a->d_k || !a->d_v || !a->d_beta))
     return lnx_set_error(LNX_ERR_NULL, "d_o, d_q, d_k, d_v and d_beta are required");
   if (tokens && a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
@@ -1128,6 +1133,7 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   // 4-byte inputs form the outputs in a separate kernel that reads the state and D back
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.out_spw = 1;
+  p.vcols = a->value_cols ? a->value_cols : a->dv;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)

@@ -192,6 +192,10 @@ template <typename T, int ROWS, int COLS> struct TileRegs {
       x[it] = __builtin_bit_cast(typename Vec16<T>::V, raw);
     }
   }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) x[it] = vec_zero<T>();
+  }
   __device__ __forceinline__ typename Vec16<T>::V get(int it, int) const { return x[it]; }
   __device__ __forceinline__ void store(T* dst, int ld, int tid) const {
 #pragma unroll

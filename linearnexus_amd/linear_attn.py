@@ -364,41 +364,56 @@ class _L2Norm(torch.autograd.Function):
         return _l2norm_rows_bwd(x, dy.to(x.dtype))
 
 
+def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, forward_only,
+                   dv_total=None, want_o=True):
+    """One lnx_chunk_fwd call.  ``dv_total`` > v's columns: the state has dv_total value columns of which v holds the
+    first ones and the others are zero (``value_cols``); ``want_o=False``: final states only.  Both forward-only."""
+    dt, B, H, T, dk, dv_in, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, None, cu_seqlens)
+    dv = dv_in if dv_total is None else dv_total
+    if initial_state is not None and tuple(initial_state.shape) != (nstate, H, dk, dv):
+        raise RuntimeError(f"initial_state shape {tuple(initial_state.shape)} != {(nstate, H, dk, dv)}")
+    tf = all(_is_token_first(t) for t in (q, k, v))  # [B,T,H,.] memory behind transposed views: used in place
+    q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
+    # the reference's chunk path normalises in the input dtype before anything else
+    # (gated_deltanet.py:273-275, kda.py:379-381)
+    qn = _l2norm_rows_fwd(q_in) if l2norm else q_in
+    kn = _l2norm_rows_fwd(k_in) if l2norm else k_in
+    v = _as_layout(v, tf)
+    beta_f = _as_layout(beta.to(torch.float32), tf)
+    g_f = None if g is None else _as_layout(g.to(torch.float32), tf)
+    s0 = None if initial_state is None else _f32(initial_state)
+    o = _empty_layout(B, H, T, (dv,), o_dtype, q.device, tf) if want_o else None
+    sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
+    a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
+    a.nseq = nseq
+    a.token_first = int(tf)
+    a.forward_only = int(forward_only)
+    a.value_cols = 0 if dv == dv_in else dv_in
+    a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
+    a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
+    lib = _lib.load()
+    nbytes = int(lib.lnx_chunk_workspace_bytes(a))
+    if nbytes == 0 and T > 0 and B > 0:
+        _lib.check(-2, "lnx_chunk_workspace_bytes")
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q.device)
+    a.workspace, a.workspace_bytes = _ptr(ws), nbytes
+    _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
+    saved = (q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
+    meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
+            None if g is None else g.dtype, initial_state is not None, tf)
+    return o, sT, saved, meta
+
+
 class _ChunkScan(torch.autograd.Function):
     """Pairs lnx_chunk_fwd with lnx_chunk_bwd (the role ``jax.custom_vjp`` plays for a JAX caller)."""
 
     @staticmethod
     def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens):
-        dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
-        tf = all(_is_token_first(t) for t in (q, k, v))  # [B,T,H,.] memory behind transposed views: used in place
-        q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
-        # the reference's chunk path normalises in the input dtype before anything else
-        # (gated_deltanet.py:273-275, kda.py:379-381)
-        qn = _l2norm_rows_fwd(q_in) if l2norm else q_in
-        kn = _l2norm_rows_fwd(k_in) if l2norm else k_in
-        v = _as_layout(v, tf)
-        beta_f = _as_layout(beta.to(torch.float32), tf)
-        g_f = None if g is None else _as_layout(g.to(torch.float32), tf)
-        s0 = None if initial_state is None else _f32(initial_state)
-        o = _empty_layout(B, H, T, (dv,), o_dtype, q.device, tf)
-        sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
-        a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
-        a.nseq = nseq
-        a.token_first = int(tf)
         # nothing to differentiate (inference, torch.no_grad()): the kernels skip what only the backward reads
-        a.forward_only = int(not any(ctx.needs_input_grad))
-        a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
-        a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
-        lib = _lib.load()
-        nbytes = int(lib.lnx_chunk_workspace_bytes(a))
-        if nbytes == 0 and T > 0 and B > 0:
-            _lib.check(-2, "lnx_chunk_workspace_bytes")
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q.device)
-        a.workspace, a.workspace_bytes = _ptr(ws), nbytes
-        _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
-        ctx.save_for_backward(q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
-        ctx.meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
-                    None if g is None else g.dtype, initial_state is not None, tf)
+        o, sT, saved, meta = _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens,
+                                            forward_only=not any(ctx.needs_input_grad))
+        ctx.save_for_backward(*saved)
+        ctx.meta = meta
         return o, sT
 
     @staticmethod
@@ -440,9 +455,9 @@ def _prefill_segments(B: int, H: int, T: int, dv: int) -> int:
     """How many segments a forward-only call is cut into (1: not at all).  The sequential kernels have one workgroup
     per (batch, head, 64 value columns); a single long prompt leaves most of the 256 CUs without one.  Segments are run
     as independent sequences -- see _segmented_forward -- for three times the scan work spread over nseg times the
-    workgroups (plus one copy of v next to zero columns), so it pays when at most an eighth of the CUs would be busy
-    and every segment keeps >= 64 chunks: measured 2.11 -> 0.92 ms for one 65536-token prompt with 4 heads of 128,
-    4.66 -> 4.21 ms for 131072 tokens with 16 heads.  LNX_PREFILL_SEGMENTS forces a count (0 or 1: never)."""
+    workgroups, so it pays when at most an eighth of the CUs would be busy and every segment keeps >= 64 chunks:
+    measured 2.11 -> 0.84 ms for one 65536-token prompt with 4 heads of 128, 4.64 -> 3.36 ms for 131072 tokens with
+    16 heads.  LNX_PREFILL_SEGMENTS forces a count (0 or 1: never)."""
     forced = os.environ.get("LNX_PREFILL_SEGMENTS")
     if forced is not None:
         return max(1, min(int(forced), -(-T // CHUNK)))
@@ -469,11 +484,11 @@ def _segmented_forward(q, k, v, g, beta, scale, initial_state, l2norm, o_dtype, 
     cu = torch.tensor(bounds, dtype=torch.int32, device=q.device)
     fold = lambda t: None if t is None else t.reshape(1, rows, *t.shape[2:])   # batch rows become heads of a packed batch
     q1, k1, v1, g1, beta1 = fold(q), fold(k), fold(v), fold(g), fold(_squeeze_beta(beta, 4))
-    v_ext = torch.cat([v1, v1.new_zeros(1, rows, T, dk)], dim=-1)
     s_ext = torch.zeros(nseg, rows, dk, dv + dk, dtype=torch.float32, device=q.device)
     s_ext[..., dv:] = torch.eye(dk, dtype=torch.float32, device=q.device)
-    _, ab = _ChunkScan.apply(q1, k1, v_ext, g1, beta1, s_ext, scale, l2norm, o_dtype, cu)
-    del v_ext, s_ext
+    _, ab, _, _ = _chunk_forward(q1, k1, v1, g1, beta1, s_ext, scale, l2norm, o_dtype, cu, forward_only=True,
+                                 dv_total=dv + dk, want_o=False)  # v's columns followed by dk zero columns
+    del s_ext
     Bs, As = ab[..., :dv], ab[..., dv:]
     s_in = torch.empty(nseg, rows, dk, dv, dtype=torch.float32, device=q.device)
     cur = torch.zeros(rows, dk, dv, dtype=torch.float32, device=q.device) if initial_state is None \

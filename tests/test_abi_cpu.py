@@ -26,13 +26,14 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() == 3
+    assert lib.lnx_abi_version() == 4
 
 
 def test_struct_layout_matches_header():
-    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size
-    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8
+    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size, value_cols (+ tail padding)
+    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8 + 8
     assert _lib.ScanArgs.q.offset == 56
+    assert _lib.ScanArgs.value_cols.offset == 56 + 18 * 8 + 8
 
 
 def test_argument_validation_without_gpu():
@@ -46,6 +47,18 @@ def test_argument_validation_without_gpu():
     a.B = 0  # an empty batch has no elements behind any pointer: accepted, nothing is launched
     for fn in (lib.lnx_decode_step, lib.lnx_recurrent_fwd, lib.lnx_chunk_fwd, lib.lnx_chunk_bwd):
         assert fn(a, None) == 0
+    # value_cols (v holds only the leading value columns) is a forward-only feature, in whole 64-column slabs
+    a.B, a.dv, a.value_cols = 1, 128, 64
+    one = ctypes.c_float(0)
+    p = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    a.q = a.k = a.v = a.beta = a.o = a.final_state = p
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"value_cols" in lib.lnx_last_error()      # forward_only not set
+    a.forward_only, a.value_cols = 1, 32
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"value_cols" in lib.lnx_last_error()      # not a whole slab
+    a.value_cols = 192
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"value_cols" in lib.lnx_last_error()      # more than dv
+    a.value_cols, a.o = 64, None
+    assert lib.lnx_chunk_fwd(a, None) == -4 and b"workspace" in lib.lnx_last_error()       # accepted up to the workspace
     assert lib.lnx_l2norm_fwd(None, None, 4, 8, 0, None) == -1
     d = _lib.DplrArgs()
     assert lib.lnx_dplr_step(d, None) == -2 and lib.lnx_dplr_recurrent_fwd(d, None) == -2
