@@ -462,7 +462,7 @@ def _prefill_segments(B: int, H: int, T: int, dv: int) -> int:
     if forced is not None:
         return max(1, min(int(forced), -(-T // CHUNK)))
     wide = B * H * -(-dv // 64)
-    if wide > 32 or T < 16384:
+    if wide > 32 or T < 16384 * max(1, wide // 16):  # measured: no gain at 32 workgroups x 16384 tokens, loss at 64
         return 1
     return max(1, min(256 // wide, T // 4096))
 

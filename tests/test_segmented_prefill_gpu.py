@@ -23,6 +23,7 @@ def test_segment_count_heuristic(monkeypatch):
     assert _prefill_segments(1, 4, 8192, 128) == 1         # too short to pay for three times the scan work
     assert _prefill_segments(1, 2, 20000, 512) == 4        # every segment keeps at least 64 chunks
     assert _prefill_segments(2, 16, 131072, 128) == 1      # 64 workgroups: three times the scan work would not pay
+    assert _prefill_segments(1, 16, 16384, 128) == 1       # 32 workgroups need 32768 tokens
     monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "5")
     assert _prefill_segments(8, 16, 4096, 128) == 5
     monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "0")
