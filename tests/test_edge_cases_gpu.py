@@ -276,3 +276,30 @@ def test_other_input_dtypes_are_computed_in_float32(kind):
     o3, S3 = la.gated_delta_rule_step(q.detach()[:, :, 0], k.detach()[:, :, 0], v.detach()[:, :, 0], g[:, :, 0], beta[:, :, 0], s0,
                                       use_qk_l2norm=False)
     assert o3.dtype == dts[0] and max_rel(o3.float().cpu().numpy(), o_ref[:, :, 0]) < tol
+
+
+@pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("bf16", [False, True])
+def test_beta_up_to_two_and_extreme_gates(gate, bf16):
+    """allow_neg_eigval doubles beta (gated_deltanet.py:803-805): learning rates in (0, 2), so I - beta k k^T has
+    eigenvalues down to -1.  Together with gates from 0 (no decay) to -30 per token (state wiped), exact zeros in
+    beta and a run of all-zero keys (padding tokens inside a sequence)."""
+    x = make_inputs(73, 1, 2, 200, 128, 128, gate=gate, with_state=True, with_grad=True)
+    r = np.random.default_rng(73)
+    x["beta"] = r.uniform(0.0, 2.0, x["beta"].shape).astype(np.float32)
+    x["beta"][:, :, 50:60] = 0.0
+    x["beta"][:, :, 60:64] = 2.0
+    x["k"][:, :, 100:110] = 0.0
+    if gate != "none":
+        g = x["g"]
+        g[:, :, 20:30] = 0.0
+        g[:, :, 120:124] = -30.0
+    xf, dt = _prep(x, bf16)
+    o_ref, S_ref = oracle_fwd(xf, gate)
+    o, S = gpu_chunk_fwd(xf, gate, dt)
+    tol = 2e-2 if bf16 else 1e-4
+    assert torch.isfinite(o).all() and torch.isfinite(S).all()
+    assert max_rel(o.float().cpu().numpy(), o_ref) < tol and max_rel(S.cpu().numpy(), S_ref) < tol
+    xb, dt = _prep_bwd(x, bf16)
+    ref = delta_rule_adjoint(xb["q"], xb["k"], xb["v"], xb["beta"], xb["dO"], xb.get("g"), xb["dS"], None, xb["S0"], False)
+    check(gpu_grads(xb, gate, dt), ref, tol)
