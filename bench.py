@@ -103,6 +103,7 @@ CHUNK_CONFIGS = {
     # fp32 inputs (the reference's models run fp32 unless told otherwise): configuration 2's shape and the presets'
     "gdn_chunk_fp32": ("gated32", 8, 16, 4096, 128, 0, False, True),
     "gdn_dk256_fp32": ("gated32", 8, 8, 4096, (256, 512), 0, False, True),
+    "kda_chunk_fp32": ("kda32", 4, 16, 8192, 128, 0, True, True),
 }
 
 
@@ -110,7 +111,7 @@ def bench_chunk(args, torch, la, _lib, name):
     variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
     seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
-            "gdn_chunk_fp32": 2, "gdn_dk256_fp32": 6}[name]
+            "gdn_chunk_fp32": 2, "gdn_dk256_fp32": 6, "kda_chunk_fp32": 3}[name]
     fp32 = variant.endswith("32")
     variant = variant[:-2] if fp32 else variant
     d, dv = d if isinstance(d, tuple) else (d, d)
