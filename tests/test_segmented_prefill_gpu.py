@@ -15,21 +15,6 @@ DEV = "cuda"
 GATES = ["none", "scalar", "vector"]
 
 
-def test_segment_count_heuristic(monkeypatch):
-    from linearnexus_amd.linear_attn import _prefill_segments
-    monkeypatch.delenv("LNX_PREFILL_SEGMENTS", raising=False)
-    assert _prefill_segments(1, 16, 131072, 128) == 8      # 32 workgroups of 64 columns -> 8 segments of 256 chunks
-    assert _prefill_segments(8, 16, 4096, 128) == 1        # configuration 2: the chip is full already
-    assert _prefill_segments(1, 4, 8192, 128) == 1         # too short to pay for three times the scan work
-    assert _prefill_segments(1, 2, 20000, 512) == 4        # every segment keeps at least 64 chunks
-    assert _prefill_segments(2, 16, 131072, 128) == 1      # 64 workgroups: three times the scan work would not pay
-    assert _prefill_segments(1, 16, 16384, 128) == 1       # 32 workgroups need 32768 tokens
-    monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "5")
-    assert _prefill_segments(8, 16, 4096, 128) == 5
-    monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "0")
-    assert _prefill_segments(1, 16, 131072, 128) == 1
-
-
 @pytest.mark.parametrize("nseg", ["2", "5"])
 @pytest.mark.parametrize("gate", GATES)
 @pytest.mark.parametrize("bf16", [False, True])

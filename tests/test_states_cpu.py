@@ -1,4 +1,4 @@
-"""The generation caches mirror the reference's dataclasses field for field and argument for argument
+"""Host-side logic that needs no GPU.  The generation caches mirror the reference's dataclasses field for field and argument for argument
 (delta_net.py:81-118, gated_deltanet.py:72-128, kda.py:57-113), so a caller's ``State.zeros(...)`` lines keep working."""
 import dataclasses
 import inspect
@@ -34,3 +34,18 @@ def test_gated_and_kda_states(cls):
     assert tuple(s.conv_state_v.shape) == (2, 3, 2048)
     s = cls.zeros(2, 4, 256, 512, key_dim_total=1024, value_dim=2048, use_conv=False, device="cpu")
     assert s.conv_state_q is None
+
+
+def test_segment_count_heuristic(monkeypatch):
+    from linearnexus_amd.linear_attn import _prefill_segments
+    monkeypatch.delenv("LNX_PREFILL_SEGMENTS", raising=False)
+    assert _prefill_segments(1, 16, 131072, 128) == 8      # 32 workgroups of 64 columns -> 8 segments of 256 chunks
+    assert _prefill_segments(8, 16, 4096, 128) == 1        # configuration 2: the chip is full already
+    assert _prefill_segments(1, 4, 8192, 128) == 1         # too short to pay for three times the scan work
+    assert _prefill_segments(1, 2, 20000, 512) == 4        # every segment keeps at least 64 chunks
+    assert _prefill_segments(2, 16, 131072, 128) == 1      # 64 workgroups: three times the scan work would not pay
+    assert _prefill_segments(1, 16, 16384, 128) == 1       # 32 workgroups need 32768 tokens
+    monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "5")
+    assert _prefill_segments(8, 16, 4096, 128) == 5
+    monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "0")
+    assert _prefill_segments(1, 16, 131072, 128) == 1
