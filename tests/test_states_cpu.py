@@ -49,3 +49,19 @@ def test_segment_count_heuristic(monkeypatch):
     assert _prefill_segments(8, 16, 4096, 128) == 5
     monkeypatch.setenv("LNX_PREFILL_SEGMENTS", "0")
     assert _prefill_segments(1, 16, 131072, 128) == 1
+
+
+def test_dtype_promotion_rules():
+    """One kernel dtype (float32 or bfloat16) passes through; anything else is computed in float32 and cast back to q's
+    dtype, like the reference's up-cast (delta_net.py:170-179, :213)."""
+    from linearnexus_amd.linear_attn import _promote
+    t = lambda dt: torch.zeros(1, 1, 2, 4, dtype=dt)
+    for dt in (torch.float32, torch.bfloat16):
+        q, k, v, back = _promote(t(dt), t(dt), t(dt))
+        assert back is None and q.dtype == dt
+    q, k, v, back = _promote(t(torch.float32), t(torch.float32), t(torch.bfloat16))   # the DeltaNet block's mix
+    assert back == torch.float32 and {q.dtype, k.dtype, v.dtype} == {torch.float32}
+    q, k, v, back = _promote(t(torch.float16), t(torch.float16), t(torch.float16))
+    assert back == torch.float16 and v.dtype == torch.float32
+    q, k, v, back = _promote(t(torch.bfloat16), t(torch.float32), t(torch.float64))
+    assert back == torch.bfloat16 and q.dtype == torch.float32
