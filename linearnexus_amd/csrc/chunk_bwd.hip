@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
 // on request, for dk = 128 with 2-byte inputs when 64-column slabs would leave most CUs idle.
 template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr int PAD = Mma<T>::PAD;
-  static constexpr int BV = (DK >= 128 && sizeof(T) == 4) ? 32 : BVW;
+  static constexpr int BV = (DK > 128 && sizeof(T) == 4) ? 32 : BVW;
   static constexpr int LDK = DK + PAD, LDU = BV + PAD;
   static constexpr int LDC = LNX_C + PAD;
   static constexpr int kRow = 64 * LDK, kSlab = 64 * LDU, kdST = BV * LDK, kdDT = BV * LDC;
@@ -100,8 +100,9 @@ template <typename T, int DK, int BVW = 64> struct BScanCfg {
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
   // 4-byte inputs with dk = 256: K (read for dD), Q and W (read for the dS update) of a chunk take turns in one tile
   static constexpr bool SHARE = sizeof(T) == 4 && DK > 128;
-  // 2-byte inputs with dk = 256 and 64-column slabs: K (read for dD) and Q (read for the dS update) share a tile
-  static constexpr bool SHAREK = sizeof(T) == 2 && DK > 128 && BV == 64;
+  // 64-column slabs of 2-byte inputs with dk = 256 and of 4-byte inputs with dk = 128: K (read for dD) and Q (read
+  // for the dS update) share a tile
+  static constexpr bool SHAREK = BV == 64 && ((sizeof(T) == 2 && DK > 128) || (sizeof(T) == 4 && DK == 128));
   static constexpr int nRow = SHARE ? 1 : SHAREK ? 2 : 3;
   // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
   static constexpr size_t bytes = sizeof(T) * (nRow * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
@@ -234,8 +235,8 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       const int mt = tid - 256;
       typedef TileRegs<T, 64, BV> Slab;
       TileRegs<T, 64, DK> rK, rQ, rW;
-      Slab rdO;
-      TileRegs<T, 64, 64> rP;
+      Slab rdO, rdD;                      // dD: the chunk-local part from bwd_local (not fused only)
+      TileRegs<T, 64, FUSE ? 64 : 8> rP;  // fused only
       float os[Slab::IT], rG = 0.f;
       const int64_t tsk = (int64_t)p.geom.ts * DK;
       auto fetch_main = [&](int n) {
@@ -247,7 +248,8 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         else rK.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, len, mt);
         rW.load(wsp<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
         rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
-        rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+        if (FUSE) rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
+        else rdD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
         if (GATE == LNX_GATE_SCALAR && mt < 64) rG = wsp<float>(p, p.off.G)[slot * 64 + mt];
         if (GATE == LNX_GATE_VECTOR && mt < DK) rG = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
 #pragma unroll
@@ -266,8 +268,12 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       auto commit_main = [&]() {
         rK.store(sK, LDK, mt);
         rW.store(sW, LDK, mt);
-        rP.store(sP, LDC, mt);
-        rdO.store(sdOr, LDU, mt);
+        if (FUSE) {
+          rP.store(sP, LDC, mt);
+          rdO.store(sdOr, LDU, mt);
+        } else {
+          rdD.store(sdDl, LDU, mt);
+        }
 #pragma unroll
         for (int it = 0; it < Slab::IT; ++it) {
           const int idx = mt + 256 * it, r = idx / Slab::VPR, c = (idx - r * Slab::VPR) * Slab::N;
@@ -290,7 +296,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       for (int n = c1 - 1; n >= c0; --n) {
         const int64_t slot = (int64_t)row * N + n;
         if (n - 1 >= c0) fetch_main(n - 1);
-        if (GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
+        if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
         unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
         lds_barrier();  // B2
         rQ.store(sQ, LDK, mt);
@@ -1125,8 +1131,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
 template <typename T, int DK, int GATE>
 int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
-  constexpr bool can_narrow = DK >= 128 && sizeof(T) == 2;
-  constexpr int WIDE = 64, NARROW = can_narrow ? 32 : WIDE;  // 4-byte inputs with dk >= 128 get 32 columns from BScanCfg
+  // 32-column slabs when 64-column ones would leave more than half of the CUs without a workgroup (2-byte inputs with
+  // dk >= 128, 4-byte inputs with dk = 128; 4-byte inputs with dk = 256 always get 32 columns from BScanCfg)
+  constexpr bool can_narrow = (DK >= 128 && sizeof(T) == 2) || (DK == 128 && sizeof(T) == 4);
+  constexpr int WIDE = 64, NARROW = can_narrow ? 32 : WIDE;
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
   auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, NARROW> : bwd_scan_kernel<T, DK, GATE, WIDE>;
   const int bv = narrow ? BScanCfg<T, DK, NARROW>::BV : BScanCfg<T, DK, WIDE>::BV;
