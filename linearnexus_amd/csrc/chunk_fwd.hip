@@ -1019,7 +1019,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   auto k1 = PrepSelect<T, DK, GATE>::kernel();
   // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs); always for 4-byte inputs
   // with dk = 256, whose tiles leave no room in LDS for a wider slab
-  constexpr bool can_narrow = DK >= 128 && sizeof(T) == 2;
+  constexpr bool can_narrow = (DK >= 128 && sizeof(T) == 2) || (DK == 128 && sizeof(T) == 4);
   constexpr int WIDE = (DK > 128 && sizeof(T) == 4) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;
   const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
   auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, NARROW> : chunk_scan_kernel<T, DK, GATE, WIDE>;
