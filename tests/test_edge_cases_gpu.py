@@ -306,3 +306,35 @@ def test_beta_up_to_two_and_extreme_gates(gate, bf16):
     xb, dt = _prep_bwd(x, bf16)
     ref = delta_rule_adjoint(xb["q"], xb["k"], xb["v"], xb["beta"], xb["dO"], xb.get("g"), xb["dS"], None, xb["S0"], False)
     check(gpu_grads(xb, gate, dt), ref, tol)
+
+
+@pytest.mark.parametrize("gate", ["none", "vector"])
+def test_packed_batch_with_hundreds_of_short_sequences(gate):
+    """More sequences than the table builder has threads, most of them a few tokens long, some empty."""
+    H, d = 2, 64
+    r = np.random.default_rng(74)
+    lens = r.integers(0, 6, 300)
+    lens[::37] = r.integers(60, 140, len(lens[::37]))
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T, nseq = int(cu[-1]), len(lens)
+    x = make_inputs(74, 1, H, T, d, d, gate=gate, with_grad=True)
+    x["S0"] = (r.standard_normal((nseq, H, d, d)) * 0.02).astype(np.float32)
+    x["dS"] = (r.standard_normal((nseq, H, d, d)) * 0.1).astype(np.float32)
+    parts, o_ref, S_ref = [], np.zeros((1, H, T, d)), []
+    for s in range(nseq):
+        a, b = cu[s], cu[s + 1]
+        sl = lambda n: x[n][:, :, a:b]
+        y = {"q": sl("q"), "k": sl("k"), "v": sl("v"), "beta": sl("beta"), "S0": x["S0"][s:s + 1]}
+        if gate != "none":
+            y["g"] = sl("g")
+        o_s, S_s = oracle_fwd(y, gate)
+        o_ref[:, :, a:b] = o_s
+        S_ref.append(S_s)
+        parts.append(delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), sl("g") if gate != "none" else None,
+                                        x["dS"][s:s + 1], None, x["S0"][s:s + 1], False))
+    o, S = gpu_chunk_fwd(x, gate, torch.float32, cu=cu)
+    assert max_rel(o.cpu().numpy(), o_ref) < 1e-4 and max_rel(S.cpu().numpy(), np.concatenate(S_ref, 0)) < 1e-4
+    names = ("dq", "dk", "dv", "dbeta") + (("dg",) if gate != "none" else ())
+    ref = {n: np.concatenate([p[n] for p in parts], 2) for n in names}
+    ref["dS0"] = np.concatenate([p["dS0"] for p in parts], 0)
+    check(gpu_grads(x, gate, torch.float32, cu=cu), ref, 1e-4)
