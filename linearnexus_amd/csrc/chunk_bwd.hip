@@ -680,12 +680,15 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
       sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(sAl[63 * LDF + c] - sAl[r * LDF + c], 0.f));
     }
     lds_barrier();
-    float dgc = 0.f;
-    if (tid < 64) {
-      for (int r = 0; r < 64; ++r) dgc += sOut[r * LDF + tid] * to_f32(sKr[r * LDC + tid]);
-      dgc += __expf(sAl[63 * LDF + tid]) * sSS[tid];
-      sSS[tid] = dgc;  // chunk-end gate term, added to row 63 below
+    {  // chunk-end gate term per channel: sum_r out[r][c] k[r][c], sixteen rows per wave (sMisc is zero: unused here)
+      const int c = tid & 63, r0 = 16 * (tid >> 6);
+      float part = 0.f;
+#pragma unroll
+      for (int r = r0; r < r0 + 16; ++r) part += sOut[r * LDF + c] * to_f32(sKr[r * LDC + c]);
+      atomicAdd(&sMisc[c], part);
     }
+    lds_barrier();
+    if (tid < 64) sSS[tid] = sMisc[tid] + __expf(sAl[63 * LDF + tid]) * sSS[tid];  // added to row 63 below
     lds_barrier();
     pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
     lds_barrier();
