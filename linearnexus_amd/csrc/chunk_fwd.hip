@@ -281,18 +281,18 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
     if (h + 1 < NH) fetch_half(h + 1);
     {  // cumulative gate along the tokens, per channel: 16-row segments in parallel, then their offsets
       const int c = tid & 63, seg = tid >> 6;
-      float run = 0.f;
+      float gs[16];  // the segment's sixteen values in registers: all loads in flight together, one write each
 #pragma unroll
-      for (int r = 16 * seg; r < 16 * seg + 16; ++r) {
-        run += sG[r * LDF + c];
-        sG[r * LDF + c] = run;
-      }
+      for (int i = 0; i < 16; ++i) gs[i] = sG[(16 * seg + i) * LDF + c];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) gs[i] += gs[i - 1];
+      float* sSeg = sX;  // segment totals [4][64] (the inverse's scratch is free here)
+      sSeg[seg * 64 + c] = gs[15];
       lds_barrier();
       float off = 0.f;
-      for (int s_ = 0; s_ < seg; ++s_) off += sG[(16 * s_ + 15) * LDF + c];
-      lds_barrier();
+      for (int s_ = 0; s_ < seg; ++s_) off += sSeg[s_ * 64 + c];
 #pragma unroll
-      for (int r = 16 * seg; r < 16 * seg + 16; ++r) sG[r * LDF + c] += off;
+      for (int i = 0; i < 16; ++i) sG[(16 * seg + i) * LDF + c] = gs[i] + off;
     }
     lds_barrier();
     {  // G, K e^{G_last - G}, scale Q e^G of this half -> workspace
