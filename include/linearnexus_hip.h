@@ -5,8 +5,10 @@
  * interface of its own; these entry points are what an XLA-FFI / ctypes binding for
  * its layer ops would bind.  Every function returns 0 on success and a negative
  * lnx_status otherwise; lnx_last_error() gives the thread-local message.  Nothing
- * here allocates or frees device memory, synchronises the device, or keeps mutable
- * global state: the caller owns all buffers (workspace included) and the stream.
+ * here allocates or frees device memory or synchronises the device, and the compute
+ * entry points keep no state between calls: the caller owns all buffers (workspace
+ * included) and the stream.  The one exception is documented where it is declared: the
+ * optional timing of lnx_profile_enable keeps a process-wide list of HIP events.
  *
  * Tensor conventions (the reference's, linearnexus/modules/linear_attn/delta_net.py:126-134):
  *   q, k  [B, H, T, dk]   v, o  [B, H, T, dv]   beta [B, H, T]   state [B, H, dk, dv] fp32
@@ -15,6 +17,10 @@
  * one element type `dtype` (fp32 or bf16); beta, g, states and their gradients are fp32.
  * With cu_seqlens != NULL the batch is packed: B must be 1, sequences are
  * [cu[s], cu[s+1]) along T, states are [nseq, H, dk, dv] and reset at every boundary.
+ * Contract: cu[0] = 0, cu non-decreasing, cu[nseq] = T.  The table is device memory the host
+ * side cannot inspect, so the kernels clamp its entries to [0, T] and read a decreasing pair as
+ * an empty sequence -- a malformed table never causes an access outside the tensors -- but
+ * tokens outside every sequence then keep unspecified outputs and gradients.
  */
 #ifndef LINEARNEXUS_HIP_H
 #define LINEARNEXUS_HIP_H

@@ -83,8 +83,8 @@ struct SeqSpan {
 };
 __device__ __forceinline__ SeqSpan seq_span(const ChunkGeom& g, int seq, int c0) {
   SeqSpan s;
-  s.t0 = g.cu ? g.cu[seq] : 0;
-  s.t1 = g.cu ? g.cu[seq + 1] : g.T;
+  s.t0 = g.cu ? seq_first(g.cu, seq, g.T) : 0;
+  s.t1 = g.cu ? seq_end(g.cu, seq, g.T) : g.T;
   s.c0 = c0;
   return s;
 }
@@ -114,29 +114,34 @@ inline int lnx_chunk_slots(const lnx_scan_args* a) {
   return a->cu_seqlens ? a->T / LNX_C + a->nseq : (a->T + LNX_C - 1) / LNX_C;
 }
 
+// With forward_only the tensors only the backward pass reads (Tm^T, X, D, the entering states for 2-byte inputs,
+// whose outputs leave the scan kernel itself) and the backward pass's own scratch are not reserved.
 inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   ChunkWs w;
   const uint64_t es = (a->dtype == LNX_BF16) ? 2 : 4;
   const uint64_t rows = a->cu_seqlens ? (uint64_t)a->H : (uint64_t)a->B * a->H;
   const uint64_t N = (uint64_t)lnx_chunk_slots(a);
   const uint64_t slots = rows * N, dk = a->dk, dv = a->dv, C = LNX_C;
+  const bool vec = a->gate == LNX_GATE_VECTOR;
+  const bool bwd = !a->forward_only;                      // a backward pass will follow
+  const bool saved = bwd || a->dtype != LNX_BF16;         // the forward pass writes its per-chunk tensors
   uint64_t off = 0;
   auto take = [&](uint64_t bytes) { uint64_t o = off; off = lnx_align256(off + bytes); return o; };
   w.tab = take(a->cu_seqlens ? (2 * N + 2 * (uint64_t)a->nseq + 1) * 4 : 0);
-  w.G = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
+  w.G = take(vec ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
-  w.X = take(a->gate == LNX_GATE_VECTOR ? slots * C * C * es : 0);
+  w.X = take(vec && saved ? slots * C * C * es : 0);
   w.W = take(slots * C * dk * es);
   w.U = take(slots * C * dv * es);
-  w.Kr = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * es : 0);
-  w.Qg = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * es : 0);
-  w.TmT = take(slots * C * C * es);
-  w.D = take(slots * C * dv * es);
-  w.SnT = take(slots * dv * dk * es);
-  w.dD = take(slots * C * dv * es);
-  w.dSn = take(slots * dk * dv * es);
-  w.dW = take(slots * C * dk * es);
-  w.dG = take(a->gate == LNX_GATE_VECTOR ? slots * C * dk * 4 : slots * C * 4);
+  w.Kr = take(vec ? slots * C * dk * es : 0);
+  w.Qg = take(vec ? slots * C * dk * es : 0);
+  w.TmT = take(saved ? slots * C * C * es : 0);
+  w.D = take(saved ? slots * C * dv * es : 0);
+  w.SnT = take(saved ? slots * dv * dk * es : 0);
+  w.dD = take(bwd ? slots * C * dv * es : 0);
+  w.dSn = take(bwd ? slots * dk * dv * es : 0);
+  w.dW = take(bwd ? slots * C * dk * es : 0);
+  w.dG = take(bwd ? (vec ? slots * C * dk * 4 : slots * C * 4) : 0);
   w.total = off;
   return w;
 }
@@ -154,8 +159,6 @@ inline bool lnx_narrow_slabs(int64_t wide_workgroups) {
 // Shared argument validation of the chunk entry points; returns LNX_OK or an error status.
 int lnx_chunk_check(const lnx_scan_args* a, bool backward);
 
-// Builds the packed-batch chunk table (no-op for dense batches).
-void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st);
 
 // ---------------------------------------------------------------------------------------
 // Vector-gate (KDA) helpers.  The per-channel decays E_ij[c] = exp(G_i[c] - G_j[c]) (i >= j, G the

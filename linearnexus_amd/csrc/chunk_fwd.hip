@@ -963,14 +963,17 @@ __global__ void copy_state_kernel(const float* src, float* dst, int64_t n) {
 // packed batches: slot table [N][2] = (token0, len), then seq_chunk0[nseq + 1], then the sequence
 // indices by decreasing length (ties by index).  One workgroup: the first chunk slot of every sequence by a serial
 // prefix over the (few) sequences, then all threads fill the slots, each finding its sequence by bisection.
-__global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* tab) {
+__global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int T, int32_t* tab) {
   int32_t* chunk0 = tab + 2 * N;
   int32_t* order = chunk0 + nseq + 1;
+  // a malformed table (entries outside [0, T] or decreasing) must not send any kernel outside the tensors
+  auto first = [&](int s) { return seq_first(cu, s, T); };
+  auto length = [&](int s) { return seq_end(cu, s, T) - seq_first(cu, s, T); };
   for (int s = threadIdx.x; s < nseq; s += blockDim.x) {
-    const int ls = cu[s + 1] - cu[s];
+    const int ls = length(s);
     int rank = 0;
     for (int u = 0; u < nseq; ++u) {
-      const int lu = cu[u + 1] - cu[u];
+      const int lu = length(u);
       rank += (lu > ls) || (lu == ls && u < s);
     }
     order[rank] = s;
@@ -979,7 +982,7 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* 
     int c = 0;
     for (int s = 0; s < nseq; ++s) {
       chunk0[s] = min(c, N);
-      c += (cu[s + 1] - cu[s] + LNX_C - 1) / LNX_C;
+      c += (length(s) + LNX_C - 1) / LNX_C;
     }
     chunk0[nseq] = min(c, N);
   }
@@ -996,8 +999,8 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int32_t* 
       }
       // skip forward over empty sequences that start at the same slot: the slot belongs to the one with tokens
       while (lo + 1 < nseq && chunk0[lo + 1] <= c) ++lo;
-      t0 = cu[lo] + (c - chunk0[lo]) * LNX_C;
-      len = min(LNX_C, cu[lo + 1] - t0);
+      t0 = first(lo) + (c - chunk0[lo]) * LNX_C;
+      len = max(0, min(LNX_C, seq_end(cu, lo, T) - t0));
     }
     tab[2 * c] = t0;
     tab[2 * c + 1] = len;
@@ -1090,24 +1093,10 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   return LNX_OK;
 }
 
-void lnx_chunk_build_table(const lnx_scan_args* a, const ChunkWs& w, hipStream_t st) {
-  if (!a->cu_seqlens) return;
-  hipLaunchKernelGGL(build_table_kernel, dim3(1), dim3(256), 0, st, a->cu_seqlens, a->nseq, lnx_chunk_slots(a),
-                     reinterpret_cast<int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab));
-}
+namespace {
 
-extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
-  // only the geometry matters here; tensor pointers may still be unset
-  if (!a || a->H <= 0 || a->T < 0 || a->B < 0 || (a->dk != 64 && a->dk != 128 && a->dk != 256) || a->dv <= 0 || a->dv % 64 != 0 ||
-      (a->cu_seqlens && a->nseq <= 0))
-    return 0;
-  return lnx_chunk_ws_layout(a).total;
-}
-
-extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
-  int rc = lnx_chunk_check(a, false);
-  if (rc != LNX_OK) return rc;
-  hipStream_t st = (hipStream_t)stream;
+// The forward pass on a caller-chosen workspace (a->workspace is not looked at).
+int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_bytes, hipStream_t st) {
   const bool packed = a->cu_seqlens != nullptr;
   const int nstate = packed ? a->nseq : a->B;
   if (nstate == 0) return LNX_OK;
@@ -1118,23 +1107,27 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
     return LNX_OK;
   }
   const ChunkWs w = lnx_chunk_ws_layout(a);
-  if (!a->workspace || a->workspace_bytes < w.total)
+  if (!workspace || workspace_bytes < w.total)
     return lnx_set_error(LNX_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)w.total,
-                         (unsigned long long)a->workspace_bytes);
-  lnx_chunk_build_table(a, w, st);
+                         (unsigned long long)workspace_bytes);
+  char* ws = reinterpret_cast<char*>(workspace);
+  if (packed)
+    hipLaunchKernelGGL(build_table_kernel, dim3(1), dim3(256), 0, st, a->cu_seqlens, a->nseq, lnx_chunk_slots(a), a->T,
+                       reinterpret_cast<int32_t*>(ws + w.tab));
   FwdParams p;
   p.geom.H = a->H; p.geom.T = a->T; p.geom.N = lnx_chunk_slots(a); p.geom.nseq = a->nseq;
   p.geom.ts = a->token_first ? a->H : 1;
   p.geom.rows = packed ? a->H : a->B * a->H;
   p.geom.cu = a->cu_seqlens;
-  p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
+  p.geom.tab = packed ? reinterpret_cast<const int32_t*>(ws + w.tab) : nullptr;
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.g = a->g; p.s0 = a->initial_state;
   p.sT_out = a->final_state; p.o = a->o; p.dv = a->dv; p.o_dtype = a->o_dtype; p.scale = a->scale;
   // 4-byte inputs form the outputs in a separate kernel that reads the state and D back
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.out_spw = 1;
   p.vcols = a->value_cols ? a->value_cols : a->dv;
-  p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
+  p.ws = ws; p.off = w;
+  int rc;
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
          : (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
@@ -1147,4 +1140,20 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk forward launch: %s", hipGetErrorString(e));
   return LNX_OK;
+}
+
+}  // namespace
+
+extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
+  // only the geometry matters here; tensor pointers may still be unset
+  if (!a || a->H <= 0 || a->T < 0 || a->B < 0 || (a->dk != 64 && a->dk != 128 && a->dk != 256) || a->dv <= 0 || a->dv % 64 != 0 ||
+      (a->cu_seqlens && a->nseq <= 0))
+    return 0;
+  return lnx_chunk_ws_layout(a).total;
+}
+
+extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
+  int rc = lnx_chunk_check(a, false);
+  if (rc != LNX_OK) return rc;
+  return chunk_fwd_on(a, a->workspace, a->workspace_bytes, (hipStream_t)stream);
 }

@@ -46,6 +46,12 @@ __device__ __forceinline__ void store4(bf16_t* p, floatx4 x) {
   *reinterpret_cast<bf16x4*>(p) = t;
 }
 
+// Token range [seq_first, seq_end) of packed sequence s, read defensively: cu_seqlens lives in device memory where the
+// host cannot check it, so entries are clamped to [0, T] and an end before its start reads as an empty sequence.  A
+// well-formed table (cu[0] = 0, non-decreasing, cu[nseq] = T) is unchanged by this.
+__device__ __forceinline__ int seq_first(const int32_t* cu, int s, int T) { return min(max(cu[s], 0), T); }
+__device__ __forceinline__ int seq_end(const int32_t* cu, int s, int T) { return max(min(max(cu[s + 1], 0), T), seq_first(cu, s, T)); }
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits until every global
 // load and store of the wave has completed, which puts the full memory latency of a register
 // prefetch (and of streamed-out results) on the critical path of each loop iteration.  Use this

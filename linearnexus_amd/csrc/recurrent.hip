@@ -158,8 +158,8 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(TokenParams p) {
   int t0 = 0, t1 = p.T;
   int64_t bh = sh;  // row of the [B*H, T, .] token tensors
   if (p.cu_seqlens) {
-    t0 = p.cu_seqlens[sb];
-    t1 = p.cu_seqlens[sb + 1];
+    t0 = seq_first(p.cu_seqlens, sb, p.T);
+    t1 = seq_end(p.cu_seqlens, sb, p.T);
     bh = h;
   }
   const int col0 = blockIdx.y * 32 + (lane & 7) * 4;

@@ -270,12 +270,31 @@ def _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens):
     if cu_seqlens is not None:
         if B != 1:
             raise RuntimeError("cu_seqlens needs a packed batch with B == 1")
-        cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()
+        cu_seqlens = _check_cu_seqlens(cu_seqlens, T).to(device=q.device, dtype=torch.int32).contiguous()
         nseq = cu_seqlens.numel() - 1
     nstate = nseq if nseq else B
     if initial_state is not None and tuple(initial_state.shape) != (nstate, H, dk, dv):
         raise RuntimeError(f"initial_state shape {tuple(initial_state.shape)} != {(nstate, H, dk, dv)}")
     return dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu_seqlens
+
+
+def _check_cu_seqlens(cu, T: int) -> Tensor:
+    """``cu_seqlens`` as an integer tensor.  A table that lives on the host (list, numpy array, CPU tensor) is
+    validated here: one-dimensional, at least two entries, ``cu[0] == 0``, non-decreasing, ``cu[-1] == T`` -- every
+    token belongs to exactly one sequence; anything else raises ``ValueError``.  A table that is already on the GPU is
+    not read back (that would synchronise the stream): the kernels clamp its entries to ``[0, T]`` and treat a
+    decreasing pair as an empty sequence, so a malformed table cannot send them outside the tensors, but tokens it
+    does not cover then keep unspecified outputs and gradients."""
+    if not isinstance(cu, torch.Tensor):
+        cu = torch.as_tensor(cu)
+    if cu.is_floating_point() or cu.dim() != 1 or cu.numel() < 2:
+        raise ValueError(f"cu_seqlens must be a 1-D integer table with at least two entries, got shape {tuple(cu.shape)} {cu.dtype}")
+    if not cu.is_cuda:
+        c = cu.to(torch.int64)
+        if int(c[0]) != 0 or int(c[-1]) != T or bool((c[1:] < c[:-1]).any()):
+            raise ValueError(f"cu_seqlens must start at 0, never decrease and end at T = {T}; got {c.tolist()[:8]}"
+                             f"{' ...' if c.numel() > 8 else ''} (last {int(c[-1])})")
+    return cu
 
 
 def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):

@@ -114,3 +114,20 @@ def test_chunk_size_error_type():
 
 def test_backend_seam():
     assert la.select_kernel_backend("pallas") is la.KernelBackend.HIP
+
+
+def test_malformed_cu_seqlens_is_refused_on_the_host():
+    """A sequence table held on the host is checked before anything reaches the GPU: it must start at 0, never
+    decrease and end at T (every kernel indexes the token tensors with it)."""
+    import numpy as np
+    import torch
+    from linearnexus_amd.linear_attn import _check_cu_seqlens
+
+    assert _check_cu_seqlens([0, 3, 3, 10], 10).tolist() == [0, 3, 3, 10]
+    assert _check_cu_seqlens(np.array([0, 10], np.int32), 10).tolist() == [0, 10]
+    for bad in ([1, 5, 10], [0, 6, 5, 10], [0, 5, 11], [0, 5, 9], [-1, 10], [0], [[0, 10]], [0.0, 10.0]):
+        with pytest.raises(ValueError):
+            _check_cu_seqlens(bad, 10)
+    with pytest.raises(ValueError):
+        _check_cu_seqlens(torch.tensor([0, 4, 2, 10]), 10)
+
