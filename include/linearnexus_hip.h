@@ -7,7 +7,8 @@
  * lnx_status otherwise; lnx_last_error() gives the thread-local message.  Nothing
  * here allocates or frees device memory or synchronises the device, and the compute
  * entry points keep no state between calls: the caller owns all buffers (workspace
- * included) and the stream.  The one exception is documented where it is declared: the
+ * included) and the stream.  The two exceptions are documented where they are declared:
+ * lnx_chunk_fwd_static works on a scratch array the library holds per GPU, and the
  * optional timing of lnx_profile_enable keeps a process-wide list of HIP events.
  *
  * Tensor conventions (the reference's, linearnexus/modules/linear_attn/delta_net.py:126-134):
@@ -121,6 +122,19 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);
+
+/*
+ * lnx_chunk_fwd for callers that cannot allocate device memory or bring a workspace (code under HIP graph
+ * capture, tight serving loops): same arguments and results as lnx_chunk_fwd with forward_only = 1 (required),
+ * but a->workspace / a->workspace_bytes are ignored and the per-chunk tensors go to a scratch array of
+ * LNX_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process ends.  Shapes whose
+ * lnx_chunk_workspace_bytes exceeds that size are refused with LNX_ERR_WORKSPACE.  It calls no hipMalloc / hipFree
+ * or other allocating routine.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race and must be serialised by the caller.  No counterpart in the reference, whose
+ * JAX ops leave allocation to XLA.
+ */
+#define LNX_STATIC_SCRATCH_BYTES (64u << 20)
+int lnx_chunk_fwd_static(const lnx_scan_args* a, void* hip_stream);
 
 /*
  * Chunked backward: gradients of <o, dO> + <final_state, d_final_state>.  The reference

@@ -11,11 +11,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liblinearnexus_hip.so")
 
 LNX_F32, LNX_BF16 = 0, 1
+STATIC_SCRATCH_BYTES = 64 << 20  # LNX_STATIC_SCRATCH_BYTES
 GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
-    "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
+    "lnx_chunk_workspace_bytes", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
     "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
     "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
     "lnx_profile_enable", "lnx_profile_read",
@@ -67,7 +68,7 @@ def load() -> C.CDLL:
     lib = C.CDLL(LIB_PATH)
     lib.lnx_abi_version.restype = C.c_int
     lib.lnx_last_error.restype = C.c_char_p
-    for name in ("lnx_decode_step", "lnx_recurrent_fwd", "lnx_chunk_fwd", "lnx_chunk_bwd"):
+    for name in ("lnx_decode_step", "lnx_recurrent_fwd", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd"):
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(ScanArgs), C.c_void_p]

@@ -16,6 +16,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "chunk_common.h"
@@ -1142,6 +1143,32 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
   return LNX_OK;
 }
 
+// Library-owned scratch of lnx_chunk_fwd_static: one copy per GPU, at its own address on each, alive until the
+// process ends.  The name below is a host-side handle only; device code gets the address looked up per device.
+static __device__ __align__(256) unsigned char scratch[LNX_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Address of `scratch` on the current device (looked up once per device, with that device current).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return lnx_set_error(LNX_ERR_DEVICE, "hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return lnx_set_error(LNX_ERR_DEVICE, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return LNX_OK;
+}
+
 }  // namespace
 
 extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
@@ -1156,4 +1183,18 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   int rc = lnx_chunk_check(a, false);
   if (rc != LNX_OK) return rc;
   return chunk_fwd_on(a, a->workspace, a->workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int lnx_chunk_fwd_static(const lnx_scan_args* a, void* stream) {
+  int rc = lnx_chunk_check(a, false);
+  if (rc != LNX_OK) return rc;
+  if (!a->forward_only)
+    return lnx_set_error(LNX_ERR_WORKSPACE, "lnx_chunk_fwd_static needs forward_only: the library's scratch does not outlive the call");
+  const uint64_t need = (a->T == 0 || a->B == 0) ? 0 : lnx_chunk_ws_layout(a).total;
+  if (need > (uint64_t)LNX_STATIC_SCRATCH_BYTES)
+    return lnx_set_error(LNX_ERR_WORKSPACE, "lnx_chunk_fwd_static: this shape needs %llu bytes of scratch, the library holds %llu",
+                         (unsigned long long)need, (unsigned long long)LNX_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if ((rc = static_scratch(&ws)) != LNX_OK) return rc;
+  return chunk_fwd_on(a, ws, LNX_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
 }

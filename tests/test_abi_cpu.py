@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() == 4
+    assert lib.lnx_abi_version() == 5
 
 
 def test_struct_layout_matches_header():
@@ -131,3 +131,17 @@ def test_malformed_cu_seqlens_is_refused_on_the_host():
     with pytest.raises(ValueError):
         _check_cu_seqlens(torch.tensor([0, 4, 2, 10]), 10)
 
+
+def test_static_scratch_entry_point_refuses_without_gpu():
+    """lnx_chunk_fwd_static checks the shape against the library's scratch size before it touches the GPU."""
+    lib = _lib.load()
+    one = ctypes.c_float(0)
+    p = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    a = _lib.ScanArgs()
+    a.B, a.H, a.T, a.dk, a.dv, a.chunk = 8, 16, 4096, 128, 128, 64
+    a.dtype = a.o_dtype = _lib.LNX_BF16
+    a.q = a.k = a.v = a.beta = a.o = a.final_state = p
+    assert lib.lnx_chunk_fwd_static(a, None) == -4 and b"forward_only" in lib.lnx_last_error()
+    a.forward_only = 1
+    assert int(lib.lnx_chunk_workspace_bytes(a)) > _lib.STATIC_SCRATCH_BYTES
+    assert lib.lnx_chunk_fwd_static(a, None) == -4 and b"scratch" in lib.lnx_last_error()
