@@ -30,23 +30,52 @@ PEAK_BF16 = 2500.0  # TFLOP/s, dense bf16 MFMA, MI355X
 PEAK_HBM = 8000.0   # GB/s
 PEAK_FP32_MFMA = 157.3  # TFLOP/s
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured for that (workload, kernel).
-TRAFFIC = {
-    ("gdn_chunk", "chunk_prepare"): 892791394, ("gdn_chunk", "chunk_scan"): 1151619330,
-    ("gdn_chunk", "bwd_scan"): 1019418003, ("gdn_chunk", "bwd_dqk"): 1617145429,
-    ("gdn_chunk", "bwd_wy"): 1084088355, ("decode", "decode_step"): 1083426478,
-    ("gdn_dk256", "chunk_prepare"): 1144179908, ("gdn_dk256", "chunk_scan"): 2350101812,
-    ("gdn_dk256", "bwd_scan"): 2082675160, ("gdn_dk256", "bwd_dqk"): 3686681985, ("gdn_dk256", "bwd_wy"): 1381163915,
-    ("kda_chunk", "chunk_prepare"): 2082771134, ("kda_chunk", "chunk_scan"): 1287886410,
-    ("kda_chunk", "bwd_scan"): 1019391118, ("kda_chunk", "bwd_dqk"): 2732077910, ("kda_chunk", "bwd_wy"): 2664907117,
-}
+def sources_sha256(files):
+    """Hash of the named kernel sources, so that counter figures are only quoted for the code they were taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted(files):
+        h.update(f.encode())
+        with open(os.path.join(ROOT, "linearnexus_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
 
 
-def chunk_flops(dk, dv):
-    """Algorithmic dense-product FLOPs per (batch, head, chunk), split by kernel.  The forward
-    terms add up to F_chunk = 2C^2(3dk+2dv) + 6C*dk*dv and the backward terms to 2*F_chunk."""
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in
+    profiles/traffic.json, and where the figure comes from; (None, reason) when the kernel sources have changed
+    since those runs."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as fh:
+            rec = json.load(fh)
+    except (OSError, ValueError):
+        return None, "profiles/traffic.json missing"
+    reason = "not measured"
+    for entry in rec.get("measurements", []):
+        if kernel in entry.get("workloads", {}).get(workload, {}):
+            try:
+                same = entry.get("sources_sha256") == sources_sha256(entry.get("sources", []))
+            except OSError:
+                same = False
+            if same:
+                return entry["workloads"][workload][kernel], f"profiles/traffic.json, commit {entry.get('commit')}"
+            reason = f"profiles/traffic.json entry of commit {entry.get('commit')} predates the current kernel sources"
+    return None, reason
+
+
+def chunk_flops(dk, dv, direct=False):
+    """Dense-product FLOPs per (batch, head, chunk) that each kernel performs.  In the WY split the forward
+    terms add up to F_chunk = 2C^2(3dk+2dv) + 6C*dk*dv and the backward terms to 2*F_chunk; `direct` is the split of
+    the kernels for 2-byte inputs with dk <= 128 and no per-channel gate."""
     cc, cd = 2 * C * C, 2 * C * dk * dv
+    if direct:
+        return {
+            "chunk_prepare": 2 * cc * dk,                     # K K^T, Q K^T
+            "chunk_scan": 3 * cd + 2 * cc * dv,               # K S, Q S, Tm R, Pm D, K^T D
+            "bwd_scan": 3 * cd + 2 * cc * dv,                 # K dS, Pm^T dO, Tm^T dD, Q^T dO, K^T dY
+            "bwd_chunk": 3 * cd + 2 * cc * dv + 4 * cc * dk,  # dO S^T, dR S^T, D dS^T, dO D^T, dR D^T, dPe K, dXa K, dPe^T Q, dXe^T K
+        }
     return {
         "chunk_prepare": cc * (3 * dk + dv),          # K K^T, Q K^T, Tm(beta K), Tm(beta V)
         "chunk_scan": 2 * cd,                         # W S, K^T D
@@ -56,6 +85,19 @@ def chunk_flops(dk, dv):
         "bwd_dqk": cc * dv + 3 * cd + 2 * cc * dk,    # dO D^T, dO S^T, dD S^T, D dS^T, dPe K, dPe^T Q
         "bwd_wy": cc * (4 * dk + 2 * dv),             # Tm^T dW, Tm^T dD, dBw W^T + dBu U^T, K K^T, Y K
     }
+
+
+def make_cu_seqlens(seed, nseq, total, lo, hi, max_tries=1000):
+    """cu_seqlens of `nseq` sequence lengths uniform in [lo, hi] that sum to `total` (configuration 5)."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    for _ in range(max_tries):
+        lens = rng.integers(lo, hi + 1, size=nseq).astype(np.int64)
+        lens = np.floor(lens * (total / lens.sum())).astype(np.int64)
+        lens[-1] += total - lens.sum()
+        if lens.min() >= lo and lens.max() <= hi:
+            return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    raise RuntimeError("could not draw sequence lengths in range")
 
 
 def make_gdn_inputs(torch, B, H, T, d, seed, device, dv=None):
@@ -125,7 +167,6 @@ def bench_chunk(args, torch, la, _lib, name):
     cu = None
     nstate = B
     if nseq:
-        from oracle.inputs import make_cu_seqlens
         cu_np = make_cu_seqlens(seed, nseq, T, 1024, 8192)
         cu = torch.from_numpy(cu_np).to(dev)
         nstate = nseq
@@ -181,16 +222,17 @@ def bench_chunk(args, torch, la, _lib, name):
         nchunks = H * int(sum(-(-int(l) // C) for l in (cu_np[1:] - cu_np[:-1])))
     else:
         nchunks = B * H * (-(-T // C))
-    fl = chunk_flops(d, dv)
     avg = {n: sum(v_) / len(v_) for n, v_ in per_kernel.items()}
-    if "chunk_output" not in avg:  # 2-byte inputs: the scan kernel also forms the outputs
+    fl = chunk_flops(d, dv, direct="bwd_chunk" in avg)
+    if "chunk_output" not in avg and "chunk_output" in fl:  # 2-byte inputs: the scan kernel also forms the outputs
         fl["chunk_scan"] += fl.pop("chunk_output")
-    if "bwd_local" not in avg:     # ... and the backward scan the chunk-local part of dD
+    if "bwd_local" not in avg and "bwd_local" in fl:     # ... and the backward scan the chunk-local part of dD
         fl["bwd_scan"] += fl.pop("bwd_local")
     dom = max(avg, key=avg.get)
     achieved = fl[dom] * nchunks / (avg[dom] * 1e-3) / 1e12
     peak = PEAK_FP32_MFMA if fp32 else PEAK_BF16
     total_fl = (3 if backward else 1) * (2 * C * C * (3 * d + 2 * dv) + 6 * C * d * dv) * nchunks
+    tr, tr_src = measured_traffic(name, dom)
     out = {
         "metric": "delta-rule chunk fwd+bwd tokens/s, % MFMA peak; decode-step HBM GB/s",
         "value": B * T / dtm, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -204,9 +246,8 @@ def bench_chunk(args, torch, la, _lib, name):
         "kernel_ms": {n: round(t, 4) for n, t in avg.items()},
         "forward_only_ms": round(fwd_only_ms, 4),
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                     "frac": achieved / peak, "traffic": TRAFFIC.get((name, dom))},
+                     "frac": achieved / peak, "traffic": tr, "traffic_source": tr_src},
     }
-    tr = TRAFFIC.get((name, dom))
     if tr:  # the same kernel against the HBM roof, from its measured traffic
         out["roofline_hbm_measured"] = {"kernel": dom, "achieved": tr / (avg[dom] * 1e-3) / 1e9, "peak": PEAK_HBM,
                                         "unit": "GB/s", "frac": tr / (avg[dom] * 1e-3) / 1e9 / PEAK_HBM}
@@ -246,12 +287,13 @@ def bench_decode(args, torch, la, _lib, steps=None):
     _lib.profile_enable(False)
     nbytes = 2 * S.numel() * 4 + 4 * B * H * d * 2 + 2 * B * H * 4
     kms = sum(kern) / len(kern)
+    tr, tr_src = measured_traffic("decode", "decode_step")
     return {
         "workload": "gated_deltanet_decode_step", "B": B, "H": H, "dk": d, "dv": d, "steps": steps,
         "ms_per_step": dt * 1e3, "tokens_per_s": B / dt, "bytes_per_step": nbytes,
         "roofline": {"bound": "hbm", "kernel": "decode_step", "achieved": nbytes / (kms * 1e-3) / 1e9, "peak": PEAK_HBM,
                      "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / PEAK_HBM,
-                     "traffic": TRAFFIC.get(("decode", "decode_step"))},
+                     "traffic": tr, "traffic_source": tr_src},
     }
 
 

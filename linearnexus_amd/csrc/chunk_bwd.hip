@@ -1210,6 +1210,21 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.dq = a->d_q; p.dk = a->d_k; p.dv_out = a->d_v; p.dbeta = a->d_beta; p.dg = a->d_g; p.ds0 = a->d_initial_state;
   p.dv = a->dv; p.gate = a->gate; p.scale = a->scale;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
+  if (lnx_chunk_direct(a)) {
+    DirectParams d = {};
+    d.geom = p.geom;
+    d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
+    d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.dv = a->dv; d.vcols = a->dv; d.gate = a->gate;
+    d.scale = a->scale; d.ws = p.ws; d.off = w;
+    d.d_o = reinterpret_cast<const bf16_t*>(a->d_o); d.d_sT = a->d_final_state;
+    d.dq = reinterpret_cast<bf16_t*>(a->d_q); d.dk = reinterpret_cast<bf16_t*>(a->d_k);
+    d.dv_out = reinterpret_cast<bf16_t*>(a->d_v); d.dbeta = a->d_beta; d.dg = a->d_g; d.ds0 = a->d_initial_state;
+    rc = lnx_direct_bwd(d, a->dk, a->gate, nstate, st);
+    if (rc != LNX_OK) return rc;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk backward launch: %s", hipGetErrorString(e));
+    return LNX_OK;
+  }
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 256)   ? launch_bwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
          : (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st)

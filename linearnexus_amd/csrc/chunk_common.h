@@ -105,8 +105,17 @@ __device__ __forceinline__ bool xcd_slot_part(int64_t slots, int parts, int64_t&
 inline unsigned lnx_xcd_grid(int64_t slots, int parts) { return (unsigned)(((slots + 7) / 8) * 8 * parts); }
 
 struct ChunkWs {
-  uint64_t tab, G, P, X, W, U, Kr, Qg, TmT, D, SnT, dD, dSn, dW, dG, total;
+  uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, TmT, D, SnT, dD, dSn, dW, dG, total;
 };
+
+// 2-byte inputs and outputs with dk <= 128 and no per-channel gate take the kernels of chunk_direct.hip, which keep G, Pm,
+// Tm, the per-chunk states and state gradients, D and dR in the workspace (no W, U, dW).  LNX_CHUNK_DIRECT=0 in the environment sends them through the
+// general kernels instead (used by the tests to keep those covered at small shapes).
+inline bool lnx_chunk_direct(const lnx_scan_args* a) {
+  if (a->dtype != LNX_BF16 || a->o_dtype != LNX_BF16 || a->dk > 128 || a->gate == LNX_GATE_VECTOR) return false;
+  const char* e = getenv("LNX_CHUNK_DIRECT");
+  return !(e && e[0] == '0');
+}
 
 inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
 
@@ -128,6 +137,19 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   uint64_t off = 0;
   auto take = [&](uint64_t bytes) { uint64_t o = off; off = lnx_align256(off + bytes); return o; };
   w.tab = take(a->cu_seqlens ? (2 * N + 2 * (uint64_t)a->nseq + 1) * 4 : 0);
+  if (lnx_chunk_direct(a)) {
+    w.X = w.W = w.U = w.Kr = w.Qg = w.TmT = w.dW = w.dG = 0;
+    w.G = take(slots * C * 4);
+    w.P = take(slots * C * C * es);
+    w.Tm = take(slots * C * C * es);
+    w.SnT = take(bwd ? slots * dv * dk * es : 0);   // states entering the chunks, [v][k]
+    w.dSn = take(bwd ? slots * dk * dv * es : 0);   // state gradients leaving the chunks, [v][k]
+    w.D = take(bwd ? slots * dv * C * es : 0);      // D^T  [v][token]
+    w.dD = take(bwd ? slots * dv * C * es : 0);     // dR^T [v][token]
+    w.total = off;
+    return w;
+  }
+  w.Tm = 0;
   w.G = take(vec ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
   w.X = take(vec && saved ? slots * C * C * es : 0);
@@ -155,6 +177,36 @@ inline bool lnx_narrow_slabs(int64_t wide_workgroups) {
   if (e && e[0] == '6') return false;
   return wide_workgroups <= 128;
 }
+
+// Arguments of the kernels of chunk_direct.hip (2-byte inputs).
+struct DirectParams {
+  ChunkGeom geom;
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  const float* beta;
+  const float* s0;
+  float* sT_out;
+  void* o;
+  int dv, o_dtype;
+  int save;   // forward scan: write the state entering every chunk (the backward pass reads it)
+  int vcols;  // leading value columns present in v (its row length); the rest of the dv columns are zero
+  int gate;
+  float scale;
+  char* ws;
+  ChunkWs off;
+  // backward only
+  const bf16_t* d_o;
+  const float* d_sT;
+  bf16_t* dq;
+  bf16_t* dk;
+  bf16_t* dv_out;
+  float* dbeta;
+  float* dg;
+  float* ds0;
+};
+int lnx_direct_scan_fwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st);
+int lnx_direct_bwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st);
 
 // Shared argument validation of the chunk entry points; returns LNX_OK or an error status.
 int lnx_chunk_check(const lnx_scan_args* a, bool backward);

@@ -1,0 +1,923 @@
+// Chunked delta-rule forward and backward for 2-byte inputs with dk <= 128 and no / a scalar gate, in the
+// "direct solve" split: the only per-chunk tensors that cross kernels are Tm = (I + A)^-1, Pm = scale tril(E * Q K^T)
+// and the cumulative gate G from the chunk-parallel prepare kernel, the states entering the chunks (forward scan ->
+// chunk-local backward) and the state gradients leaving them (reverse scan -> chunk-local backward).  W, U, D, dD, dW
+// of the WY form are never materialised: with S the state entering a chunk,
+//
+//   Y = K S          R = diag(beta) (V - diag(e^G) Y)      D = Tm R                     (forward substitution applied
+//   O = scale diag(e^G) (Q S) + Pm D                                                     to the chunk's right-hand
+//   S' = e^{G_C} S + (diag(e^{G_C - G}) K)^T D                                           side, gated_deltanet.py:450-477)
+//
+// and in reverse, with dS' the gradient of the state leaving the chunk,
+//
+//   dD = Pm^T dO + diag(e^{G_C - G}) K dS'     dR = Tm^T dD     dY = -diag(beta e^G) dR
+//   dS = e^{G_C} dS' + (scale diag(e^G) Q)^T dO + K^T dY
+//
+// which is the algorithm of linearnexus/modules/linear_attn/gated_deltanet.py:444-523 (delta_net.py:296-330 without
+// a gate) and its hand-derived adjoint (the reference's gradients come from JAX autodiff).  Three kernels:
+//
+//   scan_fwd   (one workgroup per (state, slab of dv), sequential over chunks)   O, the entering states, S_T
+//   scan_bwd   (same grid, reverse)                                              the leaving state gradients, dS_0
+//   bwd_chunk  (one workgroup per chunk, all in parallel)                         dq, dk, dv, dbeta, dg -- recomputes
+//              Y, D, dD, dR of its chunk from q, k, v, dO and the two saved states
+//
+// Both scans split their 512 threads into four compute waves (matrix work on the tiles in LDS, the fp32 state in MFMA
+// accumulators for the whole sequence) and four mover waves (global loads two chunks ahead into registers, tile
+// writes into LDS as soon as a tile's last reader is past, LDS -> global copies of results as whole rows); K, Pm and
+// the per-token scalars are double-buffered in LDS so that three LDS-only barriers per chunk suffice.
+
+#include <type_traits>
+
+#include "chunk_common.h"
+
+namespace {
+
+using T = bf16_t;
+typedef Mma<T> M;
+
+template <typename X> __device__ __forceinline__ X* at(char* ws, uint64_t off) { return reinterpret_cast<X*>(ws + off); }
+
+// dst[col][row0 + ...] = fragment (transposed store, four consecutive rows per 8-byte vector)
+__device__ __forceinline__ void store_frag_t(const floatx16& a, T* dst, int ld, int lane) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const floatx4 x = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+    store4(dst + (lane & 31) * ld + 8 * q + 4 * (lane >> 5), x);
+  }
+}
+
+// Per-token scalars of one chunk in LDS, written by the movers when they commit a chunk
+struct Scal {
+  enum { BETA = 0, GAM = 64, R = 128, SG = 192, DEC = 256, SIZE = 320 };  // beta, e^G, e^{G_C - G}, scale e^G, e^{G_C}
+};
+
+// ---------------------------------------------------------------------------------------
+// scan_fwd.  A compute wave owns a 32-column strip of the value slab: its [dk x 32] part of the state stays in MFMA
+// accumulators for the whole sequence, and the chain  S -> Y = K S -> R -> D = Tm R -> S'  never leaves the wave's
+// registers -- an accumulator fragment is the B operand of the next product as it is (Mma::from_acc), only the A
+// operands (K, Q, Tm, Pm rows) come from LDS.  All five input tiles are double-buffered, so the movers write chunk
+// n + 1 while chunk n is being read and two barriers per chunk are enough:
+//   B1    buffers of chunk n complete           compute: S^T -> LDS (saved states), Y, Q S, R, D (-> LDS, transposed), O -> LDS
+//                                               movers:  loads of chunk n + 2; chunk n + 1 -> the other buffers
+//   Bmid  O, S^T and D^T are in LDS             compute: state update        movers: O, S^T, D^T -> global
+// ---------------------------------------------------------------------------------------
+template <int DK, int BVW> struct FScanL {
+  static constexpr int PAD = M::PAD, LDK = DK + PAD, LDC = LNX_C + PAD, BV = BVW, LDV = BV + PAD, NCW = BV / 32;
+  static constexpr int kK = 64 * LDK, kST = BV * LDK, kV = 64 * LDV, kC = 64 * LDC;
+  static constexpr int kDT = BV * LDC;
+  // [2] x (K, Q, V, Tm, Pm) | O | S^T | D^T | scalars [2]
+  static constexpr size_t bytes = sizeof(T) * (2 * (2 * kK + kV + 2 * kC) + kV + kST + kDT) + sizeof(float) * 2 * Scal::SIZE;
+  static constexpr int threads = 64 * NCW + 256;
+};
+
+template <int DK, int GATE, int BVW>
+__global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(DirectParams p) {
+  typedef FScanL<DK, BVW> L;
+  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDV = L::LDV, NCW = L::NCW;
+  constexpr int KT = DK / 32;  // row tiles of the state strip
+  static_assert(DK == 64 || DK == 128, "dk = 64 or 128");
+  extern __shared__ __align__(16) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);  // [2][64][LDK]
+  T* sQ = sK + 2 * L::kK;
+  T* sV = sQ + 2 * L::kK;              // [2][64][LDV]
+  T* sTm = sV + 2 * L::kV;             // [2][64][LDC]
+  T* sP = sTm + 2 * L::kC;
+  T* sO = sP + 2 * L::kC;              // bf16 outputs on their way out [64][LDV]
+  T* sST = sO + L::kV;                 // entering state, transposed [v][dk], on its way to the workspace
+  T* sDT = sST + L::kST;               // D^T [v][token] on its way to the workspace
+  float* sSc = reinterpret_cast<float*>(sDT + L::kDT);  // [2][Scal::SIZE]
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  int sidx, row, seq;
+  int64_t chain;
+  int slab;
+  if (!xcd_slot_part((int64_t)(p.geom.tab ? p.geom.nseq : p.geom.rows / p.geom.H) * p.geom.H, p.dv / BV, chain, slab)) return;
+  scan_state(p.geom, (int)chain, sidx, row, seq);
+  const int v0 = slab * BV;
+  int c0, c1;
+  seq_chunks(p.geom, seq, c0, c1);
+  const SeqSpan span = seq_span(p.geom, seq, c0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.vcols, tso = (int64_t)p.geom.ts * p.dv;
+
+  if (wave >= NCW) {
+    // ---------------- movers ----------------
+    const int mt = tid - 64 * NCW;
+    struct Tiles {
+      TileRegs<T, 64, DK> K, Q;
+      TileRegs<T, 64, BV> V;
+      TileRegs<T, 64, 64> Tm, P;
+      float g, gc, b;
+      int len;
+    };
+    Tiles ta, tb;
+    ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
+    ta.len = tb.len = 0;
+    auto fetch = [&](Tiles& R, int n) {
+      const int64_t slot = (int64_t)row * N + n;
+      int tok0;
+      chunk_span(span, n, tok0, R.len);
+      const int64_t tbase = tok_index(p.geom, row, tok0);
+      R.K.load(p.k + tbase * DK, tsk, R.len, mt);
+      R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      R.V.load(p.v + tbase * p.vcols + v0, tsv, (v0 < p.vcols) ? R.len : 0, mt);  // columns v does not hold read as zero
+      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
+      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      // every thread loads the scalars of token mt % 64 (no load behind a branch); tokens past the end are masked below
+      const int t = mt & 63;
+      if (GATE == LNX_GATE_SCALAR) {
+        R.g = at<const float>(p.ws, p.off.G)[slot * 64 + t];
+        R.gc = at<const float>(p.ws, p.off.G)[slot * 64 + 63];
+      }
+      R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
+    };
+    auto commit = [&](const Tiles& R, int pb) {
+      R.K.store(sK + pb * L::kK, LDK, mt);
+      R.Q.store(sQ + pb * L::kK, LDK, mt);
+      R.V.store(sV + pb * L::kV, LDV, mt);
+      R.Tm.store(sTm + pb * L::kC, LDC, mt);
+      R.P.store(sP + pb * L::kC, LDC, mt);
+      if (mt < 64) {
+        float* sc = sSc + pb * Scal::SIZE;
+        const float gam = (GATE == LNX_GATE_SCALAR) ? __expf(R.g) : 1.f;
+        sc[Scal::BETA + mt] = (mt < R.len) ? R.b : 0.f;
+        sc[Scal::GAM + mt] = gam;
+        sc[Scal::R + mt] = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(R.gc - R.g, 0.f)) : 1.f;
+        sc[Scal::SG + mt] = p.scale * gam;
+        if (mt == 0) sc[Scal::DEC] = (GATE == LNX_GATE_SCALAR) ? __expf(R.gc) : 1.f;
+      }
+    };
+    // cur: the register set that held chunk n (in LDS since the last step) and now takes chunk n + 2; nxt: chunk n + 1.
+    // `steady` (a std::bool_constant): chunks n + 1 and n + 2 exist, so nothing below sits behind a branch -- behind a
+    // conditional fetch the compiler cannot count the younger loads in flight and would wait for all of them.
+    auto step = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
+      constexpr bool STEADY = decltype(steady)::value;
+      if (STEADY || n + 2 < c1) fetch(cur, n + 2);
+      if (STEADY || n + 1 < c1) commit(nxt, (n + 1 - c0) & 1);
+      lds_barrier();  // Bmid
+      int tok0, len;
+      chunk_span(span, n, tok0, len);
+      if (p.o)
+        unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
+      if (p.save) {
+        const int64_t slot = (int64_t)row * N + n;
+        unstage_tile<T, BV, DK, true>(at<T>(p.ws, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
+        unstage_tile<T, BV, 64, true>(at<T>(p.ws, p.off.D) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sDT, LDC, BV, mt);
+      }
+      lds_barrier();  // B1 of the next chunk
+    };
+    // the register sets and the LDS double buffers alternate by position in the sequence (chunk c0: set a, buffer 0)
+    if (c0 < c1) {
+      fetch(ta, c0);
+      commit(ta, 0);
+    }
+    if (c0 + 1 < c1) fetch(tb, c0 + 1);
+    lds_barrier();  // B1 of the first chunk
+    int n = c0;
+    for (; n + 3 < c1; n += 2) {  // chunks n + 2 and n + 3 exist
+      step(ta, tb, n, std::true_type{});
+      step(tb, ta, n + 1, std::true_type{});
+    }
+    for (; n < c1; n += 2) {
+      step(ta, tb, n, std::false_type{});
+      if (n + 1 < c1) step(tb, ta, n + 1, std::false_type{});
+    }
+    return;
+  }
+
+  // ---------------- compute waves: wave w owns value columns [32 w, 32 w + 32) of the slab ----------------
+  const int vs = 32 * wave;
+  const int fr = lane & 31;
+  floatx16 S[KT];
+#pragma unroll
+  for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) S[ci][e] = 0.f;
+  if (p.s0) {
+    const float* s0 = p.s0 + (int64_t)sidx * DK * p.dv + v0 + vs;
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) S[ci][e] = s0[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv + frag_col(lane)];
+  }
+  lds_barrier();  // B1 of the first chunk
+  for (int n = c0; n < c1; ++n) {
+    const int pb = (n - c0) & 1;
+    const T* sKc = sK + pb * L::kK;
+    const T* sQc = sQ + pb * L::kK;
+    const T* sVc = sV + pb * L::kV;
+    const T* sTc = sTm + pb * L::kC;
+    const T* sPc = sP + pb * L::kC;
+    const float* sc = sSc + pb * Scal::SIZE;
+    if (p.save) {
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) store_frag_t(S[ci], sST + vs * LDK + 32 * ci, LDK, lane);
+    }
+    // ---- Y = K S and Q S: the state fragments are the B operands ----
+    floatx16 y[2], o[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) y[i][e] = o[i][e] = 0.f;
+    {
+      // A fragments one step ahead of the products; the scheduling fences keep the compiler from hoisting every read
+      // of the unrolled loop to its top (and spilling the state for it)
+      M::Frag fk[2][2], fq[2][2];  // [step parity][row tile]: the unrolled loop names them statically
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fk[0][i] = M::load_chain(sKc + (32 * i + fr) * LDK, lane);
+        fq[0][i] = M::load_chain(sQc + (32 * i + fr) * LDK, lane);
+      }
+#pragma unroll
+      for (int ks = 0; ks < DK / 16; ++ks) {
+        if (ks + 1 < DK / 16) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            fk[(ks + 1) & 1][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * (ks + 1), lane);
+            fq[(ks + 1) & 1][i] = M::load_chain(sQc + (32 * i + fr) * LDK + 16 * (ks + 1), lane);
+          }
+        }
+        const M::Frag b = M::from_acc(S[ks >> 1], ks & 1);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          M::mma(y[i], fk[ks & 1][i], b);
+          M::mma(o[i], fq[ks & 1][i], b);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- R = beta (V - e^G Y), in place of Y ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 vv = M::load_acc_rows(sVc, LDV, 32 * i, q, vs, lane);
+        const int t0 = 32 * i + 8 * q + 4 * (lane >> 5);
+        const floatx4 bt = load4(sc + Scal::BETA + t0), gm = load4(sc + Scal::GAM + t0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) y[i][4 * q + u] = bt[u] * (vv[u] - gm[u] * y[i][4 * q + u]);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- D = Tm R ----
+    floatx16 d[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) d[i][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::from_acc(y[ks >> 1], ks & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(d[i], M::load_chain(sTc + (32 * i + fr) * LDC + 16 * ks, lane), b);
+    }
+    if (p.save) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) store_frag_t(d[i], sDT + vs * LDC + 32 * i, LDC, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- O = scale e^G (Q S) + Pm D ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 sg = load4(sc + Scal::SG + 32 * i + 8 * q + 4 * (lane >> 5));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o[i][4 * q + u] *= sg[u];
+      }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::from_acc(d[ks >> 1], ks & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(o[i], M::load_chain(sPc + (32 * i + fr) * LDC + 16 * ks, lane), b);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sO[(32 * i + frag_row(e, lane)) * LDV + vs + frag_col(lane)] = (bf16_t)o[i][e];
+    lds_barrier();  // Bmid
+    // ---- S <- e^{G_C} S + K^T (e^{G_C - G} D) ----
+    if (GATE == LNX_GATE_SCALAR) {
+      const float dec = sc[Scal::DEC];
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[ci][e] *= dec;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const floatx4 rr = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
+#pragma unroll
+          for (int u = 0; u < 4; ++u) d[i][4 * q + u] *= rr[u];
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::from_acc(d[ks >> 1], ks & 1);
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(S[ci], M::load_t_chain(sKc, LDK, 16 * ks, 32 * ci, lane), b);
+    }
+    lds_barrier();  // B1 of the next chunk
+  }
+  float* out = p.sT_out + (int64_t)sidx * DK * p.dv + v0 + vs + frag_col(lane);
+#pragma unroll
+  for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) out[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv] = S[ci][e];
+}
+
+template <int DK, int GATE>
+int launch_scan_fwd(const DirectParams& p, int nstate, hipStream_t st) {
+  // 32-column slabs (one compute wave) when 64-column ones would occupy at most half of the chip
+  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  auto k = narrow ? scan_fwd_kernel<DK, GATE, 32> : scan_fwd_kernel<DK, GATE, 64>;
+  const size_t b = narrow ? FScanL<DK, 32>::bytes : FScanL<DK, 64>::bytes;
+  const int bv = narrow ? 32 : 64, threads = narrow ? FScanL<DK, 32>::threads : FScanL<DK, 64>::threads;
+  hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b);
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  lnx_profile_mark("chunk_scan", st);
+  hipLaunchKernelGGL(k, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(threads), b, st, p);
+  lnx_profile_mark(nullptr, st);
+  return LNX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// scan_bwd: the reverse pass, same organisation as scan_fwd.  A compute wave owns a 32-column strip of dS (the
+// gradient of the state leaving the chunk); the chain  dS' -> Z = K dS' -> dD -> dR = Tm^T dD -> dY -> dS  stays in
+// its registers.  Needs no forward state: only K, Q, dO, Tm, Pm and the per-token scalars.
+//   B1    buffers of chunk n complete           compute: dS'^T -> LDS (saved), Z, Pm^T dO, dD, dR (-> LDS, transposed),
+//                                                        dv = beta dR -> LDS, dY
+//                                               movers:  loads of chunk n - 2; chunk n - 1 -> the other buffers
+//   Bmid  dS'^T, dR^T and dv are in LDS         compute: dS update          movers: dS'^T, dR^T -> workspace, dv out
+// ---------------------------------------------------------------------------------------
+template <int DK, int BVW> struct BScanL {
+  static constexpr int PAD = M::PAD, LDK = DK + PAD, LDC = LNX_C + PAD, BV = BVW, LDV = BV + PAD, NCW = BV / 32;
+  static constexpr int kK = 64 * LDK, kST = BV * LDK, kV = 64 * LDV, kC = 64 * LDC;
+  static constexpr int kDT = BV * LDC;
+  // [2] x (K, scaled Q, dO, Tm, Pm) | dS'^T | dR^T | dv | scalars [2]
+  static constexpr size_t bytes = sizeof(T) * (2 * (2 * kK + kV + 2 * kC) + kST + kDT + kV) + sizeof(float) * 2 * Scal::SIZE;
+  static constexpr int threads = 64 * NCW + 256;
+};
+
+template <int DK, int GATE, int BVW>
+__global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(DirectParams p) {
+  typedef BScanL<DK, BVW> L;
+  constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDV = L::LDV, NCW = L::NCW;
+  constexpr int KT = DK / 32;
+  extern __shared__ __align__(16) char smem[];
+  T* sK = reinterpret_cast<T*>(smem);  // [2][64][LDK]
+  T* sQ = sK + 2 * L::kK;              // rows scaled by scale e^G
+  T* sdO = sQ + 2 * L::kK;             // [2][64][LDV]
+  T* sTm = sdO + 2 * L::kV;
+  T* sP = sTm + 2 * L::kC;
+  T* sdST = sP + 2 * L::kC;            // dS'^T [v][dk] on its way to the workspace
+  T* sdRT = sdST + L::kST;             // dR^T [v][token] on its way to the workspace
+  T* sdV = sdRT + L::kDT;              // dv = beta dR [token][v] on its way out
+  float* sSc = reinterpret_cast<float*>(sdV + L::kV);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  int sidx, row, seq;
+  int64_t chain;
+  int slab;
+  if (!xcd_slot_part((int64_t)(p.geom.tab ? p.geom.nseq : p.geom.rows / p.geom.H) * p.geom.H, p.dv / BV, chain, slab)) return;
+  scan_state(p.geom, (int)chain, sidx, row, seq);
+  const int v0 = slab * BV;
+  int c0, c1;
+  seq_chunks(p.geom, seq, c0, c1);
+  const SeqSpan span = seq_span(p.geom, seq, c0);
+  const int64_t tsk = (int64_t)p.geom.ts * DK, tsv = (int64_t)p.geom.ts * p.dv;
+
+  if (wave >= NCW) {
+    // ---------------- movers ----------------
+    const int mt = tid - 64 * NCW;
+    typedef TileRegs<T, 64, DK> RowTile;
+    struct Tiles {
+      RowTile K, Q;
+      TileRegs<T, 64, BV> dO;
+      TileRegs<T, 64, 64> Tm, P;
+      float g, gc, b;
+      float gq[RowTile::IT];  // G of the token each of this thread's Q vectors belongs to
+      int len;
+    };
+    Tiles ta, tb;
+    ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
+    ta.len = tb.len = 0;
+#pragma unroll
+    for (int it = 0; it < RowTile::IT; ++it) ta.gq[it] = tb.gq[it] = 0.f;
+    auto fetch = [&](Tiles& R, int n) {
+      const int64_t slot = (int64_t)row * N + n;
+      int tok0;
+      chunk_span(span, n, tok0, R.len);
+      const int64_t tbase = tok_index(p.geom, row, tok0);
+      R.K.load(p.k + tbase * DK, tsk, R.len, mt);
+      R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      R.dO.load(p.d_o + tbase * p.dv + v0, tsv, R.len, mt);
+      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
+      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      const int t = mt & 63;
+      if (GATE == LNX_GATE_SCALAR) {
+        const float* G = at<const float>(p.ws, p.off.G) + slot * 64;
+        R.g = G[t];
+        R.gc = G[63];
+#pragma unroll
+        for (int it = 0; it < RowTile::IT; ++it) R.gq[it] = G[(mt + 256 * it) / RowTile::VPR];
+      }
+      R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
+    };
+    auto commit = [&](const Tiles& R, int pb) {
+      R.K.store(sK + pb * L::kK, LDK, mt);
+      {  // Q rows scaled by scale e^{G_i}: (scale diag(e^G) Q)^T dO needs no scaled copy of dO then
+        T* dst = sQ + pb * L::kK;
+#pragma unroll
+        for (int it = 0; it < RowTile::IT; ++it) {
+          const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
+          const float f = (GATE == LNX_GATE_SCALAR) ? p.scale * __expf(R.gq[it]) : p.scale;
+          typename Vec16<T>::V x = R.Q.x[it];
+#pragma unroll
+          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f);
+          *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+        }
+      }
+      R.dO.store(sdO + pb * L::kV, LDV, mt);
+      R.Tm.store(sTm + pb * L::kC, LDC, mt);
+      R.P.store(sP + pb * L::kC, LDC, mt);
+      if (mt < 64) {
+        float* sc = sSc + pb * Scal::SIZE;
+        const float gam = (GATE == LNX_GATE_SCALAR) ? __expf(R.g) : 1.f;
+        const float bt = (mt < R.len) ? R.b : 0.f;
+        sc[Scal::BETA + mt] = bt;
+        sc[Scal::GAM + mt] = bt * gam;  // beta e^G: dY = -(beta e^G) dR
+        sc[Scal::R + mt] = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(R.gc - R.g, 0.f)) : 1.f;
+        if (mt == 0) sc[Scal::DEC] = (GATE == LNX_GATE_SCALAR) ? __expf(R.gc) : 1.f;
+      }
+    };
+    // cur: the register set that held chunk n and now takes chunk n - 2; nxt: chunk n - 1 (see scan_fwd)
+    auto step = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
+      constexpr bool STEADY = decltype(steady)::value;
+      if (STEADY || n - 2 >= c0) fetch(cur, n - 2);
+      if (STEADY || n - 1 >= c0) commit(nxt, (c1 - n) & 1);  // position of chunk n - 1 from the end: c1 - 1 - (n - 1)
+      lds_barrier();  // Bmid
+      const int64_t slot = (int64_t)row * N + n;
+      unstage_tile<T, BV, DK, true>(at<T>(p.ws, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
+      unstage_tile<T, BV, 64, true>(at<T>(p.ws, p.off.dD) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdRT, LDC, BV, mt);
+      int tok0, len;
+      chunk_span(span, n, tok0, len);
+      unstage_tile<T, 64, BV>(p.dv_out + tok_index(p.geom, row, tok0) * p.dv + v0, tsv, sdV, LDV, len, mt);
+      lds_barrier();  // B1 of the next chunk
+    };
+    if (c0 < c1) {
+      fetch(ta, c1 - 1);
+      commit(ta, 0);
+    }
+    if (c1 - 2 >= c0) fetch(tb, c1 - 2);
+    lds_barrier();  // B1 of the first chunk
+    int n = c1 - 1;
+    for (; n - 3 >= c0; n -= 2) {  // chunks n - 2 and n - 3 exist
+      step(ta, tb, n, std::true_type{});
+      step(tb, ta, n - 1, std::true_type{});
+    }
+    for (; n >= c0; n -= 2) {
+      step(ta, tb, n, std::false_type{});
+      if (n - 1 >= c0) step(tb, ta, n - 1, std::false_type{});
+    }
+    return;
+  }
+
+  // ---------------- compute waves ----------------
+  const int vs = 32 * wave;
+  const int fr = lane & 31;
+  floatx16 dS[KT];
+#pragma unroll
+  for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dS[ci][e] = 0.f;
+  if (p.d_sT) {
+    const float* src = p.d_sT + (int64_t)sidx * DK * p.dv + v0 + vs;
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dS[ci][e] = src[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv + frag_col(lane)];
+  }
+  lds_barrier();  // B1 of the first chunk
+  for (int n = c1 - 1; n >= c0; --n) {
+    const int pb = (c1 - 1 - n) & 1;
+    const T* sKc = sK + pb * L::kK;
+    const T* sQc = sQ + pb * L::kK;
+    const T* sOc = sdO + pb * L::kV;
+    const T* sTc = sTm + pb * L::kC;
+    const T* sPc = sP + pb * L::kC;
+    const float* sc = sSc + pb * Scal::SIZE;
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci) store_frag_t(dS[ci], sdST + vs * LDK + 32 * ci, LDK, lane);
+    // ---- Z = K dS' (the state-gradient fragments are the B operands) and the chunk-local part Pm^T dO ----
+    floatx16 z[2], dd[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) z[i][e] = dd[i][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < DK / 16; ++ks) {
+      const M::Frag b = M::from_acc(dS[ks >> 1], ks & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(z[i], M::load_chain(sKc + (32 * i + fr) * LDK + 16 * ks, lane), b);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::load_t(sOc, LDV, 16 * ks, vs, lane);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(dd[i], M::load_t(sPc, LDC, 16 * ks, 32 * i, lane), b);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- dD = Pm^T dO + e^{G_C - G} Z ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 rr = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) dd[i][4 * q + u] += rr[u] * z[i][4 * q + u];
+      }
+    // ---- dR = Tm^T dD, dY = -beta e^G dR (in z) ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) z[i][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::from_acc(dd[ks >> 1], ks & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(z[i], M::load_t_chain(sTc, LDC, 16 * ks, 32 * i, lane), b);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      store_frag_t(z[i], sdRT + vs * LDC + 32 * i, LDC, lane);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int t0 = 32 * i + 8 * q + 4 * (lane >> 5);
+        const floatx4 bt = load4(sc + Scal::BETA + t0), bg = load4(sc + Scal::GAM + t0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          sdV[(t0 + u) * LDV + vs + fr] = (bf16_t)(bt[u] * z[i][4 * q + u]);
+          z[i][4 * q + u] *= -bg[u];
+        }
+      }
+    }
+    lds_barrier();  // Bmid
+    // ---- dS <- e^{G_C} dS' + (scale e^G Q)^T dO + K^T dY ----
+    if (GATE == LNX_GATE_SCALAR) {
+      const float dec = sc[Scal::DEC];
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dS[ci][e] *= dec;
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::load_t(sOc, LDV, 16 * ks, vs, lane);
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], M::load_t(sQc, LDK, 16 * ks, 32 * ci, lane), b);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const M::Frag b = M::from_acc(z[ks >> 1], ks & 1);
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], M::load_t_chain(sKc, LDK, 16 * ks, 32 * ci, lane), b);
+    }
+    lds_barrier();  // B1 of the next chunk
+  }
+  if (p.ds0) {
+    float* out = p.ds0 + (int64_t)sidx * DK * p.dv + v0 + vs + frag_col(lane);
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) out[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv] = dS[ci][e];
+  }
+}
+
+template <int DK, int GATE>
+int launch_scan_bwd(const DirectParams& p, int nstate, hipStream_t st) {
+  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  auto k = narrow ? scan_bwd_kernel<DK, GATE, 32> : scan_bwd_kernel<DK, GATE, 64>;
+  const size_t b = narrow ? BScanL<DK, 32>::bytes : BScanL<DK, 64>::bytes;
+  const int bv = narrow ? 32 : 64, threads = narrow ? BScanL<DK, 32>::threads : BScanL<DK, 64>::threads;
+  hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b);
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  lnx_profile_mark("bwd_scan", st);
+  hipLaunchKernelGGL(k, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(threads), b, st, p);
+  return LNX_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// bwd_chunk: the chunk-local gradients, one workgroup per chunk, all chunks in parallel.  Reads q, k, v, dO of the
+// chunk, the states S (entering) and dS' (leaving) and D, dR from the two scans; writes dq, dk, dbeta, dg (dv left
+// the reverse scan).  A loop over 32-column slabs of the value dimension accumulates every product that contracts
+// over value columns (next slab's tiles prefetched into registers):
+//   dQa = dO S^T     dK1 = dR S^T     dK2 = D dS'^T     dPm = dO D^T     dAm = dR D^T     <dR_t, v_t>     <dS', S>
+// then an epilogue over the chunk's tokens:
+//   dPe = scale tril(E * dPm)          dXa = -tril(E * dAm, -1)          dXe = diag(beta) dXa
+//   dq  = scale e^G dQa + dPe K
+//   row = dXa K - e^G dK1              m_t = <k_t, row_t>                 dbeta = <dR, v> + m
+//   dk  = beta row + e^{G_C - G} dK2 + dPe^T Q + dXe^T K
+//   dG  = <q, dq> - <k, dk> + 2 beta m;   dG_C += sum_t e^{G_C - G_t} <k_t, dK2_t> + e^{G_C} <dS', S>;   dg = reverse cumsum(dG)
+// Wave (wi, wj) owns the token-row tile wi and the key-column tiles NKT wj .. of the [64 x dk] accumulators and the
+// (wi, wj) tile of the [64 x 64] ones.  Tiles that are only read through transposing LDS loads get a row stride of
+// 64 bytes mod 256, which spreads the four rows a 16-lane group reads over all banks.
+// ---------------------------------------------------------------------------------------
+template <int DK> struct BChunkL {
+  static constexpr int SV = 32;
+  static constexpr int LDV = SV + 8;       // dO, V slabs [64][SV], read by rows
+  static constexpr int LDT = 64 + 32;      // D^T, dR^T slabs [SV][64], transposing reads only
+  static constexpr int LDKT = DK + 32;     // S^T, dS'^T slabs [SV][DK] and the K, Q tiles [64][DK], transposing reads
+  static constexpr int LDC = 64 + 8;       // dPe, dPe^T, dXa, dXe^T [64][64], read by rows
+  static constexpr int LDK = DK + 8;       // staging tile for dq, dk [64][DK]
+  static constexpr int kTok = 64 * LDV, kT = SV * LDT, kSt = SV * LDKT, kC = 64 * LDC, kRow = 64 * LDKT;
+  static constexpr size_t loop_bytes = sizeof(T) * (2 * kTok + 2 * kT + 2 * kSt);
+  static constexpr size_t epi_bytes = sizeof(T) * (2 * kRow + 4 * kC);
+  static_assert(64 * LDK <= 2 * kC, "the staging tile overlays dPe and dPe^T");
+  static constexpr int nfloat = 64 * 6;
+  static constexpr size_t bytes = sizeof(float) * nfloat + (epi_bytes > loop_bytes ? epi_bytes : loop_bytes);
+};
+
+template <int DK, int GATE>
+__global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
+  typedef BChunkL<DK> L;
+  constexpr int SV = L::SV, LDV = L::LDV, LDT = L::LDT, LDKT = L::LDKT, LDC = L::LDC, LDK = L::LDK;
+  constexpr int NKT = DK / 64;  // key-column tiles per wave
+  extern __shared__ __align__(16) char smem[];
+  float* sG = reinterpret_cast<float*>(smem);
+  float* sBeta = sG + 64;
+  float* sRdv = sBeta + 64;   // <dR_t, v_t>
+  float* sM = sRdv + 64;      // m_t
+  float* sdG = sM + 64;
+  float* sMisc = sdG + 64;    // [0] = sum_t r_t <k_t, dK2_t>, [1] = <dS', S>
+  T* tiles = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
+  // loop phase
+  T* sdO = tiles;
+  T* sV = sdO + L::kTok;
+  T* sDT = sV + L::kTok;
+  T* sdRT = sDT + L::kT;
+  T* sSn = sdRT + L::kT;
+  T* sdSn = sSn + L::kSt;
+  // epilogue
+  T* sPe = tiles;             // [i][j]
+  T* sPeT = sPe + L::kC;      // [j][i]
+  T* sXa = sPeT + L::kC;      // [i][j]
+  T* sXeT = sXa + L::kC;      // [j][i]
+  T* sK = sXeT + L::kC;       // [token][dk]
+  T* sQ = sK + L::kRow;
+  T* sSt = tiles;             // staging for dq, then dk, once the four small tiles are dead
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int N = p.geom.N;
+  const int64_t slot = blockIdx.x;
+  const int row = (int)(slot / N), n = (int)(slot % N);
+  int tok0, len;
+  chunk_span(p.geom, n, tok0, len);
+  if (len <= 0) return;
+  const int64_t tbase = tok_index(p.geom, row, tok0);
+  const int64_t ts = p.geom.ts, tsk = ts * DK, tsv = ts * p.dv;
+  const int wi = wave >> 1, wj = wave & 1;
+  const int fr = lane & 31, kg8 = 8 * (lane >> 5);
+
+  TileRegs<T, 64, SV> rdO, rV;
+  TileRegs<T, SV, 64> rDT, rdRT;
+  TileRegs<T, SV, DK> rSn, rdSn;
+  TileRegs<T, 64, DK> rK, rQ;
+  auto fetch = [&](int v0) {
+    rdO.load(p.d_o + tbase * p.dv + v0, tsv, len, tid);
+    rV.load(p.v + tbase * p.dv + v0, tsv, len, tid);
+    rDT.load(at<const T>(p.ws, p.off.D) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, SV, tid);
+    rdRT.load(at<const T>(p.ws, p.off.dD) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, SV, tid);
+    rSn.load(at<const T>(p.ws, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
+    rdSn.load(at<const T>(p.ws, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
+  };
+  floatx16 aP[1][1], aA[1][1], aQ[1][NKT], aK1[1][NKT], aK2[1][NKT];
+  frag_zero(aP);
+  frag_zero(aA);
+  frag_zero(aQ);
+  frag_zero(aK1);
+  frag_zero(aK2);
+  float ss = 0.f, rdv = 0.f;
+  fetch(0);  // first, so that the small loads below do not hold it up
+  if (tid < 64) {
+    sG[tid] = (GATE == LNX_GATE_SCALAR) ? at<const float>(p.ws, p.off.G)[slot * 64 + tid] : 0.f;
+    sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
+    sM[tid] = 0.f;
+    sMisc[tid] = 0.f;
+  }
+#pragma unroll 1
+  for (int v0 = 0; v0 < p.dv; v0 += SV) {
+    lds_barrier();  // the previous slab's tiles are dead
+    rdO.store(sdO, LDV, tid);
+    rV.store(sV, LDV, tid);
+    rDT.store(sDT, LDT, tid);
+    rdRT.store(sdRT, LDT, tid);
+    rSn.store(sSn, LDKT, tid);
+    rdSn.store(sdSn, LDKT, tid);
+    lds_barrier();
+    if (v0 + SV < p.dv) fetch(v0 + SV);
+    else {  // last slab: the epilogue's K and Q tiles instead
+      rK.load(p.k + tbase * DK, tsk, len, tid);
+      rQ.load(p.q + tbase * DK, tsk, len, tid);
+    }
+#pragma unroll
+    for (int k0 = 0; k0 < SV; k0 += 16) {
+      const M::Frag fdO = M::load(sdO + (32 * wi + fr) * LDV + k0 + kg8);
+      const M::Frag fdR = M::load_t(sdRT, LDT, k0, 32 * wi, lane);
+      const M::Frag fDi = M::load_t(sDT, LDT, k0, 32 * wi, lane);
+      const M::Frag fDj = M::load_t(sDT, LDT, k0, 32 * wj, lane);
+      M::mma(aP[0][0], fdO, fDj);
+      M::mma(aA[0][0], fdR, fDj);
+#pragma unroll
+      for (int c = 0; c < NKT; ++c) {
+        const M::Frag fS = M::load_t(sSn, LDKT, k0, 32 * (NKT * wj + c), lane);
+        const M::Frag fdS = M::load_t(sdSn, LDKT, k0, 32 * (NKT * wj + c), lane);
+        M::mma(aQ[0][c], fdO, fS);
+        M::mma(aK1[0][c], fdR, fS);
+        M::mma(aK2[0][c], fDi, fdS);
+      }
+    }
+    {  // <dR_t, v_t> over this slab: thread = (token tid / 4, eight value columns)
+      const int t = tid >> 2, c0 = 8 * (tid & 3);
+      const M::Frag vv = M::load(sV + t * LDV + c0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rdv += (float)vv[e] * (float)sdRT[(c0 + e) * LDT + t];
+    }
+    if (GATE == LNX_GATE_SCALAR) {  // <dS', S> over this slab: thread = (value row tid / 8, DK / 8 key columns)
+      const int r = tid >> 3, c0 = (tid & 7) * (DK / 8);
+#pragma unroll
+      for (int u = 0; u < DK / 8; u += 8) {
+        const M::Frag a = M::load(sSn + r * LDKT + c0 + u), b = M::load(sdSn + r * LDKT + c0 + u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += (float)a[e] * (float)b[e];
+      }
+    }
+  }
+  rdv += __shfl_xor(rdv, 1, LNX_WAVE);
+  rdv += __shfl_xor(rdv, 2, LNX_WAVE);
+  if ((tid & 3) == 0) sRdv[tid >> 2] = rdv;
+  if (GATE == LNX_GATE_SCALAR) {
+    ss = wave_sum(ss);
+    if (lane == 0) atomicAdd(&sMisc[1], ss);
+  }
+  lds_barrier();  // slab tiles are dead from here on
+
+  // ---- epilogue ----
+  {
+    floatx16 pe[1][1], xa[1][1], xe[1][1];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      pe[0][0][e] = (i >= j) ? p.scale * dec * aP[0][0][e] : 0.f;
+      xa[0][0][e] = (i > j) ? -dec * aA[0][0][e] : 0.f;
+      xe[0][0][e] = sBeta[i] * xa[0][0][e];
+    }
+    frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+    frag_store<T, 1, 1>(xa, sXa + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store_t<T, 1, 1>(xe, sXeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+  }
+  rK.store(sK, LDKT, tid);
+  rQ.store(sQ, LDKT, tid);
+  lds_barrier();
+  const float gC = sG[63];
+  // dq = scale e^G dQa + dPe K;   row = dXa K - e^G dK1 (in aK1)
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[32 * wi + frag_row(e, lane)]);
+#pragma unroll
+    for (int c = 0; c < NKT; ++c) {
+      aQ[0][c][e] *= p.scale * gm;
+      aK1[0][c][e] *= -gm;
+    }
+  }
+#pragma unroll
+  for (int k0 = 0; k0 < 64; k0 += 16) {
+    const M::Frag fPe = M::load(sPe + (32 * wi + fr) * LDC + k0 + kg8);
+    const M::Frag fXa = M::load(sXa + (32 * wi + fr) * LDC + k0 + kg8);
+#pragma unroll
+    for (int c = 0; c < NKT; ++c) {
+      const M::Frag fK = M::load_t(sK, LDKT, k0, 32 * (NKT * wj + c), lane);
+      M::mma(aQ[0][c], fPe, fK);
+      M::mma(aK1[0][c], fXa, fK);
+    }
+  }
+  // m_t = <k_t, row_t>;  chunk-end gate term sum_t r_t <k_t, dK2_t>;  dk <- beta row + r dK2 (in aK2)
+  {
+    float mv[16], tot = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int r = 32 * wi + frag_row(e, lane);
+      const float rr = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gC - sG[r], 0.f));
+      const float bt = sBeta[r];
+      mv[e] = 0.f;
+#pragma unroll
+      for (int c = 0; c < NKT; ++c) {
+        const float kk = (float)sK[r * LDKT + 32 * (NKT * wj + c) + fr];
+        mv[e] += kk * aK1[0][c][e];
+        aK2[0][c][e] *= rr;
+        tot += kk * aK2[0][c][e];
+        aK2[0][c][e] += bt * aK1[0][c][e];
+      }
+    }
+    rows_reduce_add<1>(mv, 32 * wi, lane, sM);
+    if (GATE == LNX_GATE_SCALAR) {
+      tot = wave_sum(tot);
+      if (lane == 0) atomicAdd(&sMisc[0], tot);
+    }
+  }
+  // dk += dPe^T Q + dXe^T K
+#pragma unroll
+  for (int k0 = 0; k0 < 64; k0 += 16) {
+    const M::Frag fPt = M::load(sPeT + (32 * wi + fr) * LDC + k0 + kg8);
+    const M::Frag fXt = M::load(sXeT + (32 * wi + fr) * LDC + k0 + kg8);
+#pragma unroll
+    for (int c = 0; c < NKT; ++c) {
+      M::mma(aK2[0][c], fPt, M::load_t(sQ, LDKT, k0, 32 * (NKT * wj + c), lane));
+      M::mma(aK2[0][c], fXt, M::load_t(sK, LDKT, k0, 32 * (NKT * wj + c), lane));
+    }
+  }
+  lds_barrier();  // the four small tiles are dead; sM and sMisc are complete
+  frag_store<T, 1, NKT>(aQ, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
+  lds_barrier();
+  unstage_tile<T, 64, DK>(p.dq + tbase * DK, tsk, sSt, LDK, len, tid);
+  float dgp = 0.f;  // <q_t, dq_t> - <k_t, dk_t> over this thread's quarter of the key columns; thread = (token tid / 4, quarter)
+  const int tr = tid >> 2, tq = (tid & 3) * (DK / 4);
+  if (GATE == LNX_GATE_SCALAR) {
+#pragma unroll
+    for (int u = 0; u < DK / 4; u += 4) {
+      const floatx4 a = load4(sSt + tr * LDK + tq + u), b = load4(sQ + tr * LDKT + tq + u);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dgp += a[e] * b[e];
+    }
+  }
+  lds_barrier();  // dq has left the staging tile
+  frag_store<T, 1, NKT>(aK2, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
+  lds_barrier();
+  unstage_tile<T, 64, DK>(p.dk + tbase * DK, tsk, sSt, LDK, len, tid);
+  if (GATE == LNX_GATE_SCALAR) {
+#pragma unroll
+    for (int u = 0; u < DK / 4; u += 4) {
+      const floatx4 a = load4(sSt + tr * LDK + tq + u), b = load4(sK + tr * LDKT + tq + u);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dgp -= a[e] * b[e];
+    }
+    dgp += __shfl_xor(dgp, 1, LNX_WAVE);
+    dgp += __shfl_xor(dgp, 2, LNX_WAVE);
+    if ((tid & 3) == 0) {
+      float d = dgp + 2.f * sBeta[tr] * sM[tr];
+      if (tr == 63) d += sMisc[0] + __expf(gC) * sMisc[1];
+      sdG[tr] = d;
+    }
+    lds_barrier();
+  }
+  if (wave == 0) {
+    const int t = lane;
+    if (t < len) p.dbeta[tbase + t * ts] = sRdv[t] + sM[t];
+    if (GATE == LNX_GATE_SCALAR) {  // dg = reverse cumulative sum of dG over the chunk
+      float d = sdG[t];
+#pragma unroll
+      for (int s_ = 1; s_ < 64; s_ <<= 1) {
+        const float y = __shfl_down(d, s_, LNX_WAVE);
+        if (t + s_ < 64) d += y;
+      }
+      if (t < len) p.dg[tbase + t * ts] = d;
+    }
+  }
+}
+
+template <int DK, int GATE>
+int launch_bwd_chunk(const DirectParams& p, hipStream_t st) {
+  auto k = bwd_chunk_kernel<DK, GATE>;
+  const size_t b = BChunkL<DK>::bytes;
+  hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b);
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  lnx_profile_mark("bwd_chunk", st);
+  hipLaunchKernelGGL(k, dim3((unsigned)((int64_t)p.geom.rows * p.geom.N)), dim3(256), b, st, p);
+  lnx_profile_mark(nullptr, st);
+  return LNX_OK;
+}
+
+template <int DK, int GATE>
+int launch_bwd(const DirectParams& p, int nstate, hipStream_t st) {
+  int rc = launch_scan_bwd<DK, GATE>(p, nstate, st);
+  if (rc != LNX_OK) return rc;
+  return launch_bwd_chunk<DK, GATE>(p, st);
+}
+
+}  // namespace
+
+int lnx_direct_scan_fwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {
+  if (dk == 128)
+    return gate == LNX_GATE_SCALAR ? launch_scan_fwd<128, LNX_GATE_SCALAR>(p, nstate, st) : launch_scan_fwd<128, LNX_GATE_NONE>(p, nstate, st);
+  return gate == LNX_GATE_SCALAR ? launch_scan_fwd<64, LNX_GATE_SCALAR>(p, nstate, st) : launch_scan_fwd<64, LNX_GATE_NONE>(p, nstate, st);
+}
+
+int lnx_direct_bwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {
+  if (dk == 128)
+    return gate == LNX_GATE_SCALAR ? launch_bwd<128, LNX_GATE_SCALAR>(p, nstate, st) : launch_bwd<128, LNX_GATE_NONE>(p, nstate, st);
+  return gate == LNX_GATE_SCALAR ? launch_bwd<64, LNX_GATE_SCALAR>(p, nstate, st) : launch_bwd<64, LNX_GATE_NONE>(p, nstate, st);
+}

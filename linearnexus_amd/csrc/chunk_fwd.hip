@@ -78,7 +78,9 @@ template <typename T, int DK> struct Prep2Cfg {
   static constexpr size_t bytes = r0 + r1 + r2;
 };
 
-template <typename T, int DK, int GATE>
+// LITE: stop after the inverse and leave Tm itself (row-major) next to Pm and G -- all that the kernels of
+// chunk_direct.hip read; V is not touched.
+template <typename T, int DK, int GATE, bool LITE = false>
 __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   typedef Prep2Cfg<T, DK> L;
   constexpr int LDC = L::LDC, NKS = DK / 64;
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     else if (64 * (s_ - NKS) < p.vcols) rIn.load(vg + 64 * (s_ - NKS), tsv, len, tid);
     else rIn.zero();  // value columns that v does not hold
   };
-  fetch(0);
+  if (!LITE) fetch(0);
   lds_barrier();  // slab tiles dead
   {
     floatx16 pe[1][1];
@@ -164,6 +166,14 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sKa, LDC, 64, tid);
   lds_barrier();  // Tm is built over the P tile
   tri_inverse_64(sA, sT, sX, tid);
+  if constexpr (LITE) {
+    T* Tm = ws_ptr<T>(p, p.off.Tm) + slot * 64 * 64;
+    for (int idx = tid; idx < 64 * 16; idx += 256) {
+      const int r = idx >> 4, c = (idx & 15) * 4;
+      store4(Tm + r * 64 + c, load4(sT + r * LNX_LDA + c));
+    }
+    return;
+  }
   {
     T* TmT = ws_ptr<T>(p, p.off.TmT) + slot * 64 * 64;
     // one 4x4 block of Tm per thread: four-element row reads, the transpose taken in registers
@@ -1096,6 +1106,37 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
 
 namespace {
 
+// 2-byte inputs with dk <= 128 and no per-channel gate: the prepare kernel stops at Tm, Pm and G, the scan of
+// chunk_direct.hip does the rest.
+template <int DK, int GATE>
+void launch_prepare_lite(const FwdParams& p, hipStream_t st) {
+  auto k = chunk_prepare2_kernel<bf16_t, DK, GATE, true>;
+  lnx_profile_mark("chunk_prepare", st);
+  const size_t b = Prep2Cfg<bf16_t, DK>::bytes;
+  hipLaunchKernelGGL(k, dim3((unsigned)((int64_t)p.geom.rows * p.geom.N)), dim3(256), b, st, p);
+}
+
+int launch_direct_fwd(const lnx_scan_args* a, const FwdParams& p, int nstate, hipStream_t st) {
+  if (a->dk == 128) {
+    if (a->gate == LNX_GATE_SCALAR) launch_prepare_lite<128, LNX_GATE_SCALAR>(p, st);
+    else launch_prepare_lite<128, LNX_GATE_NONE>(p, st);
+  } else {
+    if (a->gate == LNX_GATE_SCALAR) launch_prepare_lite<64, LNX_GATE_SCALAR>(p, st);
+    else launch_prepare_lite<64, LNX_GATE_NONE>(p, st);
+  }
+  DirectParams d = {};
+  d.geom = p.geom;
+  d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
+  d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.s0 = a->initial_state; d.sT_out = a->final_state;
+  d.o = a->o; d.dv = a->dv; d.o_dtype = a->o_dtype; d.save = !a->forward_only; d.vcols = p.vcols; d.gate = a->gate;
+  d.scale = a->scale; d.ws = p.ws; d.off = p.off;
+  int rc = lnx_direct_scan_fwd(d, a->dk, a->gate, nstate, st);
+  if (rc != LNX_OK) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk forward launch: %s", hipGetErrorString(e));
+  return LNX_OK;
+}
+
 // The forward pass on a caller-chosen workspace (a->workspace is not looked at).
 int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_bytes, hipStream_t st) {
   const bool packed = a->cu_seqlens != nullptr;
@@ -1129,6 +1170,7 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
   p.vcols = a->value_cols ? a->value_cols : a->dv;
   p.ws = ws; p.off = w;
   int rc;
+  if (lnx_chunk_direct(a)) return launch_direct_fwd(a, p, nstate, st);
   if (a->dtype == LNX_BF16)
     rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
          : (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st)

@@ -43,6 +43,50 @@ template <> struct Mma<bf16_t> {
     const short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(Frag, v);
   }
+
+  // ---- chaining products through registers ----
+  // A 32x32 accumulator fragment can be the B operand of the next product without a trip through LDS when the
+  // contraction runs over the fragment's rows: lane (n = lane & 31, kg = lane >> 5) holds, as elements 8 h .. 8 h + 7
+  // of the fragment (h = 0, 1), the rows  16 h + 4 kg + (0..3)  and  16 h + 8 + 4 kg + (0..3)  of column n.  The MFMA
+  // only needs both operands to agree on which contraction index sits in which slot, so the A operand is loaded in
+  // that same order ("chain order") with two 8-byte reads instead of one 16-byte read.
+  static __device__ __forceinline__ Frag from_acc(const floatx16& c, int h) {
+    Frag b;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) b[t] = (bf16_t)c[8 * h + t];
+    return b;
+  }
+  // A operand in chain order from a [rows][k] tile: p points at (this lane's row, first k of the 16-wide step)
+  static __device__ __forceinline__ Frag load_chain(const bf16_t* p, int lane) {
+    const bf16_t* q = p + 4 * (lane >> 5);
+    const bf16x4 lo = *reinterpret_cast<const bf16x4*>(q), hi = *reinterpret_cast<const bf16x4*>(q + 8);
+    Frag v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return v;
+  }
+  // A operand in chain order from a row-major [k][rows] tile (contraction along the tile's rows), like load_t
+  static __device__ __forceinline__ Frag load_t_chain(const bf16_t* tile, int ld, int k0, int c0, int lane) {
+    typedef short short4_ __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) short4_ lds_short4;
+    const int s = lane & 15, grp = lane >> 4;
+    const bf16_t* p = tile + (k0 + 4 * (grp >> 1) + (s >> 2)) * ld + c0 + 16 * (grp & 1) + 4 * (s & 3);
+    const short4_ lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p));
+    const short4_ hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p + 8 * ld));
+    typedef short short8_ __attribute__((ext_vector_type(8)));
+    const short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(Frag, v);
+  }
+  // Four consecutive rows of this lane's column of a row-major tile, i.e. elements 4 q .. 4 q + 3 of an accumulator
+  // fragment's position: tile[r0 + 8 q + 4 (lane >> 5) + (0..3)][c0 + (lane & 31)], one transposing read.
+  static __device__ __forceinline__ floatx4 load_acc_rows(const bf16_t* tile, int ld, int r0, int q, int c0, int lane) {
+    typedef short short4_ __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) short4_ lds_short4;
+    const int s = lane & 15, grp = lane >> 4;
+    const bf16_t* p = tile + (r0 + 8 * q + 4 * (grp >> 1) + (s >> 2)) * ld + c0 + 16 * (grp & 1) + 4 * (s & 3);
+    const short4_ x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p));
+    const bf16x4 y = __builtin_bit_cast(bf16x4, x);
+    floatx4 r = {(float)y[0], (float)y[1], (float)y[2], (float)y[3]};
+    return r;
+  }
 };
 
 template <> struct Mma<float> {
