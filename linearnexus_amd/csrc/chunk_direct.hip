@@ -103,16 +103,24 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
   if (wave >= NCW) {
     // ---------------- movers ----------------
     const int mt = tid - 64 * NCW;
+    typedef TileRegs<T, 64, DK> RowTile;
+    typedef TileRegs<T, 64, BV> ValTile;
     struct Tiles {
-      TileRegs<T, 64, DK> K, Q;
-      TileRegs<T, 64, BV> V;
+      RowTile K, Q;
+      ValTile V;
       TileRegs<T, 64, 64> Tm, P;
       float g, gc, b;
+      float gq[RowTile::IT];  // G of the token each of this thread's Q vectors belongs to
+      float bv[ValTile::IT];  // beta of the token each of its V vectors belongs to
       int len;
     };
     Tiles ta, tb;
     ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
     ta.len = tb.len = 0;
+#pragma unroll
+    for (int it = 0; it < RowTile::IT; ++it) ta.gq[it] = tb.gq[it] = 0.f;
+#pragma unroll
+    for (int it = 0; it < ValTile::IT; ++it) ta.bv[it] = tb.bv[it] = 0.f;
     auto fetch = [&](Tiles& R, int n) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0;
@@ -126,24 +134,49 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       // every thread loads the scalars of token mt % 64 (no load behind a branch); tokens past the end are masked below
       const int t = mt & 63;
       if (GATE == LNX_GATE_SCALAR) {
-        R.g = at<const float>(p.ws, p.off.G)[slot * 64 + t];
-        R.gc = at<const float>(p.ws, p.off.G)[slot * 64 + 63];
+        const float* G = at<const float>(p.ws, p.off.G) + slot * 64;
+        R.g = G[t];
+        R.gc = G[63];
+#pragma unroll
+        for (int it = 0; it < RowTile::IT; ++it) R.gq[it] = G[(mt + 256 * it) / RowTile::VPR];
       }
       R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
+#pragma unroll
+      for (int it = 0; it < ValTile::IT; ++it)
+        R.bv[it] = p.beta[tbase + (int64_t)min(min((mt + 256 * it) / ValTile::VPR, 63), R.len - 1) * p.geom.ts];
     };
     auto commit = [&](const Tiles& R, int pb) {
       R.K.store(sK + pb * L::kK, LDK, mt);
-      R.Q.store(sQ + pb * L::kK, LDK, mt);
-      R.V.store(sV + pb * L::kV, LDV, mt);
+      {  // Q rows scaled by scale e^{G_i}: the outputs then need no scaling of their own
+        T* dst = sQ + pb * L::kK;
+#pragma unroll
+        for (int it = 0; it < RowTile::IT; ++it) {
+          const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
+          const float f = (GATE == LNX_GATE_SCALAR) ? p.scale * __expf(R.gq[it]) : p.scale;
+          typename Vec16<T>::V x = R.Q.x[it];
+#pragma unroll
+          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f);
+          *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+        }
+      }
+      {  // V rows scaled by beta_i: R = beta V - (beta e^G) Y
+        T* dst = sV + pb * L::kV;
+#pragma unroll
+        for (int it = 0; it < ValTile::IT; ++it) {
+          const int idx = mt + 256 * it, r = idx / ValTile::VPR, c = (idx - r * ValTile::VPR) * ValTile::N;
+          typename Vec16<T>::V x = R.V.x[it];
+#pragma unroll
+          for (int e = 0; e < ValTile::N; ++e) x[e] = (bf16_t)((float)x[e] * R.bv[it]);
+          if (idx < ValTile::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDV + c) = x;
+        }
+      }
       R.Tm.store(sTm + pb * L::kC, LDC, mt);
       R.P.store(sP + pb * L::kC, LDC, mt);
       if (mt < 64) {
         float* sc = sSc + pb * Scal::SIZE;
         const float gam = (GATE == LNX_GATE_SCALAR) ? __expf(R.g) : 1.f;
-        sc[Scal::BETA + mt] = (mt < R.len) ? R.b : 0.f;
-        sc[Scal::GAM + mt] = gam;
+        sc[Scal::GAM + mt] = (mt < R.len) ? R.b * gam : 0.f;  // beta e^G
         sc[Scal::R + mt] = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(R.gc - R.g, 0.f)) : 1.f;
-        sc[Scal::SG + mt] = p.scale * gam;
         if (mt == 0) sc[Scal::DEC] = (GATE == LNX_GATE_SCALAR) ? __expf(R.gc) : 1.f;
       }
     };
@@ -201,6 +234,10 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       for (int e = 0; e < 16; ++e) S[ci][e] = s0[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv + frag_col(lane)];
   }
   lds_barrier();  // B1 of the first chunk
+  // Every LDS read is issued well ahead of the product that consumes it (A fragments two steps ahead, the next
+  // phase's first fragments and scalars during the current phase's last steps): a wave alone on its SIMD has nothing
+  // else to cover the LDS latency with.  The scheduling fences pin that order.
+  constexpr int NK = DK / 16;  // 16-wide steps over dk
   for (int n = c0; n < c1; ++n) {
     const int pb = (n - c0) & 1;
     const T* sKc = sK + pb * L::kK;
@@ -213,51 +250,64 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
 #pragma unroll
       for (int ci = 0; ci < KT; ++ci) store_frag_t(S[ci], sST + vs * LDK + 32 * ci, LDK, lane);
     }
-    // ---- Y = K S and Q S: the state fragments are the B operands ----
+    // ---- Y = K S (lane = value column) and (Q~ S)^T (lane = token): the state fragments are the shared operand ----
     floatx16 y[2], o[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) y[i][e] = o[i][e] = 0.f;
-    {
-      // A fragments one step ahead of the products; the scheduling fences keep the compiler from hoisting every read
-      // of the unrolled loop to its top (and spilling the state for it)
-      M::Frag fk[2][2], fq[2][2];  // [step parity][row tile]: the unrolled loop names them statically
+    M::Frag fa[3][2], fb[3][2];  // [step mod 3][row tile]
+    bf16x4 vr[2][4];             // beta V at this lane's accumulator positions
+    floatx4 sv[2][4];            // per-row scalars at this lane's accumulator positions: beta e^G, later e^{G_C - G}
+#pragma unroll
+    for (int s_ = 0; s_ < 2; ++s_)
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        fk[0][i] = M::load_chain(sKc + (32 * i + fr) * LDK, lane);
-        fq[0][i] = M::load_chain(sQc + (32 * i + fr) * LDK, lane);
+        fa[s_][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * s_, lane);
+        fb[s_][i] = M::load_chain(sQc + (32 * i + fr) * LDK + 16 * s_, lane);
       }
 #pragma unroll
-      for (int ks = 0; ks < DK / 16; ++ks) {
-        if (ks + 1 < DK / 16) {
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            fk[(ks + 1) & 1][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * (ks + 1), lane);
-            fq[(ks + 1) & 1][i] = M::load_chain(sQc + (32 * i + fr) * LDK + 16 * (ks + 1), lane);
-          }
-        }
-        const M::Frag b = M::from_acc(S[ks >> 1], ks & 1);
+    for (int ks = 0; ks < NK; ++ks) {
+      if (ks + 2 < NK) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-          M::mma(y[i], fk[ks & 1][i], b);
-          M::mma(o[i], fq[ks & 1][i], b);
+          fa[(ks + 2) % 3][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * (ks + 2), lane);
+          fb[(ks + 2) % 3][i] = M::load_chain(sQc + (32 * i + fr) * LDK + 16 * (ks + 2), lane);
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
+      if (ks == NK - 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            vr[i][q] = M::load_acc_rows_raw(sVc, LDV, 32 * i, q, vs, lane);
+            sv[i][q] = load4(sc + Scal::GAM + 32 * i + 8 * q + 4 * (lane >> 5));
+          }
+      }
+      const M::Frag b = M::from_acc(S[ks >> 1], ks & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        M::mma(y[i], fa[ks % 3][i], b);
+        M::mma(o[i], b, fb[ks % 3][i]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
+    // first A fragments of D = Tm R
+#pragma unroll
+    for (int s_ = 0; s_ < 2; ++s_)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_chain(sTc + (32 * i + fr) * LDC + 16 * s_, lane);
     __builtin_amdgcn_sched_barrier(0);
-    // ---- R = beta (V - e^G Y), in place of Y ----
+    // ---- R = beta V - (beta e^G) Y, in place of Y ----
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const floatx4 vv = M::load_acc_rows(sVc, LDV, 32 * i, q, vs, lane);
-        const int t0 = 32 * i + 8 * q + 4 * (lane >> 5);
-        const floatx4 bt = load4(sc + Scal::BETA + t0), gm = load4(sc + Scal::GAM + t0);
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) y[i][4 * q + u] = bt[u] * (vv[u] - gm[u] * y[i][4 * q + u]);
-      }
+        for (int u = 0; u < 4; ++u) y[i][4 * q + u] = (float)vr[i][q][u] - sv[i][q][u] * y[i][4 * q + u];
+    M::Frag br[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(y[ks >> 1], ks & 1);
     __builtin_amdgcn_sched_barrier(0);
     // ---- D = Tm R ----
     floatx16 d[2];
@@ -267,56 +317,77 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       for (int e = 0; e < 16; ++e) d[i][e] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::from_acc(y[ks >> 1], ks & 1);
+      if (ks + 2 < 4) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(d[i], M::load_chain(sTc + (32 * i + fr) * LDC + 16 * ks, lane), b);
+        for (int i = 0; i < 2; ++i) fa[(ks + 2) % 3][i] = M::load_chain(sTc + (32 * i + fr) * LDC + 16 * (ks + 2), lane);
+      } else {  // first fragments of Pm for the outputs
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fb[ks - 2][i] = M::load_chain(sPc + (32 * i + fr) * LDC + 16 * (ks - 2), lane);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(d[i], fa[ks % 3][i], br[ks]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (GATE == LNX_GATE_SCALAR) {  // e^{G_C - G} for the state update
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sv[i][q] = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
     }
     if (p.save) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) store_frag_t(d[i], sDT + vs * LDC + 32 * i, LDC, lane);
     }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(d[ks >> 1], ks & 1);
     __builtin_amdgcn_sched_barrier(0);
-    // ---- O = scale e^G (Q S) + Pm D ----
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const floatx4 sg = load4(sc + Scal::SG + 32 * i + 8 * q + 4 * (lane >> 5));
-#pragma unroll
-        for (int u = 0; u < 4; ++u) o[i][4 * q + u] *= sg[u];
-      }
+    // ---- O^T = (Q~ S)^T + D^T Pm^T ----
+    M::Frag fu[2][KT];  // K^T fragments of the state update, [step parity][row tile of the state]
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::from_acc(d[ks >> 1], ks & 1);
+      if (ks + 2 < 4) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(o[i], M::load_chain(sPc + (32 * i + fr) * LDC + 16 * ks, lane), b);
+        for (int i = 0; i < 2; ++i) fb[(ks + 2) % 3][i] = M::load_chain(sPc + (32 * i + fr) * LDC + 16 * (ks + 2), lane);
+      } else if (ks == 2) {
+#pragma unroll
+        for (int ci = 0; ci < KT; ++ci) fu[0][ci] = M::load_t_chain(sKc, LDK, 0, 32 * ci, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(o[i], br[ks], fb[ks % 3][i]);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    // the state update's operand while the last products finish: D rows scaled by e^{G_C - G}
+    if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) sO[(32 * i + frag_row(e, lane)) * LDV + vs + frag_col(lane)] = (bf16_t)o[i][e];
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) d[i][4 * q + u] *= sv[i][q][u];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(d[ks >> 1], ks & 1);
+    }
+    const float dec = (GATE == LNX_GATE_SCALAR) ? sc[Scal::DEC] : 1.f;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) store_frag_t(o[i], sO + 32 * i * LDV + vs, LDV, lane);  // [token][value column]
     lds_barrier();  // Bmid
     // ---- S <- e^{G_C} S + K^T (e^{G_C - G} D) ----
     if (GATE == LNX_GATE_SCALAR) {
-      const float dec = sc[Scal::DEC];
 #pragma unroll
       for (int ci = 0; ci < KT; ++ci)
 #pragma unroll
         for (int e = 0; e < 16; ++e) S[ci][e] *= dec;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const floatx4 rr = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
-#pragma unroll
-          for (int u = 0; u < 4; ++u) d[i][4 * q + u] *= rr[u];
-        }
     }
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::from_acc(d[ks >> 1], ks & 1);
+      if (ks + 1 < 4) {
 #pragma unroll
-      for (int ci = 0; ci < KT; ++ci) M::mma(S[ci], M::load_t_chain(sKc, LDK, 16 * ks, 32 * ci, lane), b);
+        for (int ci = 0; ci < KT; ++ci) fu[(ks + 1) & 1][ci] = M::load_t_chain(sKc, LDK, 16 * (ks + 1), 32 * ci, lane);
+      }
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(S[ci], fu[ks & 1][ci], br[ks]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();  // B1 of the next chunk
   }
@@ -501,6 +572,9 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       for (int e = 0; e < 16; ++e) dS[ci][e] = src[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv + frag_col(lane)];
   }
   lds_barrier();  // B1 of the first chunk
+  // LDS reads are issued ahead of the products that consume them, as in scan_fwd.  The products that do not depend on
+  // the incoming dS' (Pm^T dO, Q~^T dO) fill the gaps of the chain  dS' -> Z -> dD -> dR -> dY -> dS.
+  constexpr int NK = DK / 16;
   for (int n = c1 - 1; n >= c0; --n) {
     const int pb = (c1 - 1 - n) & 1;
     const T* sKc = sK + pb * L::kK;
@@ -509,81 +583,152 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
     const T* sTc = sTm + pb * L::kC;
     const T* sPc = sP + pb * L::kC;
     const float* sc = sSc + pb * Scal::SIZE;
+    M::Frag fa[3][2], fp[2][2], fo[2];
+    floatx4 sv[2][4];  // per-row scalars at this lane's accumulator positions: e^{G_C - G}, later beta e^G
+#pragma unroll
+    for (int s_ = 0; s_ < 2; ++s_)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * s_, lane);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fp[0][i] = M::load_t(sPc, LDC, 0, 32 * i, lane);
+    fo[0] = M::load_t(sOc, LDV, 0, vs, lane);
+    // the state gradient as the B operand of Z = K dS'; its accumulators are then free to take the next dS
+    M::Frag bs[NK];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) bs[ks] = M::from_acc(dS[ks >> 1], ks & 1);
 #pragma unroll
     for (int ci = 0; ci < KT; ++ci) store_frag_t(dS[ci], sdST + vs * LDK + 32 * ci, LDK, lane);
-    // ---- Z = K dS' (the state-gradient fragments are the B operands) and the chunk-local part Pm^T dO ----
+    const float dec = (GATE == LNX_GATE_SCALAR) ? sc[Scal::DEC] : 1.f;
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- Z = K dS' and the chunk-local part Pm^T dO ----
     floatx16 z[2], dd[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) z[i][e] = dd[i][e] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < DK / 16; ++ks) {
-      const M::Frag b = M::from_acc(dS[ks >> 1], ks & 1);
+    for (int ks = 0; ks < NK; ++ks) {
+      if (ks + 2 < NK) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(z[i], M::load_chain(sKc + (32 * i + fr) * LDK + 16 * ks, lane), b);
-    }
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::load_t(sOc, LDV, 16 * ks, vs, lane);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(dd[i], M::load_t(sPc, LDC, 16 * ks, 32 * i, lane), b);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- dD = Pm^T dO + e^{G_C - G} Z ----
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const floatx4 rr = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
-#pragma unroll
-        for (int u = 0; u < 4; ++u) dd[i][4 * q + u] += rr[u] * z[i][4 * q + u];
+        for (int i = 0; i < 2; ++i) fa[(ks + 2) % 3][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * (ks + 2), lane);
       }
-    // ---- dR = Tm^T dD, dY = -beta e^G dR (in z) ----
+      if (ks + 1 < 4) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) z[i][e] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::from_acc(dd[ks >> 1], ks & 1);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(z[i], M::load_t_chain(sTc, LDC, 16 * ks, 32 * i, lane), b);
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      store_frag_t(z[i], sdRT + vs * LDC + 32 * i, LDC, lane);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int t0 = 32 * i + 8 * q + 4 * (lane >> 5);
-        const floatx4 bt = load4(sc + Scal::BETA + t0), bg = load4(sc + Scal::GAM + t0);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          sdV[(t0 + u) * LDV + vs + fr] = (bf16_t)(bt[u] * z[i][4 * q + u]);
-          z[i][4 * q + u] *= -bg[u];
-        }
+        for (int i = 0; i < 2; ++i) fp[(ks + 1) & 1][i] = M::load_t(sPc, LDC, 16 * (ks + 1), 32 * i, lane);
+        fo[(ks + 1) & 1] = M::load_t(sOc, LDV, 16 * (ks + 1), vs, lane);
       }
+      if (ks == NK - 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sv[i][q] = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(z[i], fa[ks % 3][i], bs[ks]);
+      if (ks < 4) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) M::mma(dd[i], fp[ks & 1][i], fo[ks & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    lds_barrier();  // Bmid
-    // ---- dS <- e^{G_C} dS' + (scale e^G Q)^T dO + K^T dY ----
+    // first fragments of Tm^T, and of the (scale e^G Q)^T dO product that fills the wait for Z
+    M::Frag fq[2][KT];
+#pragma unroll
+    for (int s_ = 0; s_ < 2; ++s_)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_t_chain(sTc, LDC, 16 * s_, 32 * i, lane);
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci) fq[0][ci] = M::load_t(sQc, LDK, 0, 32 * ci, lane);
+    fo[0] = M::load_t(sOc, LDV, 0, vs, lane);
     if (GATE == LNX_GATE_SCALAR) {
-      const float dec = sc[Scal::DEC];
 #pragma unroll
       for (int ci = 0; ci < KT; ++ci)
 #pragma unroll
         for (int e = 0; e < 16; ++e) dS[ci][e] *= dec;
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- dS <- e^{G_C} dS' + (scale e^G Q)^T dO ----
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::load_t(sOc, LDV, 16 * ks, vs, lane);
+      if (ks + 1 < 4) {
 #pragma unroll
-      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], M::load_t(sQc, LDK, 16 * ks, 32 * ci, lane), b);
+        for (int ci = 0; ci < KT; ++ci) fq[(ks + 1) & 1][ci] = M::load_t(sQc, LDK, 16 * (ks + 1), 32 * ci, lane);
+        fo[(ks + 1) & 1] = M::load_t(sOc, LDV, 16 * (ks + 1), vs, lane);
+      }
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], fq[ks & 1][ci], fo[ks & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- dD = Pm^T dO + e^{G_C - G} Z ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) dd[i][4 * q + u] += sv[i][q][u] * z[i][4 * q + u];
+    M::Frag bd[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) bd[ks] = M::from_acc(dd[ks >> 1], ks & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- dR = Tm^T dD (lane = value column, in z) and once more with the operands exchanged (lane = token, in dd), which
+    //      is the orientation dv = beta dR leaves in ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) z[i][e] = dd[i][e] = 0.f;
+    M::Frag fu[2][KT];  // K^T fragments of the dS update
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks + 2 < 4) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fa[(ks + 2) % 3][i] = M::load_t_chain(sTc, LDC, 16 * (ks + 2), 32 * i, lane);
+      } else if (ks == 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sv[i][q] = load4(sc + Scal::GAM + 32 * i + 8 * q + 4 * (lane >> 5));
+      } else {
+#pragma unroll
+        for (int ci = 0; ci < KT; ++ci) fu[0][ci] = M::load_t_chain(sKc, LDK, 0, 32 * ci, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(z[i], fa[ks % 3][i], bd[ks]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) M::mma(dd[i], bd[ks], fa[ks % 3][i]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const float bl0 = sc[Scal::BETA + fr], bl1 = sc[Scal::BETA + 32 + fr];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) store_frag_t(z[i], sdRT + vs * LDC + 32 * i, LDC, lane);
+    // dY = -beta e^G dR
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) z[i][4 * q + u] *= -sv[i][q][u];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) bd[ks] = M::from_acc(z[ks >> 1], ks & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // dv = beta dR: fragment dd[i] holds tokens 32 i .. (one per lane) x the strip's value columns
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      dd[0][e] *= bl0;
+      dd[1][e] *= bl1;
     }
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const M::Frag b = M::from_acc(z[ks >> 1], ks & 1);
+    for (int i = 0; i < 2; ++i) store_frag_t(dd[i], sdV + 32 * i * LDV + vs, LDV, lane);
+    lds_barrier();  // Bmid
+    // ---- dS += K^T dY ----
 #pragma unroll
-      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], M::load_t_chain(sKc, LDK, 16 * ks, 32 * ci, lane), b);
+    for (int ks = 0; ks < 4; ++ks) {
+      if (ks + 1 < 4) {
+#pragma unroll
+        for (int ci = 0; ci < KT; ++ci) fu[(ks + 1) & 1][ci] = M::load_t_chain(sKc, LDK, 16 * (ks + 1), 32 * ci, lane);
+      }
+#pragma unroll
+      for (int ci = 0; ci < KT; ++ci) M::mma(dS[ci], fu[ks & 1][ci], bd[ks]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();  // B1 of the next chunk
   }
@@ -765,23 +910,24 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   lds_barrier();  // slab tiles are dead from here on
 
   // ---- epilogue ----
+  rK.store(sK, LDKT, tid);
+  rQ.store(sQ, LDKT, tid);
   {
-    floatx16 pe[1][1], xa[1][1], xe[1][1];
+    floatx16 pe[1][1];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
       pe[0][0][e] = (i >= j) ? p.scale * dec * aP[0][0][e] : 0.f;
-      xa[0][0][e] = (i > j) ? -dec * aA[0][0][e] : 0.f;
-      xe[0][0][e] = sBeta[i] * xa[0][0][e];
+      aA[0][0][e] = (i > j) ? -dec * aA[0][0][e] : 0.f;  // dXa
     }
     frag_store<T, 1, 1>(pe, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
     frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
-    frag_store<T, 1, 1>(xa, sXa + 32 * wi * LDC + 32 * wj, LDC, lane);
-    frag_store_t<T, 1, 1>(xe, sXeT + 32 * wj * LDC + 32 * wi, LDC, lane);
+    frag_store<T, 1, 1>(aA, sXa + 32 * wi * LDC + 32 * wj, LDC, lane);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) aA[0][0][e] *= sBeta[32 * wi + frag_row(e, lane)];  // dXe
+    frag_store_t<T, 1, 1>(aA, sXeT + 32 * wj * LDC + 32 * wi, LDC, lane);
   }
-  rK.store(sK, LDKT, tid);
-  rQ.store(sQ, LDKT, tid);
   lds_barrier();
   const float gC = sG[63];
   // dq = scale e^G dQa + dPe K;   row = dXa K - e^G dK1 (in aK1)

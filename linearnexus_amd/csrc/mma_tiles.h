@@ -77,6 +77,13 @@ template <> struct Mma<bf16_t> {
   }
   // Four consecutive rows of this lane's column of a row-major tile, i.e. elements 4 q .. 4 q + 3 of an accumulator
   // fragment's position: tile[r0 + 8 q + 4 (lane >> 5) + (0..3)][c0 + (lane & 31)], one transposing read.
+  static __device__ __forceinline__ bf16x4 load_acc_rows_raw(const bf16_t* tile, int ld, int r0, int q, int c0, int lane) {
+    typedef short short4_ __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) short4_ lds_short4;
+    const int s = lane & 15, grp = lane >> 4;
+    const bf16_t* p = tile + (r0 + 8 * q + 4 * (grp >> 1) + (s >> 2)) * ld + c0 + 16 * (grp & 1) + 4 * (s & 3);
+    return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(p)));
+  }
   static __device__ __forceinline__ floatx4 load_acc_rows(const bf16_t* tile, int ld, int r0, int q, int c0, int lane) {
     typedef short short4_ __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) short4_ lds_short4;
