@@ -2,8 +2,12 @@
  * Plain-C caller of liblinearnexus_hip.so: no Python, no torch -- device memory from hipMalloc,
  * the argument block filled by hand, results checked against closed forms of the delta rule
  * (beta = 0 and no gate: S_T = S0 and o_t = scale * S0^T q_t; test_deltanet.py:281-297 uses the
- * same special case).  Built by linearnexus_amd/build.py (hipcc, host code only) next to this
- * file; tests/test_c_abi_gpu.py runs it.  Exit status 0 = every check passed.
+ * same special case -- it exercises the boundary, not the arithmetic: the WY inverse and W, U, D are trivial there;
+ * then one key direction e repeated for every token with random beta in (0.1, 1): the state stays e u_t^T with
+ * u_t = (1 - beta_t) u_{t-1} + beta_t v_t, o_t = scale <q_t, e> u_t, and the chunk's triangular system is the dense
+ * all-ones lower triangle scaled by beta, so its inverse and every product of the chunk path carry weight).
+ * Built by linearnexus_amd/build.py (gcc) next to this file; tests/test_c_abi_gpu.py runs it.  Exit status 0 = every
+ * check passed.
  */
 #include <hip/hip_runtime_api.h>
 #include <math.h>
@@ -80,6 +84,62 @@ int main(void) {
     for (size_t i = 0; i < ns; ++i) { es = fmax(es, fabs((double)sT[i] - s0[i])); ms = fmax(ms, fabs((double)s0[i])); }
     printf("%s: o err %.3g, state err %.3g (relative to the maximum)\n", pass ? "lnx_recurrent_fwd" : "lnx_chunk_fwd", eo / mo, es / ms);
     worst = fmax(worst, fmax(eo / mo, es / ms));
+  }
+
+  /* one repeated key direction, beta in (0.1, 1), zero initial state */
+  {
+    float* e = malloc((size_t)B * H * D * 4);
+    for (int bh = 0; bh < B * H; ++bh) {
+      double n2 = 0;
+      for (int c = 0; c < D; ++c) { e[bh * D + c] = frand(&seed); n2 += (double)e[bh * D + c] * e[bh * D + c]; }
+      for (int c = 0; c < D; ++c) e[bh * D + c] = (float)(e[bh * D + c] / sqrt(n2));
+    }
+    float* sref = malloc(ns * 4);
+    for (int bh = 0; bh < B * H; ++bh) {
+      double u[D];
+      for (int c = 0; c < D; ++c) u[c] = 0;
+      double ee = 0;  /* <e, e> as the kernels see it (fp32 entries) */
+      for (int c = 0; c < D; ++c) ee += (double)e[bh * D + c] * e[bh * D + c];
+      for (int t = 0; t < T; ++t) {
+        const size_t row = ((size_t)bh * T + t) * D;
+        beta[(size_t)bh * T + t] = 0.55f + 0.45f * frand(&seed);
+        const double b = beta[(size_t)bh * T + t];
+        double qe = 0;
+        for (int c = 0; c < D; ++c) { k[row + c] = e[bh * D + c]; qe += (double)q[row + c] * e[bh * D + c]; }
+        for (int c = 0; c < D; ++c) u[c] = u[c] + b * (v[row + c] - ee * u[c]);
+        for (int c = 0; c < D; ++c) oref[row + c] = (float)(scale * qe * u[c]);
+      }
+      for (int r = 0; r < D; ++r)
+        for (int c = 0; c < D; ++c) sref[((size_t)bh * D + r) * D + c] = (float)(e[bh * D + r] * u[c]);
+    }
+    CHECK_HIP(hipMemcpy(dk, k, nq * 4, hipMemcpyHostToDevice));
+    CHECK_HIP(hipMemcpy(dbeta, beta, nb * 4, hipMemcpyHostToDevice));
+    a.initial_state = NULL;
+    for (int pass = 0; pass < 2; ++pass) {
+      CHECK_HIP(hipMemsetAsync(dO, 0xFF, nq * 4, st));
+      CHECK_HIP(hipMemsetAsync(dsT, 0xFF, ns * 4, st));
+      if (pass == 0) CHECK_LNX(lnx_chunk_fwd(&a, st));
+      else CHECK_LNX(lnx_recurrent_fwd(&a, st));
+      CHECK_HIP(hipStreamSynchronize(st));
+      CHECK_HIP(hipMemcpy(o, dO, nq * 4, hipMemcpyDeviceToHost));
+      CHECK_HIP(hipMemcpy(sT, dsT, ns * 4, hipMemcpyDeviceToHost));
+      double eo = 0, es = 0, mo = 0, ms = 0;
+      for (size_t i = 0; i < nq; ++i) { eo = fmax(eo, fabs((double)o[i] - oref[i])); mo = fmax(mo, fabs((double)oref[i])); }
+      for (size_t i = 0; i < ns; ++i) { es = fmax(es, fabs((double)sT[i] - sref[i])); ms = fmax(ms, fabs((double)sref[i])); }
+      printf("repeated key, %s: o err %.3g, state err %.3g (relative to the maximum)\n", pass ? "lnx_recurrent_fwd" : "lnx_chunk_fwd", eo / mo, es / ms);
+      worst = fmax(worst, fmax(eo / mo, es / ms));
+    }
+    a.initial_state = ds0;
+    /* the checks below are the beta = 0 case again */
+    memset(beta, 0, nb * 4);
+    CHECK_HIP(hipMemcpy(dbeta, beta, nb * 4, hipMemcpyHostToDevice));
+    for (int c = 0; c < D; ++c) {
+      double acc = 0;
+      for (int r = 0; r < D; ++r) acc += (double)s0[(size_t)r * D + c] * q[r];
+      oref[c] = (float)(scale * acc);
+    }
+    free(e);
+    free(sref);
   }
 
   /* decode step on the last token, state in place */

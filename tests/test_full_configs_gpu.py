@@ -9,6 +9,7 @@ import pytest
 import torch
 
 from oracle import recurrent as rc
+from oracle.adjoint import delta_rule_adjoint
 from oracle.inputs import make_cu_seqlens
 from conftest import max_rel
 
@@ -23,6 +24,62 @@ def _nrm(x):
 def _rel(a, b):
     a, b = a.detach(), b.detach()
     return float((a.double() - b.double()).abs().max() / b.double().abs().max())
+
+
+def _row_grads_against_oracle(grads, inputs, dO, b, h, t0, t1, s0_row, tol=2e-2):
+    """One (batch, head) row of a full-shape launch, tokens [t0, t1), against the token-level adjoint in fp64: every
+    gradient the backward pass returns, after the whole chain of carried state gradients."""
+    f = lambda t: t.detach()[b:b + 1, h:h + 1, t0:t1].float().cpu().numpy()
+    g = inputs.get("g")
+    ref = delta_rule_adjoint(f(inputs["q"]), f(inputs["k"]), f(inputs["v"]), f(inputs["beta"]), f(dO),
+                             None if g is None else f(g), None, None, s0_row, False)
+    for name in ("dq", "dk", "dv", "dbeta") + (("dg",) if g is not None else ()):
+        err = max_rel(f(grads[name]), ref[name])
+        assert err < tol, (name, err)
+    return ref
+
+
+def test_config2_gradients_of_one_full_row():
+    """Gated DeltaNet chunk fwd+bwd at B8 H16 T4096 d128 bf16: dq, dk, dv, dbeta, dg and dS0 of one (batch, head) row of
+    the full launch against the fp64 token-level adjoint over all 4096 tokens (64 chunks of carried dS)."""
+    import linearnexus_amd as la
+    torch.manual_seed(2)
+    B, H, T, d = 8, 16, 4096, 128
+    q = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    k = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    v = torch.randn(B, H, T, d, device=DEV).bfloat16().requires_grad_(True)
+    beta = torch.sigmoid(torch.randn(B, H, T, device=DEV)).requires_grad_(True)
+    g = (-torch.nn.functional.softplus(torch.randn(B, H, T, device=DEV)) * 0.1).requires_grad_(True)
+    S0 = torch.zeros(B, H, d, d, device=DEV, requires_grad=True)
+    dO = torch.randn(B, H, T, d, device=DEV).bfloat16()
+    o, _ = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, S0, 64, False)
+    o.backward(dO)
+    grads = dict(dq=q.grad, dk=k.grad, dv=v.grad, dbeta=beta.grad, dg=g.grad)
+    for b, h in ((5, 11), (0, 0)):
+        ref = _row_grads_against_oracle(grads, dict(q=q, k=k, v=v, beta=beta, g=g), dO, b, h, 0, T,
+                                        np.zeros((1, 1, d, d)))
+        assert max_rel(S0.grad[b:b + 1, h:h + 1].cpu().numpy(), ref["dS0"]) < 2e-2
+
+
+def test_config3_kda_gradients_of_one_full_row():
+    """KDA chunk fwd+bwd at B4 H16 T8192 d128 bf16 with a random S0: all gradients of one row over all 8192 tokens."""
+    import linearnexus_amd as la
+    torch.manual_seed(33)
+    B, H, T, d = 4, 16, 8192, 128
+    q = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    k = _nrm(torch.randn(B, H, T, d, device=DEV)).bfloat16().requires_grad_(True)
+    v = torch.randn(B, H, T, d, device=DEV).bfloat16().requires_grad_(True)
+    beta = torch.sigmoid(torch.randn(B, H, T, device=DEV)).requires_grad_(True)
+    g = (-torch.nn.functional.softplus(torch.randn(B, H, T, d, device=DEV)) * 0.05).requires_grad_(True)
+    S0 = (torch.randn(B, H, d, d, device=DEV) * 0.02).requires_grad_(True)
+    dO = torch.randn(B, H, T, d, device=DEV)
+    o, _ = la.kda_chunkwise(q, k, v, g, beta, None, S0, 64, False)
+    o.backward(dO)
+    grads = dict(dq=q.grad, dk=k.grad, dv=v.grad, dbeta=beta.grad, dg=g.grad)
+    b, h = 2, 9
+    ref = _row_grads_against_oracle(grads, dict(q=q, k=k, v=v, beta=beta, g=g), dO, b, h, 0, T,
+                                    S0.detach()[b:b + 1, h:h + 1].cpu().numpy())
+    assert max_rel(S0.grad[b:b + 1, h:h + 1].cpu().numpy(), ref["dS0"]) < 2e-2
 
 
 def test_config3_kda_full_shape():
@@ -84,7 +141,14 @@ def test_config5_deltanet_long_packed():
         for full, part in ((q.grad, qs.grad), (k.grad, ks.grad), (v.grad, vs.grad), (beta.grad, bs.grad)):
             assert _rel(full[:, :, a:b], part) < 1e-3
         assert _rel(S0.grad[s:s + 1], s0.grad) < 1e-3
-    # (c) oracle on the first 300 tokens of sequence 0, head 5
+    # (c) every gradient of one whole sequence of one head (its packed neighbours in place) against the fp64 adjoint
+    for s_, h in ((3, 17), (7, 0)):
+        a, b = int(cu[s_]), int(cu[s_ + 1])
+        grads = dict(dq=q.grad, dk=k.grad, dv=v.grad, dbeta=beta.grad)
+        ref = _row_grads_against_oracle(grads, dict(q=q, k=k, v=v, beta=beta), dO, 0, h, a, b,
+                                        S0.detach()[s_:s_ + 1, h:h + 1].cpu().numpy())
+        assert max_rel(S0.grad[s_:s_ + 1, h:h + 1].cpu().numpy(), ref["dS0"]) < 2e-2
+    # (d) oracle on the first 300 tokens of sequence 0, head 5
     a = int(cu[0])
     sl = lambda t: t.detach()[:, 5:6, a:a + 300].float().cpu().numpy()
     o_ref, _ = rc.delta_rule_recurrent(sl(q), sl(k), sl(v), sl(beta), S0.detach()[0:1, 5:6].cpu().numpy())
