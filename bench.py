@@ -137,6 +137,8 @@ def cpu_baseline_chunk(torch, B, H, T, d, seed):
 CHUNK_CONFIGS = {
     # name: (variant, B, H, T, d, packed sequences, random S0, backward)
     "gdn_chunk": ("gated", 8, 16, 4096, 128, 0, False, True),        # configuration 2 (headline)
+    # configuration 2 through the reference's default, use_qk_l2norm=True, on q and k that are not normalised
+    "gdn_chunk_l2norm": ("gated", 8, 16, 4096, 128, 0, False, True),
     "kda_chunk": ("kda", 4, 16, 8192, 128, 0, True, True),           # configuration 3
     "deltanet_varlen": ("delta", 1, 32, 32768, 128, 8, False, True),  # configuration 5
     "deltanet_fp32": ("delta32", 2, 4, 512, 64, 0, False, False),     # configuration 1 (forward only)
@@ -152,13 +154,16 @@ CHUNK_CONFIGS = {
 def bench_chunk(args, torch, la, _lib, name):
     variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
-    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
+    l2norm = name.endswith("_l2norm")
+    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "gdn_chunk_l2norm": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
             "gdn_chunk_fp32": 2, "gdn_dk256_fp32": 6, "kda_chunk_fp32": 3}[name]
     fp32 = variant.endswith("32")
     variant = variant[:-2] if fp32 else variant
     d, dv = d if isinstance(d, tuple) else (d, d)
     x = make_gdn_inputs(torch, B, H, T, d, seed, dev, dv)
     dt = torch.float32 if fp32 else torch.bfloat16
+    if l2norm:  # rows of length about sqrt(d), normalised inside the op
+        x["q"], x["k"] = x["q"] * d ** 0.5, x["k"] * d ** 0.5
     q, k, v, dO = (x[n].to(dt) for n in ("q", "k", "v", "dO"))
     beta, g = x["beta"], x["g"]
     gen = torch.Generator(device="cpu").manual_seed(seed + 100)
@@ -178,7 +183,7 @@ def bench_chunk(args, torch, la, _lib, name):
 
     def forward():
         if variant == "gated":
-            return la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, s0, 64, False)
+            return la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, s0, 64, l2norm)
         if variant == "kda":
             return la.kda_chunkwise(q, k, v, g, beta, None, s0, 64, False)
         return la.delta_rule_chunkwise(q, k, v, beta, s0, cu_seqlens=cu)
@@ -240,7 +245,8 @@ def bench_chunk(args, torch, la, _lib, name):
         "dtype": "f32" if fp32 else "bf16", "data": "synthetic",
         "config": {"workload": name + ("_fwd_bwd" if backward else "_fwd"), "variant": variant, "B": B, "H": H, "T": T,
                    "dk": d, "dv": dv, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
-                   "use_qk_l2norm": False, "inputs": "q,k pre-normalised; fp32 beta/g"},
+                   "use_qk_l2norm": l2norm,
+                   "inputs": ("q,k rows of length sqrt(d), normalised inside the op" if l2norm else "q,k pre-normalised") + "; fp32 beta/g"},
         "tflops_algorithmic": total_fl / dtm / 1e12,
         "mfma_peak_frac": total_fl / dtm / 1e12 / peak,
         "kernel_ms": {n: round(t, 4) for n, t in avg.items()},

@@ -53,7 +53,9 @@ typedef struct lnx_scan_args {
   int32_t dtype;            /* lnx_dtype of q, k, v, dO, dq, dk, dv */
   int32_t o_dtype;          /* lnx_dtype of o */
   int32_t gate;             /* lnx_gate */
-  int32_t use_qk_l2norm;    /* normalise q, k rows as x / (|x|_2 + 1e-6) inside the op */
+  int32_t use_qk_l2norm;    /* normalise q, k rows as x / (|x|_2 + 1e-6) inside the op: always honoured by the decode step
+                               and the token-by-token scan; by the chunk entry points where lnx_chunk_fuses_l2norm
+                               says so (ABI version 6), d_q and d_k are then the gradients of the raw q and k */
   int32_t nseq;             /* number of packed sequences; 0 for a dense batch */
   float scale;              /* multiplies q (after normalisation) */
   int32_t forward_only;     /* lnx_chunk_fwd: no backward pass will follow, do not write the per-chunk tensors
@@ -122,6 +124,14 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);
+/*
+ * 1 when lnx_chunk_fwd / lnx_chunk_bwd apply the in-op normalisation of q and k themselves for these arguments
+ * (use_qk_l2norm = 1: gated_deltanet.py:273-275, kda.py:379-381 normalise inside the op, and it is their default):
+ * element types bf16, dk <= 128, no per-channel gate.  The rows are scaled where the kernels stage them and the
+ * backward pass carries d_q, d_k through the normalisation, so no normalised copies of q and k exist.  0: the chunk
+ * entry points refuse use_qk_l2norm for these arguments; normalise with lnx_l2norm_fwd first.
+ */
+int lnx_chunk_fuses_l2norm(const lnx_scan_args* a);
 
 /*
  * lnx_chunk_fwd for callers that cannot allocate device memory or bring a workspace (code under HIP graph

@@ -1215,6 +1215,7 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
     d.geom = p.geom;
     d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
     d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.dv = a->dv; d.vcols = a->dv; d.gate = a->gate;
+    d.l2norm = a->use_qk_l2norm;
     d.scale = a->scale; d.ws = p.ws; d.off = w;
     d.d_o = reinterpret_cast<const bf16_t*>(a->d_o); d.d_sT = a->d_final_state;
     d.dq = reinterpret_cast<bf16_t*>(a->d_q); d.dk = reinterpret_cast<bf16_t*>(a->d_k);

@@ -105,7 +105,7 @@ __device__ __forceinline__ bool xcd_slot_part(int64_t slots, int parts, int64_t&
 inline unsigned lnx_xcd_grid(int64_t slots, int parts) { return (unsigned)(((slots + 7) / 8) * 8 * parts); }
 
 struct ChunkWs {
-  uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, TmT, D, SnT, dD, dSn, dW, dG, total;
+  uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, Nq, Nk, Fq, TmT, D, SnT, dD, dSn, dW, dG, total;
 };
 
 // 2-byte inputs and outputs with dk <= 128 and no per-channel gate take the kernels of chunk_direct.hip, which keep G, Pm,
@@ -140,6 +140,9 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   if (lnx_chunk_direct(a)) {
     w.X = w.W = w.U = w.Kr = w.Qg = w.TmT = w.dW = w.dG = 0;
     w.G = take(slots * C * 4);
+    w.Nq = take(slots * C * 4);  // 1 / (|q_t| + eps), or 1 when the inputs come normalised
+    w.Nk = take(slots * C * 4);
+    w.Fq = take(slots * C * 4);  // scale e^{G_t} / (|q_t| + eps): what the scans multiply their Q rows with
     w.P = take(slots * C * C * es);
     w.Tm = take(slots * C * C * es);
     w.SnT = take(bwd ? slots * dv * dk * es : 0);   // states entering the chunks, [v][k]
@@ -149,7 +152,7 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
     w.total = off;
     return w;
   }
-  w.Tm = 0;
+  w.Tm = w.Nq = w.Nk = w.Fq = 0;
   w.G = take(vec ? slots * C * dk * 4 : slots * C * 4);
   w.P = take(slots * C * C * es);
   w.X = take(vec && saved ? slots * C * C * es : 0);
@@ -192,6 +195,7 @@ struct DirectParams {
   int save;   // forward scan: write the state entering every chunk (the backward pass reads it)
   int vcols;  // leading value columns present in v (its row length); the rest of the dv columns are zero
   int gate;
+  int l2norm;  // q and k rows are normalised inside the kernels (factors from the prepare kernel in Nq, Nk)
   float scale;
   char* ws;
   ChunkWs off;

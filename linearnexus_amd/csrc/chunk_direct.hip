@@ -110,7 +110,7 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       ValTile V;
       TileRegs<T, 64, 64> Tm, P;
       float g, gc, b;
-      float gq[RowTile::IT];  // G of the token each of this thread's Q vectors belongs to
+      float fq[RowTile::IT], nk[RowTile::IT];  // factors of the token each of this thread's Q / K vectors belongs to
       float bv[ValTile::IT];  // beta of the token each of its V vectors belongs to
       int len;
     };
@@ -118,7 +118,7 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
     ta.len = tb.len = 0;
 #pragma unroll
-    for (int it = 0; it < RowTile::IT; ++it) ta.gq[it] = tb.gq[it] = 0.f;
+    for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
 #pragma unroll
     for (int it = 0; it < ValTile::IT; ++it) ta.bv[it] = tb.bv[it] = 0.f;
     auto fetch = [&](Tiles& R, int n) {
@@ -137,8 +137,11 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
         const float* G = at<const float>(p.ws, p.off.G) + slot * 64;
         R.g = G[t];
         R.gc = G[63];
+      }
 #pragma unroll
-        for (int it = 0; it < RowTile::IT; ++it) R.gq[it] = G[(mt + 256 * it) / RowTile::VPR];
+      for (int it = 0; it < RowTile::IT; ++it) {
+        R.fq[it] = at<const float>(p.ws, p.off.Fq)[slot * 64 + (mt + 256 * it) / RowTile::VPR];
+        R.nk[it] = at<const float>(p.ws, p.off.Nk)[slot * 64 + (mt + 256 * it) / RowTile::VPR];
       }
       R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
 #pragma unroll
@@ -146,17 +149,18 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
         R.bv[it] = p.beta[tbase + (int64_t)min(min((mt + 256 * it) / ValTile::VPR, 63), R.len - 1) * p.geom.ts];
     };
     auto commit = [&](const Tiles& R, int pb) {
-      R.K.store(sK + pb * L::kK, LDK, mt);
-      {  // Q rows scaled by scale e^{G_i}: the outputs then need no scaling of their own
+      {  // K rows normalised; Q rows normalised and scaled by scale e^{G_i}: the outputs then need no scaling of their own
+        T* dstk = sK + pb * L::kK;
         T* dst = sQ + pb * L::kK;
 #pragma unroll
         for (int it = 0; it < RowTile::IT; ++it) {
           const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
-          const float f = (GATE == LNX_GATE_SCALAR) ? p.scale * __expf(R.gq[it]) : p.scale;
-          typename Vec16<T>::V x = R.Q.x[it];
+          const float f = R.fq[it];
+          typename Vec16<T>::V x = R.Q.x[it], y = R.K.x[it];
 #pragma unroll
-          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f);
+          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f), y[e] = (bf16_t)((float)y[e] * R.nk[it]);
           *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+          *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
         }
       }
       {  // V rows scaled by beta_i: R = beta V - (beta e^G) Y
@@ -469,14 +473,14 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       TileRegs<T, 64, BV> dO;
       TileRegs<T, 64, 64> Tm, P;
       float g, gc, b;
-      float gq[RowTile::IT];  // G of the token each of this thread's Q vectors belongs to
+      float fq[RowTile::IT], nk[RowTile::IT];  // factors of the token each of this thread's Q / K vectors belongs to
       int len;
     };
     Tiles ta, tb;
     ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
     ta.len = tb.len = 0;
 #pragma unroll
-    for (int it = 0; it < RowTile::IT; ++it) ta.gq[it] = tb.gq[it] = 0.f;
+    for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
     auto fetch = [&](Tiles& R, int n) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0;
@@ -492,23 +496,27 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
         const float* G = at<const float>(p.ws, p.off.G) + slot * 64;
         R.g = G[t];
         R.gc = G[63];
+      }
 #pragma unroll
-        for (int it = 0; it < RowTile::IT; ++it) R.gq[it] = G[(mt + 256 * it) / RowTile::VPR];
+      for (int it = 0; it < RowTile::IT; ++it) {
+        R.fq[it] = at<const float>(p.ws, p.off.Fq)[slot * 64 + (mt + 256 * it) / RowTile::VPR];
+        R.nk[it] = at<const float>(p.ws, p.off.Nk)[slot * 64 + (mt + 256 * it) / RowTile::VPR];
       }
       R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
     };
     auto commit = [&](const Tiles& R, int pb) {
-      R.K.store(sK + pb * L::kK, LDK, mt);
-      {  // Q rows scaled by scale e^{G_i}: (scale diag(e^G) Q)^T dO needs no scaled copy of dO then
+      {  // K rows normalised; Q rows normalised and scaled by scale e^{G_i}: (scale diag(e^G) Q)^T dO needs no scaled copy of dO
+        T* dstk = sK + pb * L::kK;
         T* dst = sQ + pb * L::kK;
 #pragma unroll
         for (int it = 0; it < RowTile::IT; ++it) {
           const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
-          const float f = (GATE == LNX_GATE_SCALAR) ? p.scale * __expf(R.gq[it]) : p.scale;
-          typename Vec16<T>::V x = R.Q.x[it];
+          const float f = R.fq[it];
+          typename Vec16<T>::V x = R.Q.x[it], y = R.K.x[it];
 #pragma unroll
-          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f);
+          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f), y[e] = (bf16_t)((float)y[e] * R.nk[it]);
           *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+          *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
         }
       }
       R.dO.store(sdO + pb * L::kV, LDV, mt);
@@ -781,7 +789,7 @@ template <int DK> struct BChunkL {
   static constexpr size_t loop_bytes = sizeof(T) * (2 * kTok + 2 * kT + 2 * kSt);
   static constexpr size_t epi_bytes = sizeof(T) * (2 * kRow + 4 * kC);
   static_assert(64 * LDK <= 2 * kC, "the staging tile overlays dPe and dPe^T");
-  static constexpr int nfloat = 64 * 6;
+  static constexpr int nfloat = 64 * 8;
   static constexpr size_t bytes = sizeof(float) * nfloat + (epi_bytes > loop_bytes ? epi_bytes : loop_bytes);
 };
 
@@ -797,6 +805,8 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   float* sM = sRdv + 64;      // m_t
   float* sdG = sM + 64;
   float* sMisc = sdG + 64;    // [0] = sum_t r_t <k_t, dK2_t>, [1] = <dS', S>
+  float* sNq = sMisc + 64;    // normalisation factors of the q and k rows (1 when the inputs come normalised)
+  float* sNk = sNq + 64;
   T* tiles = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
   // loop phase
   T* sdO = tiles;
@@ -851,6 +861,8 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
     sM[tid] = 0.f;
     sMisc[tid] = 0.f;
+    sNq[tid] = at<const float>(p.ws, p.off.Nq)[slot * 64 + tid];
+    sNk[tid] = at<const float>(p.ws, p.off.Nk)[slot * 64 + tid];
   }
 #pragma unroll 1
   for (int v0 = 0; v0 < p.dv; v0 += SV) {
@@ -910,8 +922,19 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   lds_barrier();  // slab tiles are dead from here on
 
   // ---- epilogue ----
-  rK.store(sK, LDKT, tid);
-  rQ.store(sQ, LDKT, tid);
+  {  // K and Q rows, normalised
+    typedef TileRegs<T, 64, DK> RowTile;
+#pragma unroll
+    for (int it = 0; it < RowTile::IT; ++it) {
+      const int idx = tid + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
+      const float fk = sNk[r], fq = sNq[r];
+      typename Vec16<T>::V x = rK.x[it], y = rQ.x[it];
+#pragma unroll
+      for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * fk), y[e] = (bf16_t)((float)y[e] * fq);
+      *reinterpret_cast<typename Vec16<T>::V*>(sK + r * LDKT + c) = x;
+      *reinterpret_cast<typename Vec16<T>::V*>(sQ + r * LDKT + c) = y;
+    }
+  }
   {
     floatx16 pe[1][1];
 #pragma unroll
@@ -987,32 +1010,42 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     }
   }
   lds_barrier();  // the four small tiles are dead; sM and sMisc are complete
+  // dq, then dk, through the staging tile.  Thread = (token tid / 4, the 8-column groups tid % 4, tid % 4 + 4, ...): the
+  // row dots <q_t, dq_t> and <k_t, dk_t> give the gate gradient and carry the gradients through the normalisation,
+  //   d/dx of x / (|x| + eps) applied to dy:  dy / (|x| + eps) - y <y, dy> / |x|.
+  const int tr = tid >> 2, tq = 8 * (tid & 3);
+  float dgp = 0.f;
+  auto emit = [&](const T* sIn, float fac, T* out, float sign) {
+    float dot = 0.f;
+#pragma unroll
+    for (int u = 0; u < DK; u += 32) {
+      const M::Frag a = M::load(sSt + tr * LDK + tq + u), b = M::load(sIn + tr * LDKT + tq + u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += (float)a[e] * (float)b[e];
+    }
+    dot = quad_sum(dot);
+    dgp += sign * dot;
+    const float nrm = 1.f / fac - LNX_L2_EPS;
+    const float cf = (p.l2norm && nrm > 0.f) ? dot / nrm : 0.f;
+    if (tr < len) {
+#pragma unroll
+      for (int u = 0; u < DK; u += 32) {
+        M::Frag a = M::load(sSt + tr * LDK + tq + u);
+        const M::Frag b = M::load(sIn + tr * LDKT + tq + u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] = (bf16_t)(fac * (float)a[e] - cf * (float)b[e]);
+        *reinterpret_cast<M::Frag*>(out + tbase * DK + (int64_t)tr * tsk + tq + u) = a;
+      }
+    }
+  };
   frag_store<T, 1, NKT>(aQ, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
   lds_barrier();
-  unstage_tile<T, 64, DK>(p.dq + tbase * DK, tsk, sSt, LDK, len, tid);
-  float dgp = 0.f;  // <q_t, dq_t> - <k_t, dk_t> over this thread's quarter of the key columns; thread = (token tid / 4, quarter)
-  const int tr = tid >> 2, tq = (tid & 3) * (DK / 4);
-  if (GATE == LNX_GATE_SCALAR) {
-#pragma unroll
-    for (int u = 0; u < DK / 4; u += 4) {
-      const floatx4 a = load4(sSt + tr * LDK + tq + u), b = load4(sQ + tr * LDKT + tq + u);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) dgp += a[e] * b[e];
-    }
-  }
+  emit(sQ, sNq[tr], p.dq, 1.f);
   lds_barrier();  // dq has left the staging tile
   frag_store<T, 1, NKT>(aK2, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
   lds_barrier();
-  unstage_tile<T, 64, DK>(p.dk + tbase * DK, tsk, sSt, LDK, len, tid);
+  emit(sK, sNk[tr], p.dk, -1.f);
   if (GATE == LNX_GATE_SCALAR) {
-#pragma unroll
-    for (int u = 0; u < DK / 4; u += 4) {
-      const floatx4 a = load4(sSt + tr * LDK + tq + u), b = load4(sK + tr * LDKT + tq + u);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) dgp -= a[e] * b[e];
-    }
-    dgp += __shfl_xor(dgp, 1, LNX_WAVE);
-    dgp += __shfl_xor(dgp, 2, LNX_WAVE);
     if ((tid & 3) == 0) {
       float d = dgp + 2.f * sBeta[tr] * sM[tr];
       if (tr == 63) d += sMisc[0] + __expf(gC) * sMisc[1];

@@ -37,6 +37,7 @@ struct FwdParams {
   int save;  // write the per-chunk tensors the backward pass (or the separate output kernel) reads
   int out_spw;  // chunk_output: value slabs per workgroup
   int vcols;    // leading value columns present in v (its row length); the rest of the dv columns are zero
+  int l2norm;   // chunk_prepare2<LITE>: q and k rows are normalised as x / (|x| + 1e-6) inside the kernels
   float scale;
   char* ws;
   ChunkWs off;
@@ -127,6 +128,7 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   floatx16 ax[1][1], ap[1][1];
   frag_zero(ax);
   frag_zero(ap);
+  float nk2 = 0.f, nq2 = 0.f;  // LITE: squared row norms, thread = (row tid / 4, 16 columns of the slab)
 #pragma unroll 1
   for (int s_ = 0; s_ < NKS; ++s_) {
     lds_barrier();
@@ -140,6 +142,33 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     if (!(wi == 0 && wj == 1)) {
       mma_nt<T, 1, 1>(ax, sKa + 32 * wi * LDC, LDC, sKa + 32 * wj * LDC, LDC, 64, lane);
       mma_nt<T, 1, 1>(ap, sQa + 32 * wi * LDC, LDC, sKa + 32 * wj * LDC, LDC, 64, lane);
+    }
+    if (LITE && p.l2norm) {
+      const int r = tid >> 2, c0 = (tid & 3) * 16;
+#pragma unroll
+      for (int u = 0; u < 16; u += 4) {
+        const floatx4 k4 = load4(sKa + r * LDC + c0 + u), q4 = load4(sQa + r * LDC + c0 + u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) nk2 += k4[e] * k4[e], nq2 += q4[e] * q4[e];
+      }
+    }
+  }
+  // LITE: per-row factors 1 / (|x| + eps) (1 without the normalisation), kept behind the slab tiles and written to the
+  // workspace for the scans and the chunk-local backward, which scale the rows as they stage them
+  float* sNk = reinterpret_cast<float*>(reg2 + 2 * L::kTile * sizeof(T));
+  float* sNq = sNk + 64;
+  static_assert(!LITE || 2 * L::kTile * sizeof(T) + 512 <= L::r2, "room for the row factors behind the slab tiles");
+  if constexpr (LITE) {
+    nk2 = quad_sum(nk2);
+    nq2 = quad_sum(nq2);
+    if ((tid & 3) == 0) {
+      const int r = tid >> 2;
+      const float fk = p.l2norm ? 1.f / (sqrtf(nk2) + LNX_L2_EPS) : 1.f, fq = p.l2norm ? 1.f / (sqrtf(nq2) + LNX_L2_EPS) : 1.f;
+      sNk[r] = fk;
+      sNq[r] = fq;
+      ws_ptr<float>(p, p.off.Nk)[slot * 64 + r] = fk;
+      ws_ptr<float>(p, p.off.Nq)[slot * 64 + r] = fq;
+      ws_ptr<float>(p, p.off.Fq)[slot * 64 + r] = p.scale * fq * ((GATE == LNX_GATE_SCALAR) ? __expf(sG[r]) : 1.f);
     }
   }
   // first slab of the second loop, in flight during the inverse
@@ -157,8 +186,9 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
     for (int e = 0; e < 16; ++e) {
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * ax[0][0][e] : 0.f;
-      pe[0][0][e] = (i >= j) ? p.scale * dec * ap[0][0][e] : 0.f;
+      const float fx = LITE ? sNk[i] * sNk[j] : 1.f, fp = LITE ? sNq[i] * sNk[j] : 1.f;
+      sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * fx * ax[0][0][e] : 0.f;
+      pe[0][0][e] = (i >= j) ? p.scale * dec * fp * ap[0][0][e] : 0.f;
     }
     frag_store<T, 1, 1>(pe, sKa + 32 * wi * LDC + 32 * wj, LDC, lane);
   }
@@ -1096,7 +1126,9 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (a->chunk != LNX_C) return lnx_set_error(LNX_ERR_SHAPE, "chunk length must be %d, got %d", LNX_C, a->chunk);
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
   if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);
-  if (a->use_qk_l2norm) return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels take pre-normalised q, k (use lnx_l2norm_fwd)");
+  if (a->use_qk_l2norm && !lnx_chunk_direct(a))
+    return lnx_set_error(LNX_ERR_SHAPE, "use_qk_l2norm inside the chunk kernels needs 2-byte inputs and outputs, dk <= 128 and no per-channel gate; "
+                                        "normalise with lnx_l2norm_fwd first");
   if (a->token_first != 0 && a->token_first != 1) return lnx_set_error(LNX_ERR_SHAPE, "token_first must be 0 or 1");
   if (backward && a->forward_only) return lnx_set_error(LNX_ERR_SHAPE, "forward_only is set: the workspace holds nothing for a backward pass");
   if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
@@ -1129,6 +1161,7 @@ int launch_direct_fwd(const lnx_scan_args* a, const FwdParams& p, int nstate, hi
   d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
   d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.s0 = a->initial_state; d.sT_out = a->final_state;
   d.o = a->o; d.dv = a->dv; d.o_dtype = a->o_dtype; d.save = !a->forward_only; d.vcols = p.vcols; d.gate = a->gate;
+  d.l2norm = a->use_qk_l2norm;
   d.scale = a->scale; d.ws = p.ws; d.off = p.off;
   int rc = lnx_direct_scan_fwd(d, a->dk, a->gate, nstate, st);
   if (rc != LNX_OK) return rc;
@@ -1168,6 +1201,7 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.out_spw = 1;
   p.vcols = a->value_cols ? a->value_cols : a->dv;
+  p.l2norm = a->use_qk_l2norm;
   p.ws = ws; p.off = w;
   int rc;
   if (lnx_chunk_direct(a)) return launch_direct_fwd(a, p, nstate, st);
@@ -1220,6 +1254,8 @@ extern "C" uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a) {
     return 0;
   return lnx_chunk_ws_layout(a).total;
 }
+
+extern "C" int lnx_chunk_fuses_l2norm(const lnx_scan_args* a) { return a && lnx_chunk_direct(a) ? 1 : 0; }
 
 extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   int rc = lnx_chunk_check(a, false);

@@ -393,10 +393,6 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
         raise RuntimeError(f"initial_state shape {tuple(initial_state.shape)} != {(nstate, H, dk, dv)}")
     tf = all(_is_token_first(t) for t in (q, k, v))  # [B,T,H,.] memory behind transposed views: used in place
     q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
-    # the reference's chunk path normalises in the input dtype before anything else
-    # (gated_deltanet.py:273-275, kda.py:379-381)
-    qn = _l2norm_rows_fwd(q_in) if l2norm else q_in
-    kn = _l2norm_rows_fwd(k_in) if l2norm else k_in
     v = _as_layout(v, tf)
     beta_f = _as_layout(beta.to(torch.float32), tf)
     g_f = None if g is None else _as_layout(g.to(torch.float32), tf)
@@ -404,6 +400,14 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
     o = _empty_layout(B, H, T, (dv,), o_dtype, q.device, tf) if want_o else None
     sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
     a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
+    lib = _lib.load()
+    # The reference's chunk path normalises in the input dtype before anything else (gated_deltanet.py:273-275,
+    # kda.py:379-381).  Where the kernels scale the rows themselves (no normalised copies, gradients carried through
+    # the normalisation inside lnx_chunk_bwd) they get the raw q and k; otherwise the rows are normalised first.
+    fused = bool(l2norm) and bool(lib.lnx_chunk_fuses_l2norm(a))
+    a.use_qk_l2norm = int(fused)
+    qn = _l2norm_rows_fwd(q_in) if l2norm and not fused else q_in
+    kn = _l2norm_rows_fwd(k_in) if l2norm and not fused else k_in
     a.nseq = nseq
     a.token_first = int(tf)
     a.forward_only = int(forward_only)
@@ -419,7 +423,7 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
     _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
     saved = (q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
     meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
-            None if g is None else g.dtype, initial_state is not None, tf)
+            None if g is None else g.dtype, initial_state is not None, tf, fused)
     return o, sT, saved, meta
 
 
@@ -438,7 +442,7 @@ class _ChunkScan(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_o, d_sT):
         q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws = ctx.saved_tensors
-        dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0, tf = ctx.meta
+        dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0, tf, fused = ctx.meta
         dev = qn.device
         d_o = torch.zeros(B, H, T, dv, dtype=qn.dtype, device=dev) if d_o is None else d_o.to(qn.dtype)
         d_o = _as_layout(d_o, tf)
@@ -448,7 +452,7 @@ class _ChunkScan(torch.autograd.Function):
         dg = None if g_f is None else torch.empty_like(g_f)
         nstate = nseq if nseq else B
         ds0 = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=dev) if has_s0 else None
-        a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, False, scale)
+        a = _base_args(B, H, T, dk, dv, dt, _DT[o_dtype], gate, fused, scale)
         a.nseq = nseq
         a.token_first = int(tf)
         a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
@@ -458,7 +462,7 @@ class _ChunkScan(torch.autograd.Function):
                                                                    _ptr(dg), _ptr(ds0))
         a.workspace, a.workspace_bytes = _ptr(ws), ws.numel()
         _lib.check(_lib.load().lnx_chunk_bwd(a, _stream(qn)), "lnx_chunk_bwd")
-        if l2norm:
+        if l2norm and not fused:
             dq = _l2norm_rows_bwd(q_in, dq)
             dk_ = _l2norm_rows_bwd(k_in, dk_)
         dbeta = dbeta.to(beta_dt)

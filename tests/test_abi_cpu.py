@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() == 5
+    assert lib.lnx_abi_version() == 6
 
 
 def test_struct_layout_matches_header():

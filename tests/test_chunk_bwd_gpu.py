@@ -93,6 +93,44 @@ def test_backward_through_l2norm(gate):
     check(got, ref, 1e-4)
 
 
+@pytest.mark.parametrize("shape", [(2, 2, 200, 128, 128), (1, 2, 130, 64, 128), (1, 3, 64, 128, 64)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_backward_through_l2norm_inside_the_chunk_kernels(shape, packed):
+    """bf16 inputs with no per-channel gate: the kernels scale the q and k rows themselves (no normalised copies) and
+    lnx_chunk_bwd returns the gradients of the raw rows (gated_deltanet.py:273-275 normalises inside the op).  Rows of
+    very different lengths."""
+    import linearnexus_amd as la
+    from linearnexus_amd import _lib
+    B, H, T, dk, dv = shape
+    if packed:
+        B = 1
+    x = make_inputs(57, B, H, T, dk, dv, gate="scalar", with_state=not packed, with_grad=True, normalize=False)
+    rng = np.random.default_rng(58)
+    x["q"] = x["q"] * np.exp(rng.standard_normal((B, H, T, 1))).astype(np.float32)
+    x["k"] = x["k"] * np.exp(rng.standard_normal((B, H, T, 1))).astype(np.float32)
+    x, dt = _prep(x, True)
+    a = _lib.ScanArgs(B=B, H=H, T=T, dk=dk, dv=dv, chunk=64, dtype=_lib.LNX_BF16, o_dtype=_lib.LNX_BF16, gate=_lib.GATE_SCALAR)
+    assert _lib.load().lnx_chunk_fuses_l2norm(a) == 1
+    if packed:
+        cu = np.array([0, 3, T // 2, T], np.int32)
+        x["S0"] = (rng.standard_normal((3, H, dk, dv)) * 0.02).astype(np.float32)
+        x["dS"] = (rng.standard_normal((3, H, dk, dv)) * 0.1).astype(np.float32)
+        parts = []
+        for s_ in range(3):
+            lo, hi = cu[s_], cu[s_ + 1]
+            sl = lambda n: x[n][:, :, lo:hi]
+            parts.append(delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), sl("g"), x["dS"][s_:s_ + 1], None,
+                                            x["S0"][s_:s_ + 1], True))
+        ref = {n: np.concatenate([p_[n] for p_ in parts], 2) for n in ("dq", "dk", "dv", "dbeta", "dg")}
+        ref["dS0"] = np.concatenate([p_["dS0"] for p_ in parts], 0)
+        got = gpu_grads(x, "scalar", dt, l2=True, cu=cu)
+    else:
+        ref = delta_rule_adjoint(x["q"], x["k"], x["v"], x["beta"], x["dO"], x["g"], x["dS"], None, x["S0"], True)
+        got = gpu_grads(x, "scalar", dt, l2=True)
+    assert all(np.isfinite(t).all() for t in got.values())
+    check(got, ref, 2e-2)
+
+
 @pytest.mark.parametrize("gate", GATES)
 def test_backward_packed_sequences(gate):
     H, T, d = 2, 300, 128

@@ -85,6 +85,21 @@ def test_l2norm_inside_op(gate):
     assert max_rel(o.float().cpu().numpy(), o_ref) < 2e-2 and max_rel(S.cpu().numpy(), S_ref) < 2e-2
 
 
+@pytest.mark.parametrize("dk", [64, 128])
+def test_l2norm_inside_the_chunk_kernels_zero_rows(dk):
+    """bf16, scalar gate: the kernels normalise the rows themselves; an all-zero q row and an all-zero k row normalise
+    to zero (x / (|x| + 1e-6)) and everything stays finite."""
+    x = make_inputs(45, 2, 2, 150, dk, 128, gate="scalar", normalize=False)
+    x["q"] = x["q"] * np.exp(np.random.default_rng(46).standard_normal((2, 2, 150, 1))).astype(np.float32)
+    x["q"][0, 0, 5] = 0.0
+    x["k"][1, 1, 70] = 0.0
+    x, dt = _prep(x, True)
+    o_ref, S_ref = oracle_fwd(x, "scalar", l2=True)
+    o, S = gpu_chunk_fwd(x, "scalar", dt, l2=True)
+    assert torch.isfinite(o).all() and torch.isfinite(S).all()
+    assert max_rel(o.float().cpu().numpy(), o_ref) < 2e-2 and max_rel(S.cpu().numpy(), S_ref) < 2e-2
+
+
 @pytest.mark.parametrize("gate", GATES)
 @pytest.mark.parametrize("bf16", [False, True])
 def test_packed_sequences(gate, bf16):
