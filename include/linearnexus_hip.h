@@ -221,6 +221,22 @@ int lnx_rmsnorm_gated_bwd(const void* x, const void* gate, const float* weight, 
                           uint64_t workspace_bytes, void* hip_stream);
 
 /*
+ * Gated DeltaNet's gate and learning-rate activations (the block computes them between its projections and the scan,
+ * gated_deltanet.py:804-815) and their gradient:
+ *   g[r, h] = -exp(A_log[h]) * softplus(a[r, h] + dt_bias[h])        beta[r, h] = beta_scale * sigmoid(b[r, h])
+ * a, b, d_a, d_b [rows, H] in `dtype` (b, beta, d_beta, d_b may be NULL together: gate only); g, beta and their
+ * gradients d_g, d_beta fp32 -- what lnx_chunk_fwd and lnx_decode_step read; A_log, dt_bias [H] fp32 (dt_bias may be
+ * NULL).  beta_scale = 2 for allow_neg_eigval (gated_deltanet.py:806-807), else 1.  d_A_log, d_dt_bias (may be NULL)
+ * are summed over the rows without atomics through a caller-owned workspace.
+ */
+int lnx_gdn_gate_fwd(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, float* beta,
+                     int64_t rows, int32_t H, float beta_scale, int32_t dtype, void* hip_stream);
+uint64_t lnx_gdn_gate_bwd_workspace_bytes(int64_t rows, int32_t H);
+int lnx_gdn_gate_bwd(const void* a, const void* b, const float* A_log, const float* dt_bias, const float* d_g,
+                     const float* d_beta, void* d_a, void* d_b, float* d_A_log, float* d_dt_bias, int64_t rows, int32_t H,
+                     float beta_scale, int32_t dtype, void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
+/*
  * KDA's gate activation (kda_gate, linearnexus/modules/linear_attn/kda.py:120-172) and its gradient:
  *   g_out[r, h, c] = -exp(A_log[h]) * softplus(g[r, h*dk + c] + g_bias[h*dk + c]),  softplus(x) = x for x > threshold
  * g, d_g [rows, H*dk] in `dtype`; g_out, d_out [rows, H, dk] in `out_dtype` (fp32 feeds lnx_chunk_fwd's vector gate

@@ -18,7 +18,7 @@ EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fuses_l2norm", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
     "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
-    "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
+    "lnx_gdn_gate_fwd", "lnx_gdn_gate_bwd", "lnx_gdn_gate_bwd_workspace_bytes", "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
     "lnx_profile_enable", "lnx_profile_read",
 )
 
@@ -98,6 +98,12 @@ def load() -> C.CDLL:
     lib.lnx_kda_gate_bwd.restype = C.c_int
     lib.lnx_kda_gate_bwd.argtypes = [C.c_void_p] * 7 + [C.c_int64, C.c_int32, C.c_int32, C.c_float, C.c_int32, C.c_int32,
                                                          C.c_void_p, C.c_uint64, C.c_void_p]
+    lib.lnx_gdn_gate_fwd.restype = C.c_int
+    lib.lnx_gdn_gate_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
+    lib.lnx_gdn_gate_bwd_workspace_bytes.restype = C.c_uint64
+    lib.lnx_gdn_gate_bwd_workspace_bytes.argtypes = [C.c_int64, C.c_int32]
+    lib.lnx_gdn_gate_bwd.restype = C.c_int
+    lib.lnx_gdn_gate_bwd.argtypes = [C.c_void_p] * 10 + [C.c_int64, C.c_int32, C.c_float, C.c_int32, C.c_void_p, C.c_uint64, C.c_void_p]
     lib.lnx_sigmoid_fwd.restype = C.c_int
     lib.lnx_sigmoid_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     lib.lnx_sigmoid_bwd.restype = C.c_int

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblinearnexus_hip.so")
-SOURCES = ["c_api.hip", "recurrent.hip", "chunk_fwd.hip", "chunk_bwd.hip", "chunk_direct.hip", "conv1d.hip", "dplr.hip", "rmsnorm_gated.hip", "kda_gate.hip"]
+SOURCES = ["c_api.hip", "recurrent.hip", "chunk_fwd.hip", "chunk_bwd.hip", "chunk_direct.hip", "conv1d.hip", "dplr.hip", "rmsnorm_gated.hip", "kda_gate.hip", "gdn_gate.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -89,3 +89,51 @@ def test_errors_and_empty():
         la.kda_gate(torch.randn(1, 4, 4, device=DEV), A, 2)  # dk = 2 is not a multiple of 4
     o, b = la.kda_gate(torch.randn(1, 0, 8, device=DEV), A, 4)
     assert o.shape == (1, 0, 2, 4) and b is None
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("shape", [(2, 16, 4), (1, 1000, 16), (3, 33, 6), (1, 1, 1), (8, 4096, 16)])
+@pytest.mark.parametrize("neg,with_b,with_bias", [(False, True, True), (True, True, False), (False, False, True)])
+def test_gated_deltanet_gate_matches_oracle(shape, bf16, neg, with_b, with_bias):
+    """g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b) (* 2) and every gradient (gated_deltanet.py:804-815)."""
+    import linearnexus_amd as la
+    B, T, H = shape
+    r = np.random.default_rng(96)
+    rnd = (lambda x: to_bf16_grid(x.astype(np.float32))) if bf16 else (lambda x: x.astype(np.float32))
+    a, b = rnd(r.standard_normal((B, T, H)) * 6), rnd(r.standard_normal((B, T, H)) * 3)
+    A, bias = (r.standard_normal(H) * 0.5).astype(np.float32), r.standard_normal(H).astype(np.float32)
+    dg, dbeta = r.standard_normal((B, T, H)).astype(np.float32), r.standard_normal((B, T, H)).astype(np.float32)
+    g_ref, beta_ref = og.gdn_gate(a, A, bias if with_bias else None, b if with_b else None, neg)
+    da_ref, dA_ref, dbias_ref, db_ref = og.gdn_gate_grad(a, A, dg, bias if with_bias else None, b if with_b else None, dbeta, neg)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    ta, tA = _t(a, dt, True), _t(A, None, True)
+    tb = _t(b, dt, True) if with_b else None
+    tbias = _t(bias, None, True) if with_bias else None
+    g, beta = la.gated_deltanet_gate(ta, tA, tbias, tb, neg)
+    assert g.dtype == torch.float32 and g.shape == (B, T, H) and (beta is None) == (not with_b)
+    loss = (g * _t(dg)).sum()
+    if with_b:
+        loss = loss + (beta * _t(dbeta)).sum()
+    loss.backward()
+    assert max_rel(g.detach().cpu().numpy(), g_ref) < 1e-5
+    tol = 2e-2 if bf16 else 1e-5
+    assert max_rel(ta.grad.float().cpu().numpy(), da_ref) < tol
+    assert max_rel(tA.grad.cpu().numpy(), dA_ref) < 1e-4
+    if with_bias:
+        assert max_rel(tbias.grad.cpu().numpy(), dbias_ref) < 1e-4
+    if with_b:
+        assert max_rel(beta.detach().cpu().numpy(), beta_ref) < 1e-6
+        assert max_rel(tb.grad.float().cpu().numpy(), db_ref) < tol
+
+
+def test_gated_deltanet_gate_errors_and_empty():
+    import linearnexus_amd as la
+    A = torch.zeros(4, device=DEV)
+    with pytest.raises(RuntimeError):
+        la.gated_deltanet_gate(torch.randn(2, 3, 5, device=DEV), A)
+    with pytest.raises(RuntimeError):
+        la.gated_deltanet_gate(torch.randn(2, 3, 4), A)
+    with pytest.raises(RuntimeError):
+        la.gated_deltanet_gate(torch.randn(2, 3, 4, device=DEV), A, torch.zeros(3, device=DEV))
+    g, beta = la.gated_deltanet_gate(torch.randn(2, 0, 4, device=DEV), A)
+    assert g.shape == (2, 0, 4) and beta is None

@@ -71,8 +71,8 @@ def _pipeline(x, B, T, H, dk, dv, dt):
     q = q.view(B, T, H, dk).transpose(1, 2)  # token-first memory behind head-first views: used in place
     k = k.view(B, T, H, dk).transpose(1, 2)
     v = v.view(B, T, H, dv).transpose(1, 2)
-    beta = torch.sigmoid(t["b"]).transpose(1, 2)
-    g = (-torch.exp(t["A_log"]) * torch.nn.functional.softplus(t["a"] + t["dt_bias"])).transpose(1, 2)
+    g, beta = la.gated_deltanet_gate(t["a"], t["A_log"], t["dt_bias"], t["b"])  # [B, T, H] each, fp32
+    g, beta = g.transpose(1, 2), beta.transpose(1, 2)
     o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, None, 64, True)
     y = la.rmsnorm_gated(o.transpose(1, 2), t["gate"], t["norm_w"])
     (y.float() * t["dy"].float()).sum().backward()
@@ -172,8 +172,8 @@ def test_prefill_then_token_by_token_decode_equals_whole_sequence():
         v, cv = la.depthwise_conv1d_causal(x["v"][:, sl], x["wv"], None, cache=state.conv_state_v, activation="silu")
         n = q.shape[1]
         q, k, v = (t.view(B, n, H, -1).transpose(1, 2) for t in (q, k, v))
-        beta = torch.sigmoid(x["b"][:, sl]).transpose(1, 2)
-        g = (-torch.exp(x["A_log"]) * torch.nn.functional.softplus(x["a"][:, sl] + x["dt_bias"])).transpose(1, 2)
+        g, beta = la.gated_deltanet_gate(x["a"][:, sl], x["A_log"], x["dt_bias"], x["b"][:, sl])
+        g, beta = g.transpose(1, 2), beta.transpose(1, 2)
         if n == 1:
             o, S = la.gated_delta_rule_step(q[:, :, 0], k[:, :, 0], v[:, :, 0], g[:, :, 0], beta[:, :, 0], state.S)
             o = o[:, :, None]

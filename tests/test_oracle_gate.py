@@ -39,3 +39,24 @@ def test_closed_forms_and_finite_differences():
             ap, am = [g, A], [g, A]
             ap[which], am[which] = p, m
             assert abs((f(*ap) - f(*am)) / 2e-6 - grad[i]) < 1e-6
+
+
+def test_gdn_gate_against_torch_autograd_and_closed_forms():
+    """gated_deltanet.py:804-815 with torch's softplus / sigmoid + autograd; softplus(0) = ln 2, sigmoid(0) = 1/2."""
+    r = np.random.default_rng(3)
+    a, b = r.standard_normal((2, 7, 5)) * 10, r.standard_normal((2, 7, 5)) * 3  # softplus far into both tails
+    A, bias = r.standard_normal(5) * 0.5, r.standard_normal(5)
+    dg, dbeta = r.standard_normal((2, 7, 5)), r.standard_normal((2, 7, 5))
+    for neg in (False, True):
+        ta, tb, tA, tbias = (torch.tensor(x, requires_grad=True) for x in (a, b, A, bias))
+        g_t = -torch.exp(tA) * torch.nn.functional.softplus(ta + tbias, threshold=1e9)
+        beta_t = torch.sigmoid(tb) * (2.0 if neg else 1.0)
+        ((g_t * torch.tensor(dg)).sum() + (beta_t * torch.tensor(dbeta)).sum()).backward()
+        g, beta = og.gdn_gate(a, A, bias, b, neg)
+        assert np.allclose(g, g_t.detach().numpy(), atol=1e-12) and np.allclose(beta, beta_t.detach().numpy(), atol=1e-14)
+        d_a, d_A, d_bias, d_b = og.gdn_gate_grad(a, A, dg, bias, b, dbeta, neg)
+        assert np.allclose(d_a, ta.grad.numpy(), atol=1e-12) and np.allclose(d_b, tb.grad.numpy(), atol=1e-12)
+        assert np.allclose(d_A, tA.grad.numpy(), atol=1e-11) and np.allclose(d_bias, tbias.grad.numpy(), atol=1e-11)
+    g, beta = og.gdn_gate(np.zeros((1, 2)), np.array([0.0, np.log(3.0)]), None, np.zeros((1, 2)), True)
+    assert np.allclose(g, [[-np.log(2), -3 * np.log(2)]]) and np.allclose(beta, 1.0)
+    assert og.gdn_gate(np.zeros((1, 2)), np.zeros(2))[1] is None
