@@ -261,42 +261,47 @@ def bench_chunk(args, torch, la, _lib, name):
 
 
 def bench_decode(args, torch, la, _lib, steps=None):
-    """Gated DeltaNet decode step at B=256, H=32, dk=dv=128: fp32 state updated in place."""
+    """Gated DeltaNet decode step at B=256, H=32, dk=dv=128: fp32 state updated in place.  The timed loop replays the
+    step as a captured HIP graph (linearnexus_amd.decode.DecodeGraph -- the per-token loop of generate.py:243-271 with
+    one host call per token); the same steps through one eager op call each are reported beside it."""
+    from linearnexus_amd.decode import DecodeGraph
     B, H, d = 256, 32, 128
     dev = "cuda:0"
     gen = torch.Generator(device="cpu").manual_seed(4)
     rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
     nrm = lambda x: x / (x.norm(dim=-1, keepdim=True) + 1e-6)
     S = (rn(B, H, d, d) * 0.02).to(dev)
-    q, k = nrm(rn(B, H, d)).to(dev).bfloat16(), nrm(rn(B, H, d)).to(dev).bfloat16()
-    v = rn(B, H, d).to(dev).bfloat16()
-    beta = torch.sigmoid(rn(B, H)).to(dev)
-    g = (-torch.nn.functional.softplus(rn(B, H)) * 0.1).to(dev)
+    dg = DecodeGraph("gated", B, H, d, d, layers=1, dtype=torch.bfloat16, use_qk_l2norm=False, states=[S])
+    dg.step(nrm(rn(B, H, d)).to(dev).bfloat16(), nrm(rn(B, H, d)).to(dev).bfloat16(), rn(B, H, d).to(dev).bfloat16(),
+            torch.sigmoid(rn(B, H)).to(dev), (-torch.nn.functional.softplus(rn(B, H)) * 0.1).to(dev))
     steps = steps or 1000
 
-    def step():
-        la.gated_delta_rule_step(q, k, v, g, beta, S, use_qk_l2norm=False, inplace=True)
+    def timed(fn):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        _lib.profile_enable(True)
+        kern = []
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn()
+            if (i + 1) % 2048 == 0:
+                kern += [ms for _, ms in _lib.profile_read()]
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        kern += [ms for _, ms in _lib.profile_read()]
+        _lib.profile_enable(False)
+        return dt, kern
 
-    for _ in range(20):
-        step()
-    torch.cuda.synchronize()
-    _lib.profile_enable(True)
-    kern = []
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step()
-        if (i + 1) % 2048 == 0:
-            kern += [ms for _, ms in _lib.profile_read()]
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
-    kern += [ms for _, ms in _lib.profile_read()]
-    _lib.profile_enable(False)
+    dt_eager, kern = timed(dg._run)     # per-kernel HIP events are recorded on eager launches only
+    dt, _ = timed(dg.replay)
     nbytes = 2 * S.numel() * 4 + 4 * B * H * d * 2 + 2 * B * H * 4
     kms = sum(kern) / len(kern)
     tr, tr_src = measured_traffic("decode", "decode_step")
     return {
-        "workload": "gated_deltanet_decode_step", "B": B, "H": H, "dk": d, "dv": d, "steps": steps,
+        "workload": "gated_deltanet_decode_step", "B": B, "H": H, "dk": d, "dv": d, "steps": steps, "driver": "captured graph replay",
         "ms_per_step": dt * 1e3, "tokens_per_s": B / dt, "bytes_per_step": nbytes,
+        "wall_frac_of_hbm_peak": nbytes / dt / 1e9 / PEAK_HBM, "eager_ms_per_step": dt_eager * 1e3,
         "roofline": {"bound": "hbm", "kernel": "decode_step", "achieved": nbytes / (kms * 1e-3) / 1e9, "peak": PEAK_HBM,
                      "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / PEAK_HBM,
                      "traffic": tr, "traffic_source": tr_src},

@@ -121,24 +121,29 @@ __global__ __launch_bounds__(256) void decode_step_kernel(TokenParams p) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t bh = blockIdx.x;
   float* sm = sm_all[wave];
-  const float* gp = (GATE == LNX_GATE_VECTOR) ? p.g + bh * DK : nullptr;
-  const float qk = stage_qk<T, DK, GATE>(reinterpret_cast<const T*>(p.q) + bh * DK,
-                                         reinterpret_cast<const T*>(p.k) + bh * DK, gp, sm, lane, p.scale,
-                                         p.l2norm);
-  __syncthreads();
   const int col0 = (blockIdx.y * 4 + wave) * 32 + (lane & 7) * 4;
-  if (col0 >= p.dv) return;
+  const bool active = col0 < p.dv;
   const int row0 = (lane >> 3) * RPL;
-  const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(p.g[bh]) : 1.f;
-  const int64_t sbase = (bh * DK + row0) * p.dv + col0;
+  const int64_t sbase = (bh * DK + row0) * p.dv + (active ? col0 : 0);
+  // The state loads go out first: they do not depend on the q / k staging below, whose loads, reductions and barrier
+  // would otherwise sit in front of the only traffic that matters.
   floatx4 S[RPL];
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
     // streamed once: non-temporal, so the 512 MiB state does not churn L2 / the memory-side cache
     S[i] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p.s_in + sbase + (int64_t)i * p.dv));
   }
-  const floatx4 v4 = load4(reinterpret_cast<const T*>(p.v) + bh * p.dv + col0);
-  const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, p.beta[bh], v4, qk);
+  const floatx4 v4 = load4(reinterpret_cast<const T*>(p.v) + bh * p.dv + (active ? col0 : 0));
+  const float beta = p.beta[bh];
+  const float g_s = (GATE == LNX_GATE_SCALAR) ? p.g[bh] : 0.f;
+  const float* gp = (GATE == LNX_GATE_VECTOR) ? p.g + bh * DK : nullptr;
+  const float qk = stage_qk<T, DK, GATE>(reinterpret_cast<const T*>(p.q) + bh * DK,
+                                         reinterpret_cast<const T*>(p.k) + bh * DK, gp, sm, lane, p.scale,
+                                         p.l2norm);
+  __syncthreads();
+  if (!active) return;
+  const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(g_s) : 1.f;
+  const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, beta, v4, qk);
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
     __builtin_nontemporal_store(S[i], reinterpret_cast<floatx4*>(p.s_out + sbase + (int64_t)i * p.dv));
