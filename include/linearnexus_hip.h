@@ -170,14 +170,29 @@ int lnx_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t rows, int32_
  *   xin = concat(cache, x) along T;  y[t] = act(bias + sum_j weight[j] * xin[t + j]);  new_cache = last K-1 rows of xin.
  * x, y, dy, dx [B,T,D] and cache, new_cache [B,K-1,D] in `dtype` (D a multiple of 16 bytes of elements);
  * weight [K,D], bias [D] and their gradients fp32.  bias, cache, new_cache, d_weight, d_bias may be NULL
- * (cache NULL = zeros).  new_cache may alias cache for T <= 32 (decode).  The backward treats the cache as a
- * constant and overwrites d_weight / d_bias (it clears them with a fill kernel, then accumulates atomically).
+ * (cache NULL = zeros).  new_cache may alias cache for T <= 32 (decode).  lnx_conv1d_bwd overwrites d_weight / d_bias
+ * (it clears them with a fill kernel, then accumulates atomically); lnx_conv1d_cache_bwd gives the gradient with respect
+ * to the carry-in cache, d_cache [B,K-1,D] in `dtype` (JAX autodiff of conv.py:56-67 differentiates the concatenation).
+ * A width-1 kernel is the identity plus bias and ignores its weight (conv.py:39-44; d_weight is then zero).
+ * Packed batches (the layout the chunk ops take with cu_seqlens; the reference has no packed convolution, this is one
+ * call of conv.py:13-68 per sequence with a zero cache): x, y, dy, dx [1,T,D], cu_seqlens [nseq+1] device int32 under
+ * the contract stated at the top; the taps stop at the first token of each token's sequence, new_cache (may be NULL)
+ * receives the last K-1 rows of the last sequence.
  */
 int lnx_conv1d_fwd(const void* x, const float* weight, const float* bias, const void* cache, void* y, void* new_cache,
                    int32_t B, int32_t T, int32_t D, int32_t K, int32_t dtype, int32_t activation, void* hip_stream);
 int lnx_conv1d_bwd(const void* x, const float* weight, const float* bias, const void* cache, const void* dy, void* dx,
                    float* d_weight, float* d_bias, int32_t B, int32_t T, int32_t D, int32_t K, int32_t dtype,
                    int32_t activation, void* hip_stream);
+int lnx_conv1d_cache_bwd(const void* x, const float* weight, const float* bias, const void* cache, const void* dy,
+                         void* d_cache, int32_t B, int32_t T, int32_t D, int32_t K, int32_t dtype, int32_t activation,
+                         void* hip_stream);
+int lnx_conv1d_packed_fwd(const void* x, const float* weight, const float* bias, const int32_t* cu_seqlens, int32_t nseq,
+                          void* y, void* new_cache, int32_t T, int32_t D, int32_t K, int32_t dtype, int32_t activation,
+                          void* hip_stream);
+int lnx_conv1d_packed_bwd(const void* x, const float* weight, const float* bias, const int32_t* cu_seqlens, int32_t nseq,
+                          const void* dy, void* dx, float* d_weight, float* d_bias, int32_t T, int32_t D, int32_t K,
+                          int32_t dtype, int32_t activation, void* hip_stream);
 
 /*
  * RWKV-7's diagonal-plus-low-rank delta rule (linearnexus/modules/linear_attn/rwkv7.py:114-265), the sibling

@@ -17,7 +17,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fuses_l2norm", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
-    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
+    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_conv1d_cache_bwd", "lnx_conv1d_packed_fwd", "lnx_conv1d_packed_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
     "lnx_gdn_gate_fwd", "lnx_gdn_gate_bwd", "lnx_gdn_gate_bwd_workspace_bytes", "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
     "lnx_profile_enable", "lnx_profile_read",
 )
@@ -84,6 +84,12 @@ def load() -> C.CDLL:
     lib.lnx_conv1d_fwd.argtypes = [C.c_void_p] * 6 + [C.c_int32] * 6 + [C.c_void_p]
     lib.lnx_conv1d_bwd.restype = C.c_int
     lib.lnx_conv1d_bwd.argtypes = [C.c_void_p] * 8 + [C.c_int32] * 6 + [C.c_void_p]
+    lib.lnx_conv1d_cache_bwd.restype = C.c_int
+    lib.lnx_conv1d_cache_bwd.argtypes = [C.c_void_p] * 6 + [C.c_int32] * 6 + [C.c_void_p]
+    lib.lnx_conv1d_packed_fwd.restype = C.c_int
+    lib.lnx_conv1d_packed_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int32] + [C.c_void_p] * 2 + [C.c_int32] * 5 + [C.c_void_p]
+    lib.lnx_conv1d_packed_bwd.restype = C.c_int
+    lib.lnx_conv1d_packed_bwd.argtypes = [C.c_void_p] * 4 + [C.c_int32] + [C.c_void_p] * 4 + [C.c_int32] * 5 + [C.c_void_p]
     lib.lnx_rmsnorm_gated_fwd.restype = C.c_int
     lib.lnx_rmsnorm_gated_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
     lib.lnx_rmsnorm_gated_bwd.restype = C.c_int

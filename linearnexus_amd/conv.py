@@ -3,9 +3,11 @@
 ``depthwise_conv1d_causal(inputs, weight, bias, *, cache=None)`` mirrors linearnexus/core/conv.py:13-68:
 ``inputs [B,T,D]``, ``weight [K,D]`` (K <= 4), ``bias [D]`` or None, ``cache [B,K-1,D]`` or None; returns
 ``(output, new_cache)``.  Additive: ``activation="silu"`` fuses the SiLU the blocks apply right after
-(gated_deltanet.py:765-779) and ``inplace_cache=True`` writes the new cache over the old one (decode).
-Differentiable with respect to inputs, weight and bias through the HIP backward kernel; the cache is
-treated as a constant.  There is no other code path: the ops raise if the library is missing.
+(gated_deltanet.py:765-779), ``inplace_cache=True`` writes the new cache over the old one (decode) and
+``cu_seqlens`` makes the batch packed (``inputs [1,T,D]``: the taps stop at the start of each sequence, as if
+every sequence went through the function on its own with a zero cache -- the layout the chunk ops take).
+Differentiable with respect to inputs, weight, bias and the carry-in cache through the HIP backward kernels.
+There is no other code path: the ops raise if the library is missing.
 """
 from __future__ import annotations
 
@@ -14,7 +16,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from .linear_attn import _DT, _ptr, _stream
+from .linear_attn import _DT, _check_cu_seqlens, _ptr, _stream
 
 Tensor = torch.Tensor
 _ACT = {None: 0, "none": 0, "silu": 1}
@@ -45,7 +47,7 @@ def _check(inputs: Tensor, weight: Tensor, bias: Optional[Tensor], cache: Option
 
 class _Conv(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, cache, act, inplace_cache):
+    def forward(ctx, x, weight, bias, cache, act, inplace_cache, cu):
         B, T, D = x.shape
         K = weight.shape[0]
         lib = _lib.load()
@@ -58,23 +60,28 @@ class _Conv(torch.autograd.Function):
                     raise RuntimeError("inplace_cache=True needs a contiguous cache of the inputs' dtype")
                 cin = new_cache = cache
             else:
-                cin = cache.to(x.dtype).contiguous()
+                cin = cache.detach().to(x.dtype).contiguous()
                 new_cache = torch.empty_like(cin)
         else:
             cin = None
             new_cache = torch.empty(B, K - 1, D, dtype=x.dtype, device=x.device)
         y = torch.empty_like(x)
-        _lib.check(lib.lnx_conv1d_fwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cin), _ptr(y), _ptr(new_cache),
-                                      B, T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_fwd")
-        ctx.save_for_backward(x, w32, b32, None if inplace_cache else cin)
-        ctx.meta = (act, weight.dtype, None if bias is None else bias.dtype, inplace_cache and cin is not None)
+        if cu is None:
+            _lib.check(lib.lnx_conv1d_fwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cin), _ptr(y), _ptr(new_cache),
+                                          B, T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_fwd")
+        else:
+            _lib.check(lib.lnx_conv1d_packed_fwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cu), cu.numel() - 1, _ptr(y), _ptr(new_cache),
+                                                 T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_packed_fwd")
+        ctx.save_for_backward(x, w32, b32, None if inplace_cache else cin, cu)
+        ctx.meta = (act, weight.dtype, None if bias is None else bias.dtype, inplace_cache and cin is not None,
+                    None if cache is None else cache.dtype)
         ctx.mark_non_differentiable(new_cache)
         return y, new_cache
 
     @staticmethod
     def backward(ctx, dy, _dcache):
-        x, w32, b32, cin = ctx.saved_tensors
-        act, wdt, bdt, lost_cache = ctx.meta
+        x, w32, b32, cin, cu = ctx.saved_tensors
+        act, wdt, bdt, lost_cache, cdt = ctx.meta
         if lost_cache:
             raise RuntimeError("cannot differentiate through a convolution whose cache was updated in place")
         B, T, D = x.shape
@@ -83,16 +90,34 @@ class _Conv(torch.autograd.Function):
         dx = torch.empty_like(x)
         dw = torch.empty_like(w32)
         db = None if b32 is None else torch.empty_like(b32)
-        _lib.check(_lib.load().lnx_conv1d_bwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cin), _ptr(dy), _ptr(dx), _ptr(dw),
-                                              _ptr(db), B, T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_bwd")
-        return dx, dw.to(wdt), None if db is None else db.to(bdt), None, None, None
+        lib = _lib.load()
+        if cu is None:
+            _lib.check(lib.lnx_conv1d_bwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cin), _ptr(dy), _ptr(dx), _ptr(dw),
+                                          _ptr(db), B, T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_bwd")
+        else:
+            _lib.check(lib.lnx_conv1d_packed_bwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cu), cu.numel() - 1, _ptr(dy), _ptr(dx),
+                                                 _ptr(dw), _ptr(db), T, D, K, _DT[x.dtype], act, _stream(x)), "lnx_conv1d_packed_bwd")
+        dc = None
+        if cin is not None and ctx.needs_input_grad[3] and K > 1:
+            dc = torch.empty_like(cin)
+            _lib.check(lib.lnx_conv1d_cache_bwd(_ptr(x), _ptr(w32), _ptr(b32), _ptr(cin), _ptr(dy), _ptr(dc), B, T, D, K,
+                                                _DT[x.dtype], act, _stream(x)), "lnx_conv1d_cache_bwd")
+            dc = dc.to(cdt)
+        return dx, dw.to(wdt), None if db is None else db.to(bdt), dc, None, None, None
 
 
 def depthwise_conv1d_causal(inputs: Tensor, weight: Tensor, bias: Optional[Tensor] = None, *,
                             cache: Optional[Tensor] = None, activation: Optional[str] = None,
-                            inplace_cache: bool = False) -> Tuple[Tensor, Tensor]:
+                            inplace_cache: bool = False, cu_seqlens=None) -> Tuple[Tensor, Tensor]:
     """Depthwise causal conv1d with optional cache warm-start (linearnexus/core/conv.py:13-68)."""
-    _check(inputs, weight, bias, cache)
+    B, T, D, K = _check(inputs, weight, bias, cache)
     if activation not in _ACT:
         raise ValueError(f"activation must be None or 'silu', got {activation!r}")
-    return _Conv.apply(inputs, weight, bias, cache, _ACT[activation], bool(inplace_cache))
+    cu = None
+    if cu_seqlens is not None:
+        if B != 1:
+            raise RuntimeError("cu_seqlens needs a packed batch with B == 1")
+        if cache is not None:
+            raise RuntimeError("a packed batch starts every sequence from a zero cache: pass cache=None")
+        cu = _check_cu_seqlens(cu_seqlens, T).to(device=inputs.device, dtype=torch.int32).contiguous()
+    return _Conv.apply(inputs, weight, bias, cache, _ACT[activation], bool(inplace_cache), cu)

@@ -33,15 +33,15 @@ def depthwise_conv1d_causal(inputs, weight, bias=None, cache=None, activation=No
     xin = np.concatenate([cache, x], axis=1)
     z = np.zeros((B, T, D))
     for j in range(K):
-        z += w[j] * xin[:, j:j + T]
+        z += (1.0 if K == 1 else w[j]) * xin[:, j:j + T]  # conv.py:39-44: a width-1 kernel ignores its weight
     if bias is not None:
         z = z + np.asarray(bias, np.float64)
     y = silu(z) if activation == "silu" else z
     return y, xin[:, xin.shape[1] - (K - 1):]
 
 
-def depthwise_conv1d_causal_grad(inputs, weight, bias, dy, cache=None, activation=None):
-    """Gradients of <y, dy> with respect to inputs, weight and bias (the cache is a constant)."""
+def depthwise_conv1d_causal_grad(inputs, weight, bias, dy, cache=None, activation=None, with_cache=False):
+    """Gradients of <y, dy> with respect to inputs, weight and bias -- and the carry-in cache with ``with_cache``."""
     x = np.asarray(inputs, np.float64)
     w = np.asarray(weight, np.float64)
     dy = np.asarray(dy, np.float64)
@@ -50,7 +50,8 @@ def depthwise_conv1d_causal_grad(inputs, weight, bias, dy, cache=None, activatio
     if cache is None:
         cache = np.zeros((B, K - 1, D))
     xin = np.concatenate([np.asarray(cache, np.float64), x], axis=1)
-    z = sum(w[j] * xin[:, j:j + T] for j in range(K))
+    wk = np.ones_like(w) if K == 1 else w
+    z = sum(wk[j] * xin[:, j:j + T] for j in range(K))
     if bias is not None:
         z = z + np.asarray(bias, np.float64)
     if activation == "silu":
@@ -61,6 +62,18 @@ def depthwise_conv1d_causal_grad(inputs, weight, bias, dy, cache=None, activatio
     dxin = np.zeros_like(xin)
     dw = np.zeros_like(w)
     for j in range(K):
-        dxin[:, j:j + T] += w[j] * dz
-        dw[j] = (dz * xin[:, j:j + T]).sum((0, 1))
+        dxin[:, j:j + T] += wk[j] * dz
+        if K > 1:
+            dw[j] = (dz * xin[:, j:j + T]).sum((0, 1))
+    if with_cache:
+        return dxin[:, K - 1:], dw, dz.sum((0, 1)), dxin[:, :K - 1]
     return dxin[:, K - 1:], dw, dz.sum((0, 1))
+
+
+def packed(fn, cu_seqlens, inputs, *args, **kw):
+    """``fn`` applied to each sequence [cu[s], cu[s+1]) of a packed batch ``inputs [1,T,D]`` on its own (zero cache); the
+    first result of every call concatenated along T, the others summed (parameter gradients)."""
+    outs = [fn(inputs[:, a:b], *[x[:, a:b] if (hasattr(x, "ndim") and x.ndim == 3) else x for x in args], **kw)
+            for a, b in zip(cu_seqlens[:-1], cu_seqlens[1:])]
+    first = np.concatenate([o[0] for o in outs], axis=1)
+    return (first,) + tuple(sum(o[i] for o in outs) for i in range(1, len(outs[0])))

@@ -123,3 +123,63 @@ def test_full_size_linearity_and_shift():
     assert torch.equal(y[:, T - 2], wb[3].expand(B, D)) and torch.equal(y[:, T - 1], wb[2].expand(B, D))
     assert torch.count_nonzero(y[:, :100]) == 0 and torch.count_nonzero(y[:, 104:T - 2]) == 0
     assert torch.equal(cache[:, 1], torch.ones(B, D, device=DEV, dtype=torch.bfloat16)) and torch.count_nonzero(cache[:, 2]) == 0
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("act", [None, "silu"])
+@pytest.mark.parametrize("case", [(300, 64, 4, [0, 64, 65, 65, 200, 300]), (40, 32, 3, [0, 1, 2, 3, 40]),
+                                  (1000, 520, 4, [0, 31, 33, 500, 1000]), (130, 16, 2, [0, 130])])
+def test_packed_batch_equals_one_call_per_sequence(case, act, bf16):
+    """Packed batches: the taps stop at sequence boundaries -- outputs and all gradients equal the oracle applied to
+    every sequence on its own with a zero cache (sequences of 0, 1 and 2 tokens, boundaries inside a thread's run)."""
+    import linearnexus_amd as la
+    T, D, K, cu = case
+    x, w, b, _, dy = _data(41, 1, T, D, K, bf16, with_cache=False)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    y_ref, = oc.packed(lambda x_: (oc.depthwise_conv1d_causal(x_, w, b, None, act)[0],), cu, x)
+    dx_ref, dw_ref, db_ref = oc.packed(lambda x_, dy_: oc.depthwise_conv1d_causal_grad(x_, w, b, dy_, None, act), cu, x, dy)
+    tx, tw, tb = _t(x, dt, True), _t(w, None, True), _t(b, None, True)
+    y, nc = la.depthwise_conv1d_causal(tx, tw, tb, activation=act, cu_seqlens=torch.tensor(cu, dtype=torch.int32))
+    (y.float() * _t(dy)).sum().backward()
+    tol = 2e-2 if bf16 else 1e-5
+    assert max_rel(y.detach().float().cpu().numpy(), y_ref) < tol
+    assert max_rel(tx.grad.float().cpu().numpy(), dx_ref) < tol
+    assert max_rel(tw.grad.cpu().numpy(), dw_ref) < (1e-4 if not bf16 else 2e-2)
+    assert max_rel(tb.grad.cpu().numpy(), db_ref) < (1e-4 if not bf16 else 2e-2)
+    # the carry that leaves is that of the last sequence
+    last = x[:, cu[-2]:]
+    c_ref = np.concatenate([np.zeros((1, K - 1, D), np.float32), last], 1)[:, -(K - 1):]
+    assert np.array_equal(nc.float().cpu().numpy(), c_ref)
+    with pytest.raises(ValueError):
+        la.depthwise_conv1d_causal(tx, tw, tb, cu_seqlens=[0, 5, 3, T])
+    with pytest.raises(RuntimeError):
+        la.depthwise_conv1d_causal(tx, tw, tb, cache=torch.zeros(1, K - 1, D, device=DEV, dtype=dt), cu_seqlens=cu)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("shape", [(2, 16, 32, 4), (3, 2, 64, 4), (2, 1, 16, 3), (1, 70, 520, 2)])
+def test_gradient_of_the_carry_in_cache(shape, bf16):
+    import linearnexus_amd as la
+    B, T, D, K = shape
+    x, w, b, c, dy = _data(42, B, T, D, K, bf16)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    dc_ref = oc.depthwise_conv1d_causal_grad(x, w, b, dy, c, "silu", with_cache=True)[3]
+    tc = _t(c, dt, True)
+    y, _ = la.depthwise_conv1d_causal(_t(x, dt, True), _t(w), _t(b), cache=tc, activation="silu")
+    (y.float() * _t(dy)).sum().backward()
+    assert max_rel(tc.grad.float().cpu().numpy(), dc_ref) < (2e-2 if bf16 else 1e-5)
+
+
+def test_width_one_kernel_and_empty_sequence_without_cache():
+    """conv.py:39-44: kernel_size 1 is inputs + bias, whatever the weight holds.  An empty sequence with no cache hands
+    back the zero cache the reference builds (conv.py:46-47)."""
+    import linearnexus_amd as la
+    x = torch.randn(2, 9, 16, device=DEV, requires_grad=True)
+    w = torch.full((1, 16), 3.0, device=DEV, requires_grad=True)
+    b = torch.randn(16, device=DEV)
+    y, nc = la.depthwise_conv1d_causal(x, w, b)
+    assert torch.allclose(y, x + b, atol=1e-6) and nc.shape == (2, 0, 16)
+    y.sum().backward()
+    assert torch.allclose(x.grad, torch.ones_like(x)) and torch.count_nonzero(w.grad) == 0
+    y, nc = la.depthwise_conv1d_causal(torch.randn(2, 0, 16, device=DEV), torch.randn(4, 16, device=DEV), None)
+    assert y.shape == (2, 0, 16) and nc.shape == (2, 3, 16) and torch.count_nonzero(nc) == 0

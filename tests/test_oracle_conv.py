@@ -18,7 +18,7 @@ def _data(seed, B, T, D, K, with_cache=True):
     return x, w, b, c
 
 
-@pytest.mark.parametrize("K", [1, 2, 3, 4])
+@pytest.mark.parametrize("K", [2, 3, 4])
 def test_equals_fir_filter(K):
     x, w, b, _ = _data(1, 2, 19, 5, K, False)
     y, cache = oc.depthwise_conv1d_causal(x, w, b)
@@ -26,8 +26,38 @@ def test_equals_fir_filter(K):
         ref = scipy.signal.lfilter(w[::-1, d], [1.0], x[:, :, d], axis=1) + b[d]
         assert np.allclose(y[:, :, d], ref, atol=1e-12)
     assert cache.shape == (2, K - 1, 5)
-    if K > 1:
-        assert np.array_equal(cache, x[:, 19 - (K - 1):])
+    assert np.array_equal(cache, x[:, 19 - (K - 1):])
+
+
+def test_width_one_kernel_is_identity_plus_bias():
+    """conv.py:39-44 returns inputs + bias for kernel_size 1 and never reads the weight; the cache is empty."""
+    x, w, b, _ = _data(1, 2, 19, 5, 1, False)
+    y, cache = oc.depthwise_conv1d_causal(x, w, b)
+    assert np.array_equal(y, x + b) and cache.shape == (2, 0, 5)
+    dy = np.random.default_rng(9).standard_normal(x.shape)
+    dx, dw, db = oc.depthwise_conv1d_causal_grad(x, w, b, dy)
+    assert np.array_equal(dx, dy) and not dw.any() and np.allclose(db, dy.sum((0, 1)))
+
+
+def test_cache_gradient_finite_differences():
+    x, w, b, c = _data(10, 2, 5, 3, 4)
+    dy = np.random.default_rng(11).standard_normal(x.shape)
+    for T in (5, 2):  # also a sequence shorter than the cache
+        dc = oc.depthwise_conv1d_causal_grad(x[:, :T], w, b, dy[:, :T], c, "silu", with_cache=True)[3]
+        f = lambda c_: (oc.depthwise_conv1d_causal(x[:, :T], w, b, c_, "silu")[0] * dy[:, :T]).sum()
+        for i in np.ndindex(c.shape):
+            p, m = c.copy(), c.copy()
+            p[i] += 1e-6
+            m[i] -= 1e-6
+            assert abs((f(p) - f(m)) / 2e-6 - dc[i]) < 1e-6
+
+
+def test_packed_helper_is_one_call_per_sequence():
+    x, w, b, _ = _data(12, 1, 11, 3, 3, False)
+    cu = [0, 4, 4, 9, 11]
+    y, = oc.packed(lambda x_: (oc.depthwise_conv1d_causal(x_, w, b, None, "silu")[0],), cu, x)
+    for a, e in zip(cu[:-1], cu[1:]):
+        assert np.array_equal(y[:, a:e], oc.depthwise_conv1d_causal(x[:, a:e], w, b, None, "silu")[0])
 
 
 def test_brute_force_with_cache_and_silu():
