@@ -108,7 +108,7 @@ def _dense(x: Tensor):
     """A contiguous tensor over x's memory (or a copy) and the function that maps results back to x's layout."""
     if x.is_contiguous():
         return x, (lambda y: y)
-    if _is_token_first(x):
+    if x.dim() >= 4 and _is_token_first(x):  # with fewer dimensions the transposition would move the last axis itself
         return x.transpose(1, 2), (lambda y: y.transpose(1, 2))
     return x.contiguous(), (lambda y: y)
 
@@ -205,10 +205,13 @@ def _step(q, k, v, g, beta, state, scale, l2norm, o_dtype_from_state, inplace):
     if _wants_grad(q, k, v, g, beta, state):
         if inplace:
             raise RuntimeError("inplace=True overwrites the state a backward pass would need")
-        o, s_out = _chunk(q[:, :, None], k[:, :, None], v[:, :, None], None if g is None else g[:, :, None],
+        # the token kernels normalise and compute in fp32 (gated_deltanet.py:193-195): so does this path, so that the
+        # values do not depend on whether a gradient is wanted
+        up = (lambda t: t.to(torch.float32)) if (l2norm and q.dtype != torch.float32) else (lambda t: t)
+        o, s_out = _chunk(up(q)[:, :, None], up(k)[:, :, None], up(v)[:, :, None], None if g is None else g[:, :, None],
                           _squeeze_beta(beta, 3)[:, :, None], scale, state, CHUNK, l2norm,
-                          torch.float32 if o_dtype_from_state else q.dtype, False, None)
-        return o[:, :, 0], s_out
+                          torch.float32 if (o_dtype_from_state or l2norm) else q.dtype, False, None)
+        return o[:, :, 0].to(state.dtype if o_dtype_from_state else q.dtype), s_out
     B, H, dk = q.shape
     dv = v.shape[-1]
     beta = _squeeze_beta(beta, 3)
@@ -303,6 +306,10 @@ def _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens=None):
         o, sT = _recurrent(q, k, v, g, beta, scale, initial_state, l2norm, cu_seqlens)
         return o.to(back), sT
     if _wants_grad(q, k, v, g, beta, initial_state):
+        if l2norm and q.dtype != torch.float32:  # fp32 normalisation and arithmetic, like the token kernels
+            o, sT = _chunk(q.to(torch.float32), k.to(torch.float32), v.to(torch.float32), g, beta, scale, initial_state, CHUNK,
+                           l2norm, torch.float32, False, cu_seqlens)
+            return o.to(q.dtype), sT
         return _chunk(q, k, v, g, beta, scale, initial_state, CHUNK, l2norm, q.dtype, False, cu_seqlens)
     dt, B, H, T, dk, dv, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, initial_state, cu_seqlens)
     if scale is None:

@@ -173,3 +173,21 @@ def test_l2norm_rows_fwd_bwd(rows, d, bf16):
         xa = x.detach().to(dt).requires_grad_(True)
         la.l2norm_rows(xa).backward(dy.to(dt))
         assert torch.equal(xa.grad, dx)
+
+
+def test_l2norm_rows_on_transposed_views():
+    """A non-contiguous [B, T, d] view whose transpose(1, 2) is contiguous is normalised over its LAST axis (forward
+    and backward), and a [B, H, T, d] view over token-first memory keeps its memory order."""
+    import linearnexus_amd as la
+    base = torch.randn(3, 16, 5, device=DEV)          # memory [B, d, T]
+    x = base.transpose(1, 2).requires_grad_(True)     # view [B, T, d], non-contiguous
+    assert not x.is_contiguous() and x.transpose(1, 2).is_contiguous()
+    xr = x.detach().clone().requires_grad_(True)
+    dy = torch.randn(3, 5, 16, device=DEV)
+    la.l2norm_rows(x).backward(dy)
+    (xr / (xr.norm(dim=-1, keepdim=True) + 1e-6)).backward(dy)
+    assert torch.allclose(la.l2norm_rows(x.detach()), xr.detach() / (xr.detach().norm(dim=-1, keepdim=True) + 1e-6), atol=1e-6)
+    assert torch.allclose(x.grad, xr.grad, atol=1e-5)
+    tf = torch.randn(2, 7, 3, 16, device=DEV).transpose(1, 2)  # [B, H, T, d] over [B, T, H, d] memory
+    y = la.l2norm_rows(tf)
+    assert y.stride() == tf.stride() and torch.allclose(y, tf / (tf.norm(dim=-1, keepdim=True) + 1e-6), atol=1e-6)
