@@ -213,15 +213,17 @@ def bench_chunk(args, torch, la, _lib, name):
     _lib.profile_enable(False)
 
     # the same forward without gradients (prefill / inference): forward_only is set, nothing is saved
-    with torch.no_grad():
-        for _ in range(2):
-            forward()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for _ in range(args.steps):
-            forward()
-        torch.cuda.synchronize()
-        fwd_only_ms = (time.perf_counter() - t1) / args.steps * 1e3
+    fwd_only_ms = float("nan")
+    if not args.no_forward_only:
+        with torch.no_grad():
+            for _ in range(2):
+                forward()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(args.steps):
+                forward()
+            torch.cuda.synchronize()
+            fwd_only_ms = (time.perf_counter() - t1) / args.steps * 1e3
 
     if nseq:
         nchunks = H * int(sum(-(-int(l) // C) for l in (cu_np[1:] - cu_np[:-1])))
@@ -250,7 +252,7 @@ def bench_chunk(args, torch, la, _lib, name):
         "tflops_algorithmic": total_fl / dtm / 1e12,
         "mfma_peak_frac": total_fl / dtm / 1e12 / peak,
         "kernel_ms": {n: round(t, 4) for n, t in avg.items()},
-        "forward_only_ms": round(fwd_only_ms, 4),
+        "forward_only_ms": None if fwd_only_ms != fwd_only_ms else round(fwd_only_ms, 4),
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": tr, "traffic_source": tr_src},
     }
@@ -524,6 +526,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated", "kda_gate", "prefill_long"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-forward-only", action="store_true",
+                    help="skip the extra forward-without-gradients timing (profiler runs: keeps the per-kernel averages to the differentiable step)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
     args = ap.parse_args()
