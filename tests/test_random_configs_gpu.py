@@ -42,15 +42,33 @@ def _cases():
         T = int(r.integers(1, 200))
         nseq = int(r.integers(1, 5)) if packed else 0
         out.append((i, gate, bf16, B, H, T, dk, dv, nseq, bool(r.integers(2)), bool(r.integers(2))))
+    # a third list: the in-op L2 normalisation (the reference's default) on rows of very different lengths -- inside the
+    # kernels for bf16 with a scalar gate, stand-alone kernels around them otherwise
+    r = np.random.default_rng(2026)
+    for i in range(60, 84):
+        gate = ("scalar", "scalar", "vector")[i % 3]
+        bf16 = bool(r.integers(4) > 0)
+        dk = int(r.choice([64, 128, 128, 96, 256]))
+        dv = int(r.choice([64, 128, 256, 80] if bf16 or dk < 256 else [64, 128]))
+        H = int(r.integers(1, 4))
+        packed = bool(r.integers(3) == 0)
+        B = 1 if packed else int(r.integers(1, 3))
+        T = int(r.integers(1, 300))
+        nseq = int(r.integers(1, 5)) if packed else 0
+        out.append((i, gate, bf16, B, H, T, dk, dv, nseq, bool(r.integers(2)), bool(r.integers(2)), True))
     return out
 
 
-@pytest.mark.parametrize("case", _cases(), ids=lambda c: f"{c[0]}-{c[1]}-{'bf16' if c[2] else 'f32'}-B{c[3]}H{c[4]}T{c[5]}k{c[6]}v{c[7]}s{c[8]}")
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: f"{c[0]}-{c[1]}-{'bf16' if c[2] else 'f32'}-B{c[3]}H{c[4]}T{c[5]}k{c[6]}v{c[7]}s{c[8]}{'-l2' if len(c) > 11 else ''}")
 def test_random_configuration(case):
     import linearnexus_amd as la
-    i, gate, bf16, B, H, T, dk, dv, nseq, with_state, token_first = case
-    x = make_inputs(500 + i, B, H, T, dk, dv, gate=gate, with_grad=True)
+    i, gate, bf16, B, H, T, dk, dv, nseq, with_state, token_first = case[:11]
+    l2 = len(case) > 11 and case[11]
+    x = make_inputs(500 + i, B, H, T, dk, dv, gate=gate, with_grad=True, normalize=not l2)
     r = np.random.default_rng(900 + i)
+    if l2:
+        x["q"] = x["q"] * np.exp(r.standard_normal((B, H, T, 1))).astype(np.float32)
+        x["k"] = x["k"] * np.exp(r.standard_normal((B, H, T, 1))).astype(np.float32)
     cu = None
     nstate = B
     if nseq:
@@ -80,10 +98,10 @@ def test_random_configuration(case):
             o_s, S_s = rc.delta_rule_recurrent(sl("q"), sl("k"), sl("v"), sl("beta"), S0)
         else:
             fn = rc.gated_delta_rule_recurrent if gate == "scalar" else rc.kda_recurrent
-            o_s, S_s = fn(sl("q"), sl("k"), sl("v"), gg, sl("beta"), None, S0, False)
+            o_s, S_s = fn(sl("q"), sl("k"), sl("v"), gg, sl("beta"), None, S0, l2)
         o_ref[:, :, a:b] = o_s
         S_ref.append(S_s)
-        ad = delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), gg, x["dS"][st], None, S0, False)
+        ad = delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), gg, x["dS"][st], None, S0, l2)
         for n in names:
             g_ref[n].append(ad[n])
         dS0_ref.append(ad["dS0"])
@@ -106,9 +124,9 @@ def test_random_configuration(case):
     if gate == "none":
         o, S = la.delta_rule_chunkwise(q, k, v, beta, S0, cu_seqlens=cu_t)
     elif gate == "scalar":
-        o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, S0, 64, False, cu_seqlens=cu_t)
+        o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, S0, 64, l2, cu_seqlens=cu_t)
     else:
-        o, S = la.kda_chunkwise(q, k, v, g, beta, None, S0, 64, False, cu_seqlens=cu_t)
+        o, S = la.kda_chunkwise(q, k, v, g, beta, None, S0, 64, l2, cu_seqlens=cu_t)
     dO = torch.from_numpy(x["dO"]).to(DEV)
     ((o.float() * dO).sum() + (S * torch.from_numpy(x["dS"]).to(DEV)).sum()).backward()
     tol = 2e-2 if bf16 else 1e-4
