@@ -536,7 +536,7 @@ template <typename T, int DK, int GATE> struct DqkCfg {
 };
 
 template <typename T, int DK, int GATE>
-__global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 ? 3 : 2)) void bwd_dqk_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2 : 1) : sizeof(T) == 2 ? 3 : 2)) void bwd_dqk_kernel(BwdParams p) {
   typedef DqkCfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF;
   extern __shared__ __align__(16) char smem[];
@@ -663,7 +663,16 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
       sOut[r * LDF + c] = aQ[0][0][e] * p.scale * __expf(sAl[r * LDF + c]);
     }
     lds_barrier();
-    pair_row<T, 64, false>(sOut, sR, sAl, LDF, sKr, LDC, p.scale, tid);
+    // both pair sums of dP: 2-byte inputs take them together on the bf16 MFMA and keep them in registers until used
+    float pr[16], pc[16];
+    const int pch = 16 * wave + (lane & 15), ptok = 4 * (lane >> 4);  // this lane's channel; its tokens are 16 t + ptok + e
+    if constexpr (sizeof(T) == 2) {
+      pair_levels<false>(pr, pc, sR, sAl, LDF, sKr, LDC, sQr, LDC, tid);
+#pragma unroll
+      for (int x = 0; x < 16; ++x) sOut[(16 * (x >> 2) + ptok + (x & 3)) * LDF + pch] += p.scale * pr[x];
+    } else {
+      pair_row<T, 64, false>(sOut, sR, sAl, LDF, sKr, LDC, p.scale, tid);
+    }
     lds_barrier();
     T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK + ch0;
     for (int idx = tid; idx < 64 * 16; idx += 256) {
@@ -690,7 +699,12 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? 1 : sizeof(T) == 2 
     lds_barrier();
     if (tid < 64) sSS[tid] = sMisc[tid] + __expf(sAl[63 * LDF + tid]) * sSS[tid];  // added to row 63 below
     lds_barrier();
-    pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int x = 0; x < 16; ++x) sOut[(16 * (x >> 2) + ptok + (x & 3)) * LDF + pch] += p.scale * pc[x];
+    } else {
+      pair_col<T, 64, false>(sOut, sR, sAl, LDF, sQr, LDC, p.scale, tid);
+    }
     lds_barrier();
     T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + ch0;
     for (int idx = tid; idx < 64 * 16; idx += 256) {
@@ -957,17 +971,25 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       rs += __shfl_xor(rs, 2, LNX_WAVE);
       if ((tid & 3) == 0) atomicAdd(&sdB[r], rs);
     }
+#pragma unroll 1
     for (int h = 0; h < DK / 64; ++h) {
       const int ch0 = 64 * h;
       floatx4 dk0[4], dg0[4], up[4];
       lds_barrier();  // X tile / the previous half's tiles are dead
+      auto fetch_partial = [&]() {  // what bwd_dqk left of dk and dG for this half
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {  // all global reads of the half first
+        for (int it = 0; it < 4; ++it) {
+          const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+          dk0[it] = (r < len) ? load4(dkg + (int64_t)r * tsk + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+          dg0[it] = load4(dGg + r * DK + ch0 + c);
+        }
+      };
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {  // all global reads of the half first (2-byte inputs: the partial sums after the pair terms)
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         up[it] = load4(Gg + r * DK + ch0 + c);
-        dk0[it] = (r < len) ? load4(dkg + (int64_t)r * tsk + ch0 + c) : floatx4{0.f, 0.f, 0.f, 0.f};
-        dg0[it] = load4(dGg + r * DK + ch0 + c);
       }
+      fetch_partial();
       stage_tile<T, 64, 64>(sKr, LDC, kg + ch0, tsk, len, tid);
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
@@ -1000,16 +1022,30 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         if ((tid & 3) == 0) atomicAdd(&sdB[r], t);
       }
       lds_barrier();
-      pair_row<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      float pr[16], pc[16];
+      const int pch = 16 * wave + (lane & 15), ptok = 4 * (lane >> 4);  // this lane's channel; its tokens are 16 t + ptok + e
+      constexpr bool LEVELS = DK <= 128;  // beyond that the live accumulators leave too few registers for it
+      if constexpr (sizeof(T) == 2 && LEVELS) {  // both pair sums of dA together on the bf16 MFMA
+        pair_levels<true>(pr, pc, sR, sGc, LDF, sKr, LDC, sKr, LDC, tid);
+#pragma unroll
+        for (int x = 0; x < 16; ++x) sOut[(16 * (x >> 2) + ptok + (x & 3)) * LDF + pch] += pr[x];
+      } else {
+        pair_row<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      }
       lds_barrier();
 #pragma unroll
       for (int it = 0; it < 4; ++it) {  // row-type part to registers, out restarts from zero
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         up[it] = load4(sOut + r * LDF + c);
-        store4(sOut + r * LDF + c, floatx4{0.f, 0.f, 0.f, 0.f});
+        if (!(sizeof(T) == 2 && LEVELS)) store4(sOut + r * LDF + c, floatx4{0.f, 0.f, 0.f, 0.f});
       }
       lds_barrier();
-      pair_col<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      if constexpr (sizeof(T) == 2 && LEVELS) {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) sOut[(16 * (x >> 2) + ptok + (x & 3)) * LDF + pch] = pc[x];
+      } else {
+        pair_col<T, 64, true>(sOut, sR, sGc, LDF, sKr, LDC, 1.f, tid);
+      }
       lds_barrier();
 #pragma unroll
       for (int it = 0; it < 4; ++it) {

@@ -360,3 +360,182 @@ __device__ __forceinline__ void pair_col(float* out, const float* M, const float
     }
   }
 }
+
+// ---------------------------------------------------------------------------------------
+// pair_levels: both pair sums of a 64-channel tile at once for 2-byte inputs, on the bf16 MFMA, with every decay taken
+// once.  For i > j let h be the highest bit in which i and j differ; then m = (i with the bits below h cleared) lies
+// in (j, i], and E_ij = exp(G_i - G_m) exp(G_m - G_j) with both factors <= 1.  At "level" h every token has exactly
+// one role -- bit h set: a row token i with factor exp(G_i - G_m), clear: a column token j with factor
+// exp(G_m - G_j), m = (token with the bits below 2h cleared) + h -- so one exponential per (token, channel, level)
+// serves both sums:
+//   ro[i][c] = sum_{j < i} X[i][j] E_ij[c] b[j][c] = sum_h  F_h[i][c] * sum_j X_h[i][j] (F_h b)[j][c]
+//   co[j][c] = sum_{i > j} X[i][j] E_ij[c] a[i][c] = sum_h  F_h[j][c] * sum_i X_h[i][j] (F_h a)[i][c]
+// with X_h the entries of X whose (i, j) belong to level h: whole 16x16 blocks for h = 32, 16, 8, lane-masked diagonal
+// blocks for h = 4, 2, 1.  Wave w owns channels 16 w .. 16 w + 15; lane (c = lane % 16, kq = lane / 16) holds the
+// sixteen tokens 16 t + 4 kq + e (t, e = 0..3) of its channel, which is at once the k-slot order of the scaled B
+// operands of v_mfma_f32_16x16x16_bf16 and the accumulator rows of its results, so factors, operands and results
+// never leave the lane.  Not STRICT: the diagonal X[i][i] (E = 1) is added to both sums.
+// X [64][LNX_LDA] fp32, G [64][ldf] fp32, b / a [64][ld] bf16, all in LDS; results are per lane, index 4 t + e.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ bf16x4 pack_bf16x4(floatx4 v) {
+  // Two v_cvt_pk_bf16_f32, joined as integers: a four-element conversion is taken apart element by element and
+  // permuted back together.
+  typedef float floatx2_ __attribute__((ext_vector_type(2)));
+  typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
+  const uint2_ r = {__builtin_bit_cast(unsigned, __builtin_convertvector((floatx2_{v[0], v[1]}), bf16x2)),
+                    __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2_{v[2], v[3]}), bf16x2))};
+  return __builtin_bit_cast(bf16x4, r);
+}
+__device__ __forceinline__ floatx4 mfma16_bf16(bf16x4 a, bf16x4 b, floatx4 c) {
+  typedef short short4_ __attribute__((ext_vector_type(4)));
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_, a), __builtin_bit_cast(short4_, b), c, 0, 0, 0);
+}
+
+// A operands from X: block (ti, t) with lane = (row l16, k-slots 4 kq + e), and the same block transposed,
+// lane = (column l16, k-slots = rows 4 kq + e)
+__device__ __forceinline__ bf16x4 pair_x_rows(const float* __restrict__ X, int ti, int t, int l16, int kq) {
+  return pack_bf16x4(load4(X + (16 * ti + l16) * LNX_LDA + 16 * t + 4 * kq));
+}
+__device__ __forceinline__ bf16x4 pair_x_cols(const float* __restrict__ X, int ti, int t, int l16, int kq) {
+  const float* p = X + (16 * ti + 4 * kq) * LNX_LDA + 16 * t + l16;
+  return pack_bf16x4(floatx4{p[0], p[LNX_LDA], p[2 * LNX_LDA], p[3 * LNX_LDA]});
+}
+
+// Levels 32 and 16: whole 16x16 blocks of X, roles fixed per block -- row blocks (2, 3) against column blocks (0, 1)
+// at level 32; (1) against (0) and (3) against (2) at level 16.
+template <int H>
+__device__ __forceinline__ void pair_cross(float (&ro)[16], float (&co)[16], const float (&g)[16], const float (&dec)[16],
+                                           const float (&bv)[16], const float (&av)[16], const float* __restrict__ X,
+                                           const float* __restrict__ G, int ldf, int c, int l16, int kq) {
+  constexpr float LOG2E = 1.4426950408889634f;  // g arrives multiplied by log2(e): the factors are plain exp2
+  const float m0 = LOG2E * G[H * ldf + c], m1 = H == 32 ? m0 : LOG2E * G[48 * ldf + c];
+  float F[16];
+  bf16x4 B[4];  // block t as B operand: F b of a column block (row sums), F a of a row block (column sums)
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const bool up = ((16 * t) & H) != 0;
+    const float ref = (H == 32 || t < 2) ? m0 : m1;
+    // one exponential per four tokens, the others by the single-step decays: away from the reference the factors shrink
+    if (up) {
+      F[4 * t] = __builtin_amdgcn_exp2f(fminf(g[4 * t] - ref, 0.f));
+#pragma unroll
+      for (int e = 1; e < 4; ++e) F[4 * t + e] = F[4 * t + e - 1] * dec[4 * t + e];
+    } else {
+      F[4 * t + 3] = __builtin_amdgcn_exp2f(fminf(ref - g[4 * t + 3], 0.f));
+#pragma unroll
+      for (int e = 2; e >= 0; --e) F[4 * t + e] = F[4 * t + e + 1] * dec[4 * t + e + 1];
+    }
+    floatx4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = F[4 * t + e] * (up ? av[4 * t + e] : bv[4 * t + e]);
+    B[t] = pack_bf16x4(v);
+  }
+  const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ti = 1; ti < 4; ++ti) {
+    if (H == 32 ? ti < 2 : !(ti & 1)) continue;
+    floatx4 acc = zero;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      if (H == 32 ? t < 2 : t == ti - 1) acc = mfma16_bf16(pair_x_rows(X, ti, t, l16, kq), B[t], acc);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ro[4 * ti + e] += F[4 * ti + e] * acc[e];
+  }
+#pragma unroll
+  for (int tj = 0; tj < 3; ++tj) {
+    if (H == 32 ? tj >= 2 : (tj & 1)) continue;
+    floatx4 acc = zero;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      if (H == 32 ? t >= 2 : t == tj + 1) acc = mfma16_bf16(pair_x_cols(X, t, tj, l16, kq), B[t], acc);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) co[4 * tj + e] += F[4 * tj + e] * acc[e];
+  }
+}
+
+// Levels 8, 4, 2, 1 of one diagonal 16x16 block: lane = (row l16 of the block, k-slots 4 kq + e), and a row and a
+// k-slot only meet inside the same 2H-token segment.  g, b, a, ro, co: the lane's four tokens of this block.
+__device__ __forceinline__ void pair_diag(floatx4& ro, floatx4& co, const floatx4 g, const floatx4 dec, const floatx4 bv, const floatx4 av,
+                                          const float* __restrict__ X, const float* __restrict__ G, int ldf, int c, int t,
+                                          int l16, int kq) {
+  typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
+  constexpr float LOG2E = 1.4426950408889634f;
+  const uint2_ xr = __builtin_bit_cast(uint2_, pair_x_rows(X, t, t, l16, kq)), xc = __builtin_bit_cast(uint2_, pair_x_cols(X, t, t, l16, kq));
+  const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int H = 8; H >= 1; H >>= 1) {
+    floatx4 fu, fl;  // the factor of each token in its role at this level (row token: fu, column token: fl), 0 in the other
+    if (H >= 4) {  // all four tokens share the role and the reference: one exponential, the rest by the single-step decays
+      const bool up = H == 8 ? (kq & 2) != 0 : (kq & 1) != 0;
+      const float ref = LOG2E * G[(16 * t + (H == 8 ? 8 : 8 * (kq >> 1) + 4)) * ldf + c];
+      const float f = __builtin_amdgcn_exp2f(fminf(up ? g[0] - ref : ref - g[3], 0.f));
+      floatx4 F;
+      F[0] = up ? f : f * dec[3] * dec[2] * dec[1];
+      F[1] = up ? f * dec[1] : f * dec[3] * dec[2];
+      F[2] = up ? F[1] * dec[2] : f * dec[3];
+      F[3] = up ? F[2] * dec[3] : f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        fu[e] = up ? F[e] : 0.f;
+        fl[e] = up ? 0.f : F[e];
+      }
+    } else if (H == 2) {  // reference: token 2 of the four
+      fl = floatx4{dec[1] * dec[2], dec[2], 0.f, 0.f};
+      fu = floatx4{0.f, 0.f, 1.f, dec[3]};
+    } else {  // references: tokens 1 and 3
+      fl = floatx4{dec[1], 0.f, dec[3], 0.f};
+      fu = floatx4{0.f, 1.f, 0.f, 1.f};
+    }
+    // k-slots (0, 1) and (2, 3) each share a 2-token segment, so the masks act on whole dwords of the packed operand
+    uint2_ mk;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const bool on = H == 8 ? true : H == 4 ? (l16 >> 3) == (kq >> 1) : H == 2 ? (l16 >> 2) == kq : (l16 >> 1) == 2 * kq + w;
+      mk[w] = on ? 0xffffffffu : 0u;
+    }
+    const floatx4 r = mfma16_bf16(__builtin_bit_cast(bf16x4, xr & mk), pack_bf16x4(fl * bv), zero);
+    const floatx4 q = mfma16_bf16(__builtin_bit_cast(bf16x4, xc & mk), pack_bf16x4(fu * av), zero);
+    ro += fu * r;
+    co += fl * q;
+  }
+}
+
+template <bool STRICT>
+__device__ __forceinline__ void pair_levels(float (&ro)[16], float (&co)[16], const float* __restrict__ X,
+                                            const float* __restrict__ G, int ldf, const bf16_t* __restrict__ b, int ldb,
+                                            const bf16_t* __restrict__ a, int lda, int tid) {
+  const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, kq = lane >> 4;
+  const int c = 16 * wave + l16;
+  float g[16], bv[16], av[16];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int tok = 16 * t + 4 * kq + e, x = 4 * t + e;
+      g[x] = 1.4426950408889634f * G[tok * ldf + c];
+      bv[x] = (float)b[tok * ldb + c];
+      av[x] = (float)a[tok * lda + c];
+      const float d = STRICT ? 0.f : X[tok * LNX_LDA + tok];
+      ro[x] = d * bv[x];
+      co[x] = d * av[x];
+    }
+  float dec[16];  // single-step decays exp(G_tok - G_{tok-1}) inside each group of four (the first entry of a group is unused)
+#pragma unroll
+  for (int x = 0; x < 16; ++x) dec[x] = (x & 3) ? __builtin_amdgcn_exp2f(fminf(g[x] - g[x - 1], 0.f)) : 1.f;
+  pair_cross<32>(ro, co, g, dec, bv, av, X, G, ldf, c, l16, kq);
+  __builtin_amdgcn_sched_barrier(0);  // one part at a time: interleaving them multiplies the live factors
+  pair_cross<16>(ro, co, g, dec, bv, av, X, G, ldf, c, l16, kq);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    __builtin_amdgcn_sched_barrier(0);
+    floatx4 r4 = {ro[4 * t], ro[4 * t + 1], ro[4 * t + 2], ro[4 * t + 3]}, c4 = {co[4 * t], co[4 * t + 1], co[4 * t + 2], co[4 * t + 3]};
+    pair_diag(r4, c4, floatx4{g[4 * t], g[4 * t + 1], g[4 * t + 2], g[4 * t + 3]},
+              floatx4{1.f, dec[4 * t + 1], dec[4 * t + 2], dec[4 * t + 3]}, floatx4{bv[4 * t], bv[4 * t + 1], bv[4 * t + 2], bv[4 * t + 3]},
+              floatx4{av[4 * t], av[4 * t + 1], av[4 * t + 2], av[4 * t + 3]}, X, G, ldf, c, t, l16, kq);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ro[4 * t + e] = r4[e];
+      co[4 * t + e] = c4[e];
+    }
+  }
+}
