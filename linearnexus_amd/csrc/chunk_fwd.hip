@@ -247,6 +247,116 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
+// One 64-channel half of the forward pair products X_ij = sum_c k_i k_j E_ij and <q_i, k_j>_E for 2-byte inputs, on
+// v_mfma_f32_16x16x32_bf16.  Level H (32 .. 1) pairs a row token i (bit H set) with a column token j (bit H clear) of
+// the same 2H-token segment through the reference m = segment start + H:  E_ij = exp(G_i - G_m) exp(G_m - G_j), both
+// factors <= 1; each operand row is a token's K (or Q) times its factor, rounded to bf16.  Lane = (token l16 of a
+// 16-token block, kq): channels 8 kq .. 8 kq + 7 of each 32-channel step.  Nothing is shared between waves, so there is
+// no barrier: wave w forms block (2 + w / 2, w % 2) of both products (level 32), one product of block (1, 0) or (3, 2)
+// (level 16) and the diagonal block w (levels 8 .. 1 and the plain diagonal <q_i, k_i>).
+// K, Q [64][ldc] bf16, G [64][ldf] fp32 (cumulative gate), all in LDS.
+// ---------------------------------------------------------------------------------------
+struct PairOp {
+  bf16x8 lo, hi;  // channels 8 kq + 0..7 and 32 + 8 kq + 0..7 of this lane's token
+};
+__device__ __forceinline__ void pair_row_f32(float (&v)[16], const float* __restrict__ rowp) {  // rowp: row + 8 kq
+  const floatx4 a = load4(rowp), b = load4(rowp + 4), c = load4(rowp + 32), d = load4(rowp + 36);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[e] = a[e];
+    v[4 + e] = b[e];
+    v[8 + e] = c[e];
+    v[12 + e] = d[e];
+  }
+}
+__device__ __forceinline__ PairOp pair_row_raw(const bf16_t* __restrict__ rowp) {
+  return PairOp{*reinterpret_cast<const bf16x8*>(rowp), *reinterpret_cast<const bf16x8*>(rowp + 32)};
+}
+__device__ __forceinline__ PairOp pair_scaled(const PairOp& x, const float (&F)[16]) {  // F x, rounded to bf16
+  typedef unsigned uint4_ __attribute__((ext_vector_type(4)));
+  typedef float floatx2_ __attribute__((ext_vector_type(2)));
+  uint4_ lo, hi;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const floatx2_ a = {F[2 * w] * (float)x.lo[2 * w], F[2 * w + 1] * (float)x.lo[2 * w + 1]};
+    const floatx2_ b = {F[8 + 2 * w] * (float)x.hi[2 * w], F[8 + 2 * w + 1] * (float)x.hi[2 * w + 1]};
+    lo[w] = __builtin_bit_cast(unsigned, __builtin_convertvector(a, bf16x2));
+    hi[w] = __builtin_bit_cast(unsigned, __builtin_convertvector(b, bf16x2));
+  }
+  return PairOp{__builtin_bit_cast(bf16x8, lo), __builtin_bit_cast(bf16x8, hi)};
+}
+__device__ __forceinline__ PairOp pair_masked(const PairOp& x, unsigned m) {
+  typedef unsigned uint4_ __attribute__((ext_vector_type(4)));
+  return PairOp{__builtin_bit_cast(bf16x8, __builtin_bit_cast(uint4_, x.lo) & m), __builtin_bit_cast(bf16x8, __builtin_bit_cast(uint4_, x.hi) & m)};
+}
+__device__ __forceinline__ void pair_mma(floatx4& acc, const PairOp& a, const PairOp& b) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.lo, b.lo, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.hi, b.hi, acc, 0, 0, 0);
+}
+// factors exp(-(ga - gb)) clamped to <= 1 (ga >= gb up to rounding: the cumulative gate does not increase)
+__device__ __forceinline__ void pair_factors(float (&F)[16], const float (&ga)[16], const float (&gb)[16]) {
+#pragma unroll
+  for (int x = 0; x < 16; ++x) F[x] = __expf(fminf(gb[x] - ga[x], 0.f));
+}
+
+__device__ __forceinline__ void kda_pair_half(floatx4 (&a32)[2], floatx4& a16, floatx4 (&aD)[5][2], const bf16_t* __restrict__ K,
+                                              const bf16_t* __restrict__ Q, int ldc, const float* __restrict__ G, int ldf,
+                                              int wave, int lane) {
+  const int l16 = lane & 15, kq = lane >> 4;
+  const bf16_t* Kc = K + 8 * kq;
+  const bf16_t* Qc = Q + 8 * kq;
+  const float* Gc = G + 8 * kq;
+  float gi[16], gj[16], gm[16], F[16];
+  {  // level 32: rows 16 ti + l16 against columns 16 tj + l16, reference token 32
+    const int i = 16 * (2 + (wave >> 1)) + l16, j = 16 * (wave & 1) + l16;
+    pair_row_f32(gm, Gc + 32 * ldf);
+    pair_row_f32(gi, Gc + i * ldf);
+    pair_row_f32(gj, Gc + j * ldf);
+    pair_factors(F, gm, gi);  // exp(G_i - G_32)
+    const PairOp kr = pair_scaled(pair_row_raw(Kc + i * ldc), F), qr = pair_scaled(pair_row_raw(Qc + i * ldc), F);
+    pair_factors(F, gj, gm);  // exp(G_32 - G_j)
+    const PairOp kc = pair_scaled(pair_row_raw(Kc + j * ldc), F);
+    pair_mma(a32[0], kr, kc);
+    pair_mma(a32[1], qr, kc);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // one level at a time keeps the live operands few
+  {  // level 16: block (1, 0) or (3, 2), reference its first row token; waves 0, 2: K rows, waves 1, 3: Q rows
+    const int m = (wave < 2) ? 16 : 48, i = m + l16, j = m - 16 + l16;
+    pair_row_f32(gm, Gc + m * ldf);
+    pair_row_f32(gi, Gc + i * ldf);
+    pair_row_f32(gj, Gc + j * ldf);
+    pair_factors(F, gm, gi);
+    const PairOp r = pair_scaled(pair_row_raw(((wave & 1) ? Qc : Kc) + i * ldc), F);
+    pair_factors(F, gj, gm);
+    const PairOp kc = pair_scaled(pair_row_raw(Kc + j * ldc), F);
+    pair_mma(a16, r, kc);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  {  // diagonal block `wave`: token i = 16 wave + l16 is a row token of level H when bit H of l16 is set
+    const int i = 16 * wave + l16;
+    pair_row_f32(gi, Gc + i * ldf);
+    const PairOp kraw = pair_row_raw(Kc + i * ldc), qraw = pair_row_raw(Qc + i * ldc);
+    pair_mma(aD[4][1], qraw, kraw);  // only its diagonal is kept
+#pragma unroll
+    for (int lv = 0; lv < 4; ++lv) {
+      const int H = 8 >> lv;
+      const bool up = (l16 & H) != 0;
+      const int m = 16 * wave + ((l16 & ~(2 * H - 1)) | H);
+      pair_row_f32(gm, Gc + m * ldf);
+#pragma unroll
+      for (int x = 0; x < 16; ++x) F[x] = __expf(fminf(up ? gi[x] - gm[x] : gm[x] - gi[x], 0.f));
+      const PairOp pk = pair_scaled(kraw, F), pq = pair_scaled(qraw, F);
+      const unsigned mu = up ? 0xffffffffu : 0u;
+      const PairOp kb = pair_masked(pk, ~mu);
+      pair_mma(aD[lv][0], pair_masked(pk, mu), kb);
+      pair_mma(aD[lv][1], pair_masked(pq, mu), kb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------
 // kda_prepare: chunk_prepare for a per-channel (vector) gate.  The pairwise products carry the
 // decay inside the dk sum, X_ij = sum_c k_i[c] k_j[c] exp(G_i[c] - G_j[c]).  The channels are
 // taken in 64-wide halves (K, Q and the fp32 gate tile of one half fit LDS twice per CU): per half
@@ -307,6 +417,15 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   floatx4 acc[3];  // this wave's three below-diagonal tasks (block, product), summed over the halves
 #pragma unroll
   for (int u = 0; u < 3; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // 2-byte inputs: the pair products by levels on the bf16 MFMA (see pair_levels in chunk_common.h for the splitting).
+  // Wave w holds, summed over the halves: block (2 + w / 2, w % 2) of both products (level 32), one product of block
+  // (1, 0) or (3, 2) (level 16), and the diagonal block w of both products, one accumulator per level 8, 4, 2, 1 (each
+  // level has its own mask) plus the plain <q_i, k_i> diagonal.
+  constexpr bool LEVELS = sizeof(T) == 2;
+  floatx4 a32[2], a16, aD[5][2];
+  a32[0] = a32[1] = a16 = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < 5; ++u) aD[u][0] = aD[u][1] = floatx4{0.f, 0.f, 0.f, 0.f};
   for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) {  // the diagonal blocks accumulate here over the halves
     sA[idx] = 0.f;
     sT[idx] = 0.f;
@@ -355,6 +474,9 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         store4(Qgg + r * DK + c, qgv);
       }
     }
+    if constexpr (LEVELS) {
+      kda_pair_half(a32, a16, aD, reinterpret_cast<const bf16_t*>(sK), reinterpret_cast<const bf16_t*>(sQ), LDC, sG, LDF, wave, lane);
+    } else {
     // blocks below the diagonal: six blocks x two products = twelve tasks, three per wave
 #pragma unroll
     for (int u = 0; u < 3; ++u) {
@@ -400,8 +522,32 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         }
       }
     }
+    }
   }
   // ---- phase B: assemble X and <q, k>_E in sA / sT, write X and P, A = beta X, inverse ----
+  if constexpr (LEVELS) {
+    const int ti = 2 + (wave >> 1), tj = wave & 1, t16 = (wave < 2) ? 1 : 3;
+    float* d16 = (wave & 1) ? sT : sA;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int il = 4 * kq + e;  // row inside the 16x16 block, column l16
+      sA[(16 * ti + il) * LNX_LDA + 16 * tj + l16] = a32[0][e];
+      sT[(16 * ti + il) * LNX_LDA + 16 * tj + l16] = a32[1][e];
+      d16[(16 * t16 + il) * LNX_LDA + 16 * (t16 - 1) + l16] = a16[e];
+      // diagonal block: level H keeps the pairs inside one 2H-token segment (the roles are in the operands already)
+      const int x = il ^ l16;
+      float va = aD[0][0][e], vp = aD[0][1][e];
+      va += (x < 8) ? aD[1][0][e] : 0.f;
+      vp += (x < 8) ? aD[1][1][e] : 0.f;
+      va += (x < 4) ? aD[2][0][e] : 0.f;
+      vp += (x < 4) ? aD[2][1][e] : 0.f;
+      va += (x < 2) ? aD[3][0][e] : 0.f;
+      vp += (x < 2) ? aD[3][1][e] : 0.f;
+      vp += (x == 0) ? aD[4][1][e] : 0.f;
+      sA[(16 * wave + il) * LNX_LDA + 16 * wave + l16] = va;
+      sT[(16 * wave + il) * LNX_LDA + 16 * wave + l16] = vp;
+    }
+  } else {
 #pragma unroll
   for (int u = 0; u < 3; ++u) {
     const int t = wave + 4 * u;
@@ -409,6 +555,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
     float* dst = (t < 6) ? sA : sT;
 #pragma unroll
     for (int e = 0; e < 4; ++e) dst[(16 * I + 4 * kq + e) * LNX_LDA + 16 * J + l16] = acc[u][e];
+  }
   }
   lds_barrier();
   {

@@ -105,9 +105,13 @@ def test_config3_kda_full_shape():
     dO = torch.randn(B, H, T, d, device=DEV)
     o3, _ = la.kda_chunkwise(q, k, v, g, beta, None, None, 64, False)
     o3.backward(dO)
-    lhs = (o3.detach().double() * dO.bfloat16().double()).sum()
-    rhs = (v.grad.double() * v.detach().double()).sum()
-    assert abs(lhs - rhs) <= 5e-3 * abs(lhs), (float(lhs), float(rhs))
+    tl, tr = o3.detach().double() * dO.bfloat16().double(), v.grad.double() * v.detach().double()
+    lhs, rhs = tl.sum(), tr.sum()
+    # o leaves the kernels as bf16 and dv is bf16: independent relative errors, uniform within +-2^-9, on each of the
+    # 6.7e7 terms of either sum; sigma is the standard deviation of their accumulated effect.  The tiles between the
+    # kernels (D, dD, the states, W, U, the scaled pair operands) are rounded the same way, hence 8 sigma, not 4.
+    sigma = 2.0 ** -9 / 3 ** 0.5 * torch.sqrt((tl * tl).sum() + (tr * tr).sum())
+    assert abs(lhs - rhs) <= 8 * sigma, (float(lhs), float(rhs), float(sigma))
 
 
 def test_config5_deltanet_long_packed():
