@@ -675,11 +675,13 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     }
     lds_barrier();
     T* dqg = reinterpret_cast<T*>(p.dq) + tbase * DK + ch0;
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int r = idx >> 4, c = (idx & 15) * 4;
+    floatx4 qdq[4];  // q dq, kept until k dk is known: the gate gradient leaves once
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
       const floatx4 v = load4(sOut + r * LDF + c), qq = load4(sQr + r * LDC + c);
       if (r < len) store4(dqg + (int64_t)r * tsk + c, v);
-      store4(dGg + r * DK + c, qq * v);
+      qdq[it] = qq * v;
     }
     lds_barrier();
     // dk (column-type parts): e^{G_last - G} dKr + P part; chunk-end gate term from the Kr part
@@ -707,11 +709,12 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     }
     lds_barrier();
     T* dkg = reinterpret_cast<T*>(p.dk) + tbase * DK + ch0;
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int r = idx >> 4, c = (idx & 15) * 4;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
       const floatx4 v = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
       if (r < len) store4(dkg + (int64_t)r * tsk + c, v);
-      floatx4 dgv = load4(dGg + r * DK + c) - kk * v;  // written above by this same thread
+      floatx4 dgv = qdq[it] - kk * v;
       if (r == 63) dgv += load4(sSS + c);
       store4(dGg + r * DK + c, dgv);
     }
@@ -1052,22 +1055,28 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         const floatx4 um = load4(sOut + r * LDF + c), kk = load4(sKr + r * LDC + c);
         if (r < len) store4(dkg + (int64_t)r * tsk + ch0 + c, dk0[it] + up[it] + um);
-        store4(dGg + r * DK + ch0 + c, dg0[it] + kk * (up[it] - um));
+        store4(sOut + r * LDF + c, dg0[it] + kk * (up[it] - um));  // dG of this half, in place of the column-type part
+      }
+      lds_barrier();
+      {  // dg = reverse cumulative sum of dG over the chunk, per channel: 16-token segments in parallel, then their offsets
+        const int c = tid & 63, seg = tid >> 6;
+        float acc = 0.f;  // running sums written back in place: no array of sixteen values held across the barrier
+#pragma unroll 4
+        for (int i = 15; i >= 0; --i) {
+          acc += sOut[(16 * seg + i) * LDF + c];
+          sOut[(16 * seg + i) * LDF + c] = acc;
+        }
+        float* sSeg = reinterpret_cast<float*>(sKr);  // segment totals [4][64]: the K tile is dead
+        sSeg[seg * 64 + c] = acc;
+        lds_barrier();
+        float off = 0.f;
+        for (int s_ = seg + 1; s_ < 4; ++s_) off += sSeg[s_ * 64 + c];
+#pragma unroll 4
+        for (int i = 0; i < 16; ++i)
+          if (16 * seg + i < len) p.dg[(tbase + (16 * seg + i) * ts) * DK + ch0 + c] = sOut[(16 * seg + i) * LDF + c] + off;
       }
     }
-    __syncthreads();  // dG is read back below by other threads than wrote it: global memory must be ordered too
     if (tid < 64 && tid < len) p.dbeta[tbase + tid * ts] = sdB[tid];
-    if (tid < DK) {  // dg = reverse cumulative sum of dG over the chunk, per channel
-      float gv[64];
-#pragma unroll
-      for (int r = 0; r < 64; ++r) gv[r] = dGg[r * DK + tid];  // all loads in flight together
-      float acc = 0.f;
-#pragma unroll
-      for (int r = 63; r >= 0; --r) {
-        acc += gv[r];
-        if (r < len) p.dg[(tbase + r * ts) * DK + tid] = acc;
-      }
-    }
     return;
   }
   // The K slabs are still in LDS (the last one in the slab tile, the others in tiles of their own); the partial dk of
