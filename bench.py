@@ -381,6 +381,51 @@ def bench_dplr_step(torch, la, _lib, steps):
                          "frac": ach / PEAK_HBM, "traffic": None}}
 
 
+def bench_dplr_train(torch, la, _lib, steps, warmup):
+    """RWKV-7 DPLR scan forward + backward at B8 H16 T4096 dk=dv=64 bf16 (the block's head size 64): tokens/s, and the
+    backward kernel against the HBM roofline.  Algorithmic bytes of the backward: every token's starting state is written
+    to the segment tape and read back once (2 * 4 B per state element and token; the checkpoints add 1/64 of that), the
+    token vectors are read three times (checkpoint sweep, tape sweep, reverse sweep), six fp32 gradients leave."""
+    B, H, T, d = 8, 16, 4096, 64
+    gen = torch.Generator(device="cpu").manual_seed(9)
+    rn = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float32)
+    q, k, v = (rn(B, H, T, d).to("cuda:0").bfloat16().requires_grad_(True) for _ in range(3))
+    a, b = ((rn(B, H, T, d) * 0.1).to("cuda:0").bfloat16().requires_grad_(True) for _ in range(2))
+    gk = (-rn(B, H, T, d).abs() * 0.1).to("cuda:0").requires_grad_(True)
+    dO = rn(B, H, T, d).to("cuda:0").bfloat16()
+    leaves = (q, k, v, a, b, gk)
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        o, _ = la.dplr_delta_rule_recurrent(q, k, v, a, b, gk, d ** -0.5)
+        o.backward(dO)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    acc = {}
+    for n, ms in _lib.profile_read():
+        acc.setdefault(n, []).append(ms)
+    _lib.profile_enable(False)
+    avg = {n: sum(x) / len(x) for n, x in acc.items()}
+    tok = B * H * T
+    nbytes = tok * d * d * 4 * (2 + 1 / 64) + 3 * tok * (5 * d * 2 + d * 4 + d * 2) + tok * d * 2 + 6 * tok * d * 4
+    ach = nbytes / (avg["dplr_bwd"] * 1e-3) / 1e9
+    return {"metric": "DPLR scan fwd+bwd tokens/s", "value": B * T / dt, "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+            "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "rwkv7_dplr_scan_fwd_bwd", "B": B, "H": H, "T": T, "dk": d, "dv": d, "inputs": "bf16, fp32 gk"},
+            "kernel_ms": {n: round(x, 4) for n, x in avg.items()},
+            "roofline": {"bound": "hbm", "kernel": "dplr_bwd", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s",
+                         "frac": ach / PEAK_HBM, "traffic": None}}
+
+
 def bench_rmsnorm_gated(torch, la, _lib, steps, warmup):
     """Gated RMSNorm epilogue over config 2's outputs: x, gate [B8, T4096, H16, d128] bf16, forward + backward.
     Algorithmic bytes: x, gate in, y out; x, gate, dy in, dx, dgate out."""
@@ -524,7 +569,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "rmsnorm_gated", "kda_gate", "prefill_long"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "dplr_train", "rmsnorm_gated", "kda_gate", "prefill_long"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-forward-only", action="store_true",
                     help="skip the extra forward-without-gradients timing (profiler runs: keeps the per-kernel averages to the differentiable step)")
@@ -561,6 +606,9 @@ def main():
         return
     if args.workload == "dplr_decode":
         print(json.dumps(bench_dplr_step(torch, la, _lib, max(args.steps, 500))))
+        return
+    if args.workload == "dplr_train":
+        print(json.dumps(bench_dplr_train(torch, la, _lib, min(args.steps, 5), min(args.warmup, 2))))
         return
     if args.workload == "conv":
         print(json.dumps(bench_conv(torch, la, _lib, args.steps, args.warmup)))

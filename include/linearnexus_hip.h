@@ -200,7 +200,7 @@ int lnx_conv1d_packed_bwd(const void* x, const float* weight, const float* bias,
  * q, k, a, b [B,H,T,dk] and v, o [B,H,T,dv] in `dtype` / `o_dtype`; gk [B,H,T,dk] and the states [B,H,dk,dv] fp32.
  * lnx_dplr_recurrent_fwd replaces dplr_delta_rule_recurrent (rwkv7.py:114-213; initial_state NULL = zeros),
  * lnx_dplr_step replaces dplr_delta_rule_step (rwkv7.py:216-265; token tensors [B,H,d], T ignored, the state is
- * updated in place when final_state == initial_state).  dk in {8,16,32,64,128,256}, dv a multiple of 4.
+ * updated in place when final_state == initial_state).  dk in {8,16,32,64,128}, dv a multiple of 4.
  */
 typedef struct lnx_dplr_args {
   int32_t B, H, T, dk, dv;
@@ -219,6 +219,33 @@ typedef struct lnx_dplr_args {
 } lnx_dplr_args;
 int lnx_dplr_recurrent_fwd(const lnx_dplr_args* a, void* hip_stream);
 int lnx_dplr_step(const lnx_dplr_args* a, void* hip_stream);
+
+/*
+ * Backward pass of lnx_dplr_recurrent_fwd: the gradients of <o, d_o> + <final state, d_final_state>, what jax.grad of
+ * the reference's scan returns (the reference has no backward code of its own: its blocks train through autodiff of
+ * dplr_delta_rule_recurrent, rwkv7.py:148-213).  `fwd` holds the forward call's inputs (its o and final_state are not
+ * read); d_o [B,H,T,dv] in fwd.o_dtype; d_final_state [B,H,dk,dv] fp32 or NULL (zero).  Outputs, all fp32: dq, dk,
+ * da, db, dgk [B,H,T,dk], dv [B,H,T,dv], d_initial_state [B,H,dk,dv] (may be NULL).  The states the tokens start from
+ * are recomputed from checkpoints every 64 tokens kept in a caller-owned workspace of
+ * lnx_dplr_recurrent_bwd_workspace_bytes bytes.  dk in {8,16,32,64,128}, dv a multiple of 4, at most 256.  No
+ * atomics: the result is the same from run to run.
+ */
+typedef struct lnx_dplr_bwd_args {
+  lnx_dplr_args fwd;
+  const void* d_o;
+  const float* d_final_state;
+  float* dq;
+  float* dk;
+  float* dv;
+  float* da;
+  float* db;
+  float* dgk;
+  float* d_initial_state;
+  void* workspace;
+  uint64_t workspace_bytes;
+} lnx_dplr_bwd_args;
+uint64_t lnx_dplr_recurrent_bwd_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t dk, int32_t dv);
+int lnx_dplr_recurrent_bwd(const lnx_dplr_bwd_args* a, void* hip_stream);
 
 /*
  * RMSNorm with an optional sigmoid gate over the rows of [rows, d] matrices, the output epilogue of the reference's

@@ -17,7 +17,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
     "lnx_chunk_workspace_bytes", "lnx_chunk_fuses_l2norm", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
-    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_conv1d_cache_bwd", "lnx_conv1d_packed_fwd", "lnx_conv1d_packed_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
+    "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_conv1d_cache_bwd", "lnx_conv1d_packed_fwd", "lnx_conv1d_packed_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_dplr_recurrent_bwd", "lnx_dplr_recurrent_bwd_workspace_bytes", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
     "lnx_gdn_gate_fwd", "lnx_gdn_gate_bwd", "lnx_gdn_gate_bwd_workspace_bytes", "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
     "lnx_profile_enable", "lnx_profile_read",
 )
@@ -49,6 +49,16 @@ class DplrArgs(C.Structure):
         ("dtype", C.c_int32), ("o_dtype", C.c_int32), ("scale", C.c_float),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("a", C.c_void_p), ("b", C.c_void_p),
         ("gk", C.c_void_p), ("initial_state", C.c_void_p), ("o", C.c_void_p), ("final_state", C.c_void_p),
+    ]
+
+
+class DplrBwdArgs(C.Structure):
+    """Mirror of ``struct lnx_dplr_bwd_args``."""
+
+    _fields_ = [
+        ("fwd", DplrArgs), ("d_o", C.c_void_p), ("d_final_state", C.c_void_p),
+        ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p), ("da", C.c_void_p), ("db", C.c_void_p),
+        ("dgk", C.c_void_p), ("d_initial_state", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
     ]
 
 
@@ -118,6 +128,10 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(DplrArgs), C.c_void_p]
+    lib.lnx_dplr_recurrent_bwd.restype = C.c_int
+    lib.lnx_dplr_recurrent_bwd.argtypes = [C.POINTER(DplrBwdArgs), C.c_void_p]
+    lib.lnx_dplr_recurrent_bwd_workspace_bytes.restype = C.c_uint64
+    lib.lnx_dplr_recurrent_bwd_workspace_bytes.argtypes = [C.c_int32] * 5
     lib.lnx_profile_enable.restype = C.c_int
     lib.lnx_profile_enable.argtypes = [C.c_int]
     lib.lnx_profile_read.restype = C.c_int

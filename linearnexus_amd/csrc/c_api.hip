@@ -20,7 +20,7 @@ int lnx_set_error(int code, const char* fmt, ...) {
 }
 
 extern "C" const char* lnx_last_error(void) { return g_error; }
-extern "C" int lnx_abi_version(void) { return 6; }
+extern "C" int lnx_abi_version(void) { return 7; }
 
 // ---- optional per-kernel timing with HIP events on the caller's stream.  Process-wide (one
 // mutex-guarded list) because a framework may run the backward entry point on another thread. ----

@@ -33,6 +33,11 @@ template <typename T> __device__ __forceinline__ T from_f32(float x);
 template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
 
+// Four consecutive elements as they lie in memory: what a prefetch keeps in registers until the value is used.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef floatx4 V; };
+template <> struct Vec4<bf16_t> { typedef bf16x4 V; };
+
 // Loads 4 consecutive elements as fp32.
 __device__ __forceinline__ floatx4 load4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
 __device__ __forceinline__ floatx4 load4(const bf16_t* p) {
@@ -72,7 +77,11 @@ __device__ __forceinline__ float quad_sum(float x) {
 }
 
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, LNX_WAVE);
+  // inside a row of 16 lanes with DPP (no LDS crossbar): quads, the two quads of a half row, the two half rows
+  x = quad_sum(x);
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x141, 0xF, 0xF, true));  // row_half_mirror: lane i <-> 7 - i
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x128, 0xF, 0xF, true));  // row_ror:8 = lane ^ 8
+  x += __shfl_xor(x, 16, LNX_WAVE);
+  x += __shfl_xor(x, 32, LNX_WAVE);
   return x;
 }

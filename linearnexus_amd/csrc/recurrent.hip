@@ -38,7 +38,10 @@ template <int DK> struct Lanes {
 // Reduces over the 8 row groups (lane bits 3..5); all lanes get the column totals.
 __device__ __forceinline__ floatx4 rowgroup_sum(floatx4 x) {
 #pragma unroll
-  for (int m = 8; m <= 32; m <<= 1) {
+  for (int c = 0; c < 4; ++c)
+    x[c] += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x[c]), 0x128, 0xF, 0xF, true));  // row_ror:8 = lane ^ 8
+#pragma unroll
+  for (int m = 16; m <= 32; m <<= 1) {
     x[0] += __shfl_xor(x[0], m, LNX_WAVE);
     x[1] += __shfl_xor(x[1], m, LNX_WAVE);
     x[2] += __shfl_xor(x[2], m, LNX_WAVE);
@@ -52,43 +55,63 @@ __device__ __forceinline__ void store_o4(void* o, int64_t idx, floatx4 x, int o_
   else store4(reinterpret_cast<float*>(o) + idx, x);
 }
 
+// One q/k row pair (and the gate row of a vector gate) in the registers of a wavefront, as loaded: the scan fetches a
+// token's rows one token ahead, and a conversion here would make the fetch wait for its own loads.
+template <typename T, int DK, int GATE> struct QkRegs {
+  static constexpr int EPL = Lanes<DK>::EPL;
+  T k[EPL], q[EPL];
+  float g[EPL];
+  __device__ __forceinline__ void fetch(const T* qp, const T* kp, const float* gp, int lane) {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const int idx = min(lane + 64 * e, DK - 1);  // lanes past the row repeat its last element and drop it in commit
+      k[e] = kp[idx];
+      q[e] = qp[idx];
+      if (GATE == LNX_GATE_VECTOR) g[e] = gp[idx];
+    }
+  }
+  // Normalises / scales the rows and leaves k^, q~ (and exp(g) for a vector gate) in `sm` ([3][DK] floats).  Returns <q~, k^>.
+  __device__ __forceinline__ float commit(float* sm, int lane, float scale, int l2norm) const {
+    float kv[EPL], qv[EPL];
+    float ksq = 0.f, qsq = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const bool ok = lane + 64 * e < DK;
+      kv[e] = ok ? to_f32(k[e]) : 0.f;
+      qv[e] = ok ? to_f32(q[e]) : 0.f;
+      ksq += kv[e] * kv[e];
+      qsq += qv[e] * qv[e];
+    }
+    float kmul = 1.f, qmul = scale;
+    if (l2norm) {
+      kmul = 1.f / (sqrtf(wave_sum(ksq)) + LNX_L2_EPS);
+      qmul = scale / (sqrtf(wave_sum(qsq)) + LNX_L2_EPS);
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const int idx = lane + 64 * e;
+      kv[e] *= kmul;
+      qv[e] *= qmul;
+      dot += kv[e] * qv[e];
+      if (idx < DK) {
+        sm[idx] = kv[e];
+        sm[DK + idx] = qv[e];
+        if (GATE == LNX_GATE_VECTOR) sm[2 * DK + idx] = expf(g[e]);
+      }
+    }
+    return wave_sum(dot);
+  }
+};
+
 // Loads one q/k row pair with a full wavefront, normalises/scales it and leaves
 // k^, q~ (and exp(g) for a vector gate) in `sm` ([3][DK] floats).  Returns <q~, k^>.
 template <typename T, int DK, int GATE>
 __device__ __forceinline__ float stage_qk(const T* qp, const T* kp, const float* gp, float* sm,
                                           int lane, float scale, int l2norm) {
-  constexpr int EPL = Lanes<DK>::EPL;
-  float kv[EPL], qv[EPL], gv[EPL];
-  float ksq = 0.f, qsq = 0.f;
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    const int idx = lane + 64 * e;
-    const bool ok = idx < DK;
-    kv[e] = ok ? to_f32(kp[idx]) : 0.f;
-    qv[e] = ok ? to_f32(qp[idx]) : 0.f;
-    gv[e] = (GATE == LNX_GATE_VECTOR && ok) ? gp[idx] : 0.f;
-    ksq += kv[e] * kv[e];
-    qsq += qv[e] * qv[e];
-  }
-  float kmul = 1.f, qmul = scale;
-  if (l2norm) {
-    kmul = 1.f / (sqrtf(wave_sum(ksq)) + LNX_L2_EPS);
-    qmul = scale / (sqrtf(wave_sum(qsq)) + LNX_L2_EPS);
-  }
-  float dot = 0.f;
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    const int idx = lane + 64 * e;
-    kv[e] *= kmul;
-    qv[e] *= qmul;
-    dot += kv[e] * qv[e];
-    if (idx < DK) {
-      sm[idx] = kv[e];
-      sm[DK + idx] = qv[e];
-      if (GATE == LNX_GATE_VECTOR) sm[2 * DK + idx] = expf(gv[e]);
-    }
-  }
-  return wave_sum(dot);
+  QkRegs<T, DK, GATE> r;
+  r.fetch(qp, kp, gp, lane);
+  return r.commit(sm, lane, scale, l2norm);
 }
 
 // One token applied to the register slab S[RPL] (rows row0.., columns of this lane).
@@ -187,17 +210,32 @@ __global__ __launch_bounds__(64) void recurrent_fwd_kernel(TokenParams p) {
   const float* gb = nullptr;
   if (GATE == LNX_GATE_SCALAR) gb = p.g + tok0;
   if (GATE == LNX_GATE_VECTOR) gb = p.g + tok0 * DK;
+  // The rows of token t + 1 are fetched (raw, nothing converted) while token t is applied, and the barriers order LDS
+  // only: with __syncthreads() or a conversion at the fetch every token would wait for a round trip to memory.
+  struct Ahead {
+    QkRegs<T, DK, GATE> qk;
+    typename Vec4<T>::V v;
+    float beta, g;
+  };
+  auto fetch = [&](Ahead& r, int t) {
+    const int64_t tt = (int64_t)min(t, t1 - 1) * ts;  // past the end: the last token again, never used
+    r.qk.fetch(qb + tt * DK, kb + tt * DK, (GATE == LNX_GATE_VECTOR) ? gb + tt * DK : nullptr, lane);
+    r.v = *reinterpret_cast<const typename Vec4<T>::V*>(vb + tt * p.dv);
+    r.beta = betab[tt];
+    r.g = (GATE == LNX_GATE_SCALAR) ? gb[tt] : 0.f;
+  };
+  Ahead cur, nxt;
+  if (t0 < t1) fetch(cur, t0);
   for (int t = t0; t < t1; ++t) {
-    const int64_t tt = t * ts;
-    const float* gp = (GATE == LNX_GATE_VECTOR) ? gb + tt * DK : nullptr;
-    const floatx4 v4 = load4(vb + tt * p.dv);
-    const float beta = betab[tt];
-    const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(gb[tt]) : 1.f;
-    __syncthreads();  // previous token's reads of sm are done
-    const float qk = stage_qk<T, DK, GATE>(qb + tt * DK, kb + tt * DK, gp, sm, lane, p.scale, p.l2norm);
-    __syncthreads();
-    const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, beta, v4, qk);
-    if ((lane >> 3) == 0 && active) store_o4(p.o, (tok0 + tt) * p.dv + col0, o4, p.o_dtype);
+    fetch(nxt, t + 1);
+    lds_barrier();  // previous token's reads of sm are done
+    const float qk = cur.qk.commit(sm, lane, p.scale, p.l2norm);
+    lds_barrier();
+    const float alpha_s = (GATE == LNX_GATE_SCALAR) ? expf(cur.g) : 1.f;
+    const floatx4 v4 = {to_f32(cur.v[0]), to_f32(cur.v[1]), to_f32(cur.v[2]), to_f32(cur.v[3])};
+    const floatx4 o4 = apply_token<DK, GATE>(S, sm, row0, alpha_s, cur.beta, v4, qk);
+    if ((lane >> 3) == 0 && active) store_o4(p.o, (tok0 + (int64_t)t * ts) * p.dv + col0, o4, p.o_dtype);
+    cur = nxt;
   }
   if (active) {
 #pragma unroll

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() == 6
+    assert lib.lnx_abi_version() == 7
 
 
 def test_struct_layout_matches_header():
@@ -64,6 +64,13 @@ def test_argument_validation_without_gpu():
     assert lib.lnx_dplr_step(d, None) == -2 and lib.lnx_dplr_recurrent_fwd(d, None) == -2
     d.B, d.H, d.T, d.dk, d.dv = 1, 1, 1, 64, 64
     assert lib.lnx_dplr_step(d, None) == -1 and lib.lnx_dplr_recurrent_fwd(d, None) == -1
+    g = _lib.DplrBwdArgs()
+    assert lib.lnx_dplr_recurrent_bwd(None, None) == -1 and lib.lnx_dplr_recurrent_bwd(g, None) == -2
+    g.fwd = d
+    g.fwd.T = 4
+    assert lib.lnx_dplr_recurrent_bwd(g, None) == -1 and b"required" in lib.lnx_last_error()
+    assert lib.lnx_dplr_recurrent_bwd_workspace_bytes(2, 3, 130, 64, 64) == 2 * 3 * (3 + 64) * 64 * 64 * 4
+    assert lib.lnx_dplr_recurrent_bwd_workspace_bytes(0, 3, 130, 64, 64) == 0
     assert lib.lnx_conv1d_fwd(None, None, None, None, None, None, 1, 4, 16, 5, 0, 0, None) == -2  # K > 4
     assert lib.lnx_conv1d_fwd(None, None, None, None, None, None, 1, 4, 18, 4, 0, 0, None) == -2  # D % 4
     assert lib.lnx_conv1d_bwd(None, None, None, None, None, None, None, None, 1, 4, 16, 4, 0, 0, None) == -1
