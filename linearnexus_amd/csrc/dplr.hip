@@ -250,6 +250,8 @@ __global__ __launch_bounds__(512) void dplr_bwd_kernel(DplrBwdParams p) {
   constexpr int RPL = DK / 8;
   __shared__ float sm[5 * DK];          // q~, k, a, b, w of the current token
   __shared__ float red[8][5][DK];       // per wave: its share of dq / scale, dk, db, dgk / w, da
+  constexpr int NB = 8;                 // tokens whose five gradient rows wait in LDS for one coalesced write
+  __shared__ __align__(16) float outb[5][NB][DK];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nthr = blockDim.x;
   const int64_t bh = blockIdx.x;
   const int col0 = wave * 32 + (lane & 7) * 4;
@@ -366,9 +368,34 @@ __global__ __launch_bounds__(512) void dplr_bwd_kernel(DplrBwdParams p) {
     load_do(dr, t0 + len - 1);
 #pragma unroll
     for (int i = 0; i < RPL; ++i) hp[i] = load_state(tape + (len - 1) * ssz + slab + (int64_t)i * p.dv);
+    // Two barriers per token.  Between them: the sums over the waves of the token before (its shares are complete at the
+    // first barrier) go to the output buffer while wave 0 writes this token's vectors.
+    int pend = -1;  // position in the segment of the token whose shares wait in `red`
+    auto reduce_pending = [&]() {
+      if (pend < 0) return;
+      const int nw = nthr >> 6, slot = (len - 1 - pend) % NB;
+      for (int idx = tid; idx < 5 * DK; idx += nthr) {
+        const int x = idx / DK, kk = idx - x * DK;
+        float sum = 0.f;
+        for (int w_ = 0; w_ < nw; ++w_) sum += red[w_][x][kk];
+        outb[x][NB - 1 - slot][kk] = x == 0 ? sum * p.scale : sum;  // rows in increasing token order
+      }
+    };
+    auto flush = [&](int tfirst, int rows) {  // tokens tfirst .. tfirst + rows - 1 lie in buffer rows NB - rows .. NB - 1
+      for (int idx = tid; idx < 5 * rows * (DK / 4); idx += nthr) {
+        const int x = idx / (rows * (DK / 4)), rem = idx - x * rows * (DK / 4), j = rem / (DK / 4), c4 = (rem - j * (DK / 4)) * 4;
+        float* dst = x == 0 ? p.dq : x == 1 ? p.dk : x == 2 ? p.db : x == 3 ? p.dgk : p.da;
+        store4(dst + (tok0 + tfirst + j) * DK + c4, load4(&outb[x][NB - rows + j][c4]));
+      }
+    };
     for (int tl = len - 1; tl >= 0; --tl) {
       const int t = t0 + tl;
-      stage(tl > 0 ? t - 1 : -1);
+      lds_barrier();
+      reduce_pending();
+      if (wave == 0) tr.template commit<false>(sm, lane, p.scale);
+      fetch_tok(tl > 0 ? t - 1 : -1);
+      lds_barrier();
+      if (pend >= 0 && (len - 1 - pend) % NB == NB - 1) flush(t0 + pend, NB);
       const int tn = max(tl - 1, 0);
       constexpr int NPRE = DK <= 64 ? RPL : 1;  // at dk = 128 a second set of state registers would spill: the tape is read in place
       floatx4 hn[NPRE];
@@ -408,26 +435,21 @@ __global__ __launch_bounds__(512) void dplr_bwd_kernel(DplrBwdParams p) {
           red[wave][0][row0 + i] = sq;
           red[wave][1][row0 + i] = sk;
           red[wave][2][row0 + i] = sb;
-          red[wave][3][row0 + i] = sw;
+          red[wave][3][row0 + i] = sw * sm[4 * DK + row0 + i];
           red[wave][4][row0 + i] = pa;
         }
         D[i] = D[i] * sm[4 * DK + row0 + i] + du * sm[2 * DK + row0 + i];  // gradient of the state before the token
       }
-      lds_barrier();
-      const int nw = nthr >> 6;
-      for (int idx = tid; idx < 5 * DK; idx += nthr) {
-        const int x = idx / DK, kk = idx - x * DK;
-        float sum = 0.f;
-        for (int w_ = 0; w_ < nw; ++w_) sum += red[w_][x][kk];
-        float* dst = x == 0 ? p.dq : x == 1 ? p.dk : x == 2 ? p.db : x == 3 ? p.dgk : p.da;
-        const float f = x == 0 ? p.scale : x == 3 ? sm[4 * DK + kk] : 1.f;
-        dst[(tok0 + t) * DK + kk] = sum * f;
-      }
+      pend = tl;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) hp[i] = DK <= 64 ? hn[DK <= 64 ? i : 0] : (load_state(tape + tn * ssz + slab + (int64_t)i * p.dv));
       vr = vnr;
       dr = dnr;
     }
+    lds_barrier();
+    reduce_pending();
+    lds_barrier();
+    flush(t0, (len - 1) % NB + 1);
   }
   if (p.ds0 && active) {
 #pragma unroll
