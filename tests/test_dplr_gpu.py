@@ -204,3 +204,18 @@ def test_backward_through_the_c_abi_rejects_bad_arguments():
     g.workspace, g.workspace_bytes = ws.data_ptr(), ws.numel()
     assert lib.lnx_dplr_recurrent_bwd(g, None) == -2          # dk = 12
     assert lib.lnx_dplr_recurrent_bwd_workspace_bytes(2, 3, 130, 64, 64) == 2 * 3 * (3 + 64) * 64 * 64 * 4
+
+
+def test_gradients_of_empty_scans():
+    """No tokens: the state passes through and so does its gradient; no batch rows: empty gradients."""
+    import linearnexus_amd as la
+    e = torch.zeros(1, 2, 0, 16, device=DEV, requires_grad=True)
+    h0 = torch.randn(1, 2, 16, 16, device=DEV, requires_grad=True)
+    o, h = la.dplr_delta_rule_recurrent(e, e, e, e, e, e, initial_state=h0)
+    dS = torch.randn_like(h)
+    (h * dS).sum().backward()
+    assert o.shape == (1, 2, 0, 16) and torch.equal(h0.grad, dS) and e.grad.shape == e.shape
+    z = torch.zeros(0, 2, 5, 16, device=DEV, requires_grad=True)
+    o, h = la.dplr_delta_rule_recurrent(z, z, z, z, z, z)
+    (o.sum() + h.sum()).backward()
+    assert z.grad.shape == z.shape
