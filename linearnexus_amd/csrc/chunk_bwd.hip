@@ -811,7 +811,11 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   // for the epilogue (other gates; 4-byte inputs with dk <= 128 read K again instead, so that two workgroups fit a CU)
   static constexpr bool KEEP_K = GATE != LNX_GATE_VECTOR && (sizeof(T) == 2 || DK > 128);
   static constexpr int ntile = (GATE == LNX_GATE_VECTOR) ? 5 : KEEP_K ? 4 + (DK / 64 - 1) : 4;
-  static constexpr size_t bytes = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
+  // vector gate, 2-byte inputs, dk = 128: the second half's dBw fragments wait in LDS while the first half's pair sums
+  // run (one value per thread and fragment element; in registers they went to scratch memory)
+  static constexpr bool STASH = GATE == LNX_GATE_VECTOR && sizeof(T) == 2 && DK == 128;
+  static constexpr size_t stash_off = sizeof(T) * ntile * kTile + sizeof(float) * nfloat;
+  static constexpr size_t bytes = stash_off + (STASH ? sizeof(float) * 16 * 256 : 0);
 };
 
 template <typename T, int DK, int GATE>
@@ -959,6 +963,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
       sR[i * LNX_LDA + j] = (i > j) ? -aM[0][0][e] : 0.f;  // dA
     }
+    float* sStash = reinterpret_cast<float*>(smem + L::stash_off);
+    if constexpr (L::STASH) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sStash[e * 256 + tid] = aBw[NKS - 1][0][0][e];
+    }
     lds_barrier();
     {  // dbeta += sum_j dA_ij X_ij, then dX = beta_i dA_ij in place; thread = (row, quarter of the columns)
       const int r = tid >> 2, j0 = (tid & 3) * 16;
@@ -988,7 +997,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         }
       };
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {  // all global reads of the half first (2-byte inputs: the partial sums after the pair terms)
+      for (int it = 0; it < 4; ++it) {  // all global reads of the half first
         const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
         up[it] = load4(Gg + r * DK + ch0 + c);
       }
@@ -1000,15 +1009,23 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         store4(sGc + r * LDF + c, up[it]);
       }
       lds_barrier();
+      if (L::STASH && h == NKS - 1) {  // out = e^G dBw
 #pragma unroll
-      for (int u = 0; u < NKS; ++u)
-        if (u == h) {  // out = e^G dBw
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
-            sOut[r * LDF + c] = aBw[u][0][0][e] * __expf(sGc[r * LDF + c]);
-          }
+        for (int e = 0; e < 16; ++e) {
+          const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+          sOut[r * LDF + c] = sStash[e * 256 + tid] * __expf(sGc[r * LDF + c]);
         }
+      } else {
+#pragma unroll
+        for (int u = 0; u < NKS; ++u)
+          if (u == h) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int r = 32 * wi + frag_row(e, lane), c = 32 * wj + frag_col(lane);
+              sOut[r * LDF + c] = aBw[u][0][0][e] * __expf(sGc[r * LDF + c]);
+            }
+          }
+      }
       lds_barrier();
       {  // dbeta += <e^G dBw, k>;  out = beta e^G dBw; thread = (row, quarter of the channels)
         const int r = tid >> 2, q0 = (tid & 3) * 16;
