@@ -686,8 +686,15 @@ template <typename T, int DK, int BVW = 64> struct ScanSmem {
   static constexpr int kW = 64 * LDK, kKT = SHARE ? 0 : 64 * LDK, kU = 64 * (BV + PAD), kST = BV * LDK, kDT = BV * LDC;
   static constexpr int kQ = (FUSE_OUT && !SHAREQ) ? 64 * LDK : 0, kP = FUSE_OUT ? 64 * LDC : 0;
   static constexpr int kG = DK > 128 ? DK : 128;  // gate values: 64 tokens (scalar gate) or dk channels (vector gate)
-  static constexpr size_t bytes = sizeof(T) * (kW + kKT + kU + kST + kDT + kQ + kP) +
-                                  (FUSE_OUT ? sizeof(bf16_t) * 64 * LDO : 0) + sizeof(float) * (kG + 4);
+  // 32-column slabs of 2-byte inputs with dk = 128: every input tile twice, so that the movers write chunk n + 1
+  // while chunk n is being read
+  static constexpr bool DB = sizeof(T) == 2 && DK == 128 && BV == 32;
+  static constexpr int NB = DB ? 2 : 1;
+  // staging tile of the outputs: bf16 [64][LDO]; double-buffered form: also fp32 [64][LDOF], so that every global store
+  // of the kernel is a mover's
+  static constexpr int LDOF = BV + 4;
+  static constexpr size_t o_bytes = !FUSE_OUT ? 0 : DB ? sizeof(float) * 64 * LDOF : sizeof(bf16_t) * 64 * LDO;
+  static constexpr size_t bytes = sizeof(T) * (NB * (kW + kKT + kU + kQ + kP) + kST + kDT) + o_bytes + sizeof(float) * NB * (kG + 4);
 };
 
 template <typename T, int DK, int GATE, int BVW = 64>
@@ -702,16 +709,20 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   constexpr int NT = (DK >= 128) ? CT : 1;
   static_assert(BV == 64 || (BV == 32 && DK >= 128), "32-column slabs: the wave's state tile must be a full row tile");
   extern __shared__ __align__(16) char smem[];
+  constexpr int NB = L::NB;  // buffers per input tile (the second of a pair follows the first)
   T* sW = reinterpret_cast<T*>(smem);
-  T* sK = L::SHARE ? sW : sW + L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
-  T* sU = sW + L::kW + L::kKT;         // U rows [token][v], replaced by D
-  T* sST = sU + L::kU;
+  T* sK = L::SHARE ? sW : sW + NB * L::kW;  // K rows [token][dk] (vector gate: K * e^{G_last - G})
+  T* sU = sW + NB * (L::kW + L::kKT);       // U rows [token][v], replaced by D
+  T* sST = sU + NB * L::kU;
   T* sDT = sST + L::kST;
   T* sQ = L::SHAREQ ? sW : sDT + L::kDT;  // fused output only: Q rows (vector gate: scale Q e^G), P, output staging
-  T* sP = sDT + L::kDT + L::kQ;
-  bf16_t* sO = reinterpret_cast<bf16_t*>(sP + L::kP);
-  float* sG = reinterpret_cast<float*>(sO + (FUSE ? 64 * LDO : 0));
-  int* sMeta = reinterpret_cast<int*>(sG + L::kG);  // first token and length of the chunk whose tiles are in LDS
+  T* sP = sDT + L::kDT + NB * L::kQ;
+  bf16_t* sO = reinterpret_cast<bf16_t*>(sP + NB * L::kP);
+  float* sOf = reinterpret_cast<float*>(sO);  // double-buffered form with fp32 outputs
+  float* sG = reinterpret_cast<float*>(reinterpret_cast<char*>(sO) + L::o_bytes);  // [NB][kG + 4]: gate values, then first token and
+                                                                     // length of the chunk whose tiles are in the buffer
+  int* sMeta = reinterpret_cast<int*>(sG + L::kG);
+  constexpr int kGM = L::kG + 4;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -872,20 +883,21 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, R.len, mt);
         R.P.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       }
-      if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = ws_ptr<float>(p, p.off.G)[slot * 64 + mt];
-      if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];  // G_last[c]
+      // every thread loads (clamped index): a load behind a branch cannot be counted
+      if (GATE == LNX_GATE_SCALAR) R.G = ws_ptr<float>(p, p.off.G)[slot * 64 + (mt & 63)];
+      if (GATE == LNX_GATE_VECTOR) R.G = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + min(mt, DK - 1)];  // G_last[c]
     };
-    auto commit_rest = [&](const Tiles& R) {
-      R.K.store(sK, LDK, mt);
-      R.U.store(sU, LDU, mt);
+    auto commit_rest = [&](const Tiles& R, int pb) {
+      R.K.store(sK + pb * L::kKT, LDK, mt);
+      R.U.store(sU + pb * L::kU, LDU, mt);
       if (FUSE) {
-        R.Q.store(sQ, LDK, mt);
-        R.P.store(sP, LDC, mt);
+        R.Q.store(sQ + pb * L::kQ, LDK, mt);
+        R.P.store(sP + pb * L::kP, LDC, mt);
       }
-      if (mt < L::kG) sG[mt] = R.G;
+      if (mt < L::kG) sG[pb * kGM + mt] = R.G;
       if (mt == 0) {
-        sMeta[0] = R.tok0;
-        sMeta[1] = R.len;
+        sMeta[pb * kGM] = R.tok0;
+        sMeta[pb * kGM + 1] = R.len;
       }
     };
     // cur: chunk n (in LDS already), nxt: chunk n + 1.  `steady` (a std::bool_constant) says that chunks n + 1 and
@@ -896,23 +908,50 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       constexpr bool STEADY = decltype(steady)::value;
       const int64_t slot = (int64_t)row * N + n;
       const int tok0 = cur.tok0, len = cur.len;
+      if constexpr (L::DB) {
+        // Chunk n + 1 goes to the buffers chunk n - 1 was read from, so no tile write waits for a reader, and every
+        // global store of the kernel is issued here: stores issued by the compute waves queued behind the movers'
+        // loads and held the chain up.  Loads in the first phase, the chunk's state and D and the next chunk's tile
+        // writes in the second (the compute waves' longest), the outputs in the third.
+        const int pb = (n - c0) & 1;
+        if (STEADY || n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
+        lds_barrier();  // B2
+        if (p.save) {
+          unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
+          unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU + pb * L::kU, LDU, 64, mt);
+        }
+        if (STEADY || n + 1 < c1) {
+          nxt.W.store(sW + (pb ^ 1) * L::kW, LDK, mt);
+          commit_rest(nxt, pb ^ 1);
+        }
+        lds_barrier();  // B3
+        if (p.o) {
+          if (p.o_dtype == LNX_BF16)
+            unstage_tile_checked<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
+                                                 (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
+          else
+            unstage_tile_checked<float, 64, BV>(reinterpret_cast<float*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
+                                                (int64_t)p.geom.ts * p.dv, sOf, L::LDOF, len, mt);
+        }
+        lds_barrier();  // B1 of the next chunk
+        return;
+      }
       if (STEADY || n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
       lds_barrier();  // B2
       if (STEADY || n + 1 < c1) nxt.W.store(sW, LDK, mt);
       if (p.save) unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU, LDU, 64, mt);
       lds_barrier();  // B3
-      // the output rows first: the next fetch recycles the registers these stores read, which the compiler
-      // protects with a wait for the stores -- the tile commits in between give them time to complete
+      // the output rows first, the tile commits behind them
       if (FUSE && p.o_dtype == LNX_BF16 && p.o)
         unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0,
                                      (int64_t)p.geom.ts * p.dv, sO, LDO, len, mt);
-      if (STEADY || n + 1 < c1) commit_rest(nxt);
+      if (STEADY || n + 1 < c1) commit_rest(nxt, 0);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
       fetch(ta, c0);
       ta.W.store(sW, LDK, mt);
-      commit_rest(ta);
+      commit_rest(ta, 0);
     }
     if (AHEAD == 2 && c0 + 1 < c1) fetch(tb, c0 + 1);
     lds_barrier();  // B1 of the first chunk
@@ -956,29 +995,37 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
   if (c0 < c1) frag_store_t<T, RT, NT>(S, sST + scol * LDK + srow, LDK, lane);
   lds_barrier();  // B1 of the first chunk
   for (int n = c0; n < c1; ++n) {
+    const int pb = L::DB ? (n - c0) & 1 : 0;  // buffer of this chunk's tiles
+    const T* cW = sW + pb * L::kW;
+    const T* cK = sK + pb * L::kKT;
+    T* cU = sU + pb * L::kU;
+    const T* cQ = sQ + pb * L::kQ;
+    const T* cP = sP + pb * L::kP;
+    const float* cG = sG + pb * kGM;
+    const int* cMeta = sMeta + pb * kGM;
     // D = U - W S  (one 32x32 tile per wave)
-    const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
+    const float gl = (GATE == LNX_GATE_SCALAR) ? cG[63] : 0.f;
     if (has_tile) {
       floatx16 d[1][1];
       frag_zero(d);
-      mma_nt<T, 1, 1>(d, sW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+      mma_nt<T, 1, 1>(d, cW + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
       // D replaces U in place (all reads first: interleaved with the writes they would be serialised)
       float u[16];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) u[e] = to_f32(sU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
+      for (int e = 0; e < 16; ++e) u[e] = to_f32(cU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)]);
 #pragma unroll
       for (int e = 0; e < 16; ++e) d[0][0][e] = u[e] - d[0][0][e];
 #pragma unroll
       for (int e = 0; e < 16; ++e)
-        sU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)] = from_f32<T>(d[0][0][e]);
+        cU[(32 * wi + frag_row(e, lane)) * LDU + 32 * wj + frag_col(lane)] = from_f32<T>(d[0][0][e]);
       if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f));
+        for (int e = 0; e < 16; ++e) d[0][0][e] *= __expf(fminf(gl - cG[32 * wi + frag_row(e, lane)], 0.f));
       }
       frag_store_t<T, 1, 1>(d, sDT + 32 * wj * LDC + 32 * wi, LDC, lane);
     }
-    // S_n -> workspace (the movers are busy issuing loads in this phase)
-    if (p.save)
+    // S_n -> workspace (the movers are busy issuing loads in this phase; double-buffered form: they do it after B2)
+    if (p.save && !L::DB)
       unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + ((int64_t)row * N + n) * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, tid);
     lds_barrier();  // B2
 
@@ -987,17 +1034,19 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         // o = scale e^G (Q S) + P D for this slab
         floatx16 o[1][1];
         frag_zero(o);
-        mma_nt<T, 1, 1>(o, sQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
+        mma_nt<T, 1, 1>(o, cQ + 32 * wi * LDK, LDK, sST + 32 * wj * LDK, LDK, DK, lane);
         if (GATE != LNX_GATE_VECTOR) {
 #pragma unroll
           for (int e = 0; e < 16; ++e)
-            o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(sG[32 * wi + frag_row(e, lane)]);
+            o[0][0][e] *= (GATE == LNX_GATE_NONE) ? p.scale : p.scale * __expf(cG[32 * wi + frag_row(e, lane)]);
         }
-        mma_x<T, 1, 1, false, true>(o, sP + 32 * wi * LDC, LDC, sU + 32 * wj, LDU, 64, lane);
+        mma_x<T, 1, 1, false, true>(o, cP + 32 * wi * LDC, LDC, cU + 32 * wj, LDU, 64, lane);
         if (p.o_dtype == LNX_BF16) {
           frag_store<bf16_t, 1, 1>(o, sO + 32 * wi * LDO + 32 * wj, LDO, lane);  // the movers write it out
+        } else if (L::DB) {
+          frag_store<float, 1, 1>(o, sOf + 32 * wi * L::LDOF + 32 * wj, L::LDOF, lane);
         } else if (p.o) {
-          const int tok0 = sMeta[0], len = sMeta[1];
+          const int tok0 = cMeta[0], len = cMeta[1];
           frag_store<float, 1, 1>(o, reinterpret_cast<float*>(p.o) + (tok_index(p.geom, row, tok0) + (int64_t)32 * wi * p.geom.ts) * p.dv + v0 + 32 * wj,
                                   (int64_t)p.geom.ts * p.dv, lane, len - 32 * wi);
         }
@@ -1020,9 +1069,9 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
 #pragma unroll
           for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) S[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
+            for (int e = 0; e < 16; ++e) S[i][j][e] *= __expf(cG[srow + 32 * i + frag_row(e, lane)]);
       }
-      mma_x<T, RT, NT, true, false>(S, sK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
+      mma_x<T, RT, NT, true, false>(S, cK + srow, LDK, sDT + scol * LDC, LDC, 64, lane);
     };
     if (L::SHAREQ) {
       update();

@@ -294,6 +294,29 @@ __device__ __forceinline__ void unstage_tile(T* dst, int64_t stride, const T* sr
   }
 }
 
+// The same through a buffer descriptor that covers rows < valid only: the hardware drops the stores past the end, so
+// no store sits behind a branch and a loop that also prefetches can count its memory instructions exactly.
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void unstage_tile_checked(T* dst, int64_t stride, const T* src, int ld, int valid, int tid) {
+  typedef typename Vec16<T>::V V;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int N = Vec16<T>::N, VPR = COLS / N, TOTAL = ROWS * VPR, IT = TOTAL / 256;
+  static_assert(TOTAL % 256 == 0, "whole passes only");
+  const int bytes = valid > 0 ? (int)(valid * stride * (int64_t)sizeof(T)) : 0;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(dst, 0, bytes, 0x00020000);
+  V x[IT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+    x[it] = *reinterpret_cast<const V*>(src + r * ld + c);
+  }
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * N;
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x[it]), rsrc, (int)((r * stride + c) * (int64_t)sizeof(T)), 0, 0);
+  }
+}
+
 // Sums f(e) * acc[i][0][e] over the 32 lanes that share rows, for all 16*MT rows of a wave's
 // fragments at once, by a transpose-reduce (31 shuffles per 32 values instead of 160), then adds
 // the row totals into rows[] (LDS) with one atomic per row and wave.
