@@ -104,8 +104,12 @@ template <typename T, int DK, int BVW = 64> struct BScanCfg {
   // for the dS update) share a tile
   static constexpr bool SHAREK = BV == 64 && ((sizeof(T) == 2 && DK > 128) || (sizeof(T) == 4 && DK == 128));
   static constexpr int nRow = SHARE ? 1 : SHAREK ? 2 : 3;
+  // 32-column slabs of 2-byte inputs with dk = 128: every input tile twice, so that the movers write chunk n - 1
+  // while chunk n is being read
+  static constexpr bool DB = sizeof(T) == 2 && DK == 128 && BV == 32;
+  static constexpr int NB = DB ? 2 : 1;
   // K, Q, W rows [token][dk];  dO, dD slabs [token][BV];  -dD^T [BV][token];  dS^T [BV][dk];  P;  unscaled dO
-  static constexpr size_t bytes = sizeof(T) * (nRow * kRow + 2 * kSlab + kdDT + kdST + kP + kRaw) + sizeof(float) * kG;
+  static constexpr size_t bytes = sizeof(T) * (NB * (nRow * kRow + kSlab + kP + kRaw) + kSlab + kdDT + kdST) + sizeof(float) * NB * kG;
 };
 
 template <typename T, int DK, int GATE, int BVW = 64>
@@ -118,16 +122,17 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   constexpr int NT = (DK >= 128) ? CT : 1;         //   for dk = 64) x NT column tiles
   static_assert(DK >= 128 || BV == 64, "dk = 64 needs a 64-column slab");
   extern __shared__ __align__(16) char smem[];
+  constexpr int NB = L::NB;  // buffers per input tile (the second of a pair follows the first)
   T* sK = reinterpret_cast<T*>(smem);
-  T* sQ = (L::SHARE || L::SHAREK) ? sK : sK + L::kRow;
-  T* sW = L::SHARE ? sK : sQ + L::kRow;
-  T* sdO = sK + L::nRow * L::kRow;
-  T* sdDl = sdO + L::kSlab;
+  T* sQ = (L::SHARE || L::SHAREK) ? sK : sK + NB * L::kRow;
+  T* sW = L::SHARE ? sK : sQ + NB * L::kRow;
+  T* sdO = sK + NB * L::nRow * L::kRow;
+  T* sdDl = sdO + NB * L::kSlab;
   T* sdDT = sdDl + L::kSlab;
   T* sdST = sdDT + L::kdDT;
   T* sP = sdST + L::kdST;   // fused local part only: P [i][j] and the unscaled dO slab
-  T* sdOr = sP + L::kP;
-  float* sG = reinterpret_cast<float*>(sdOr + L::kRaw);
+  T* sdOr = sP + NB * L::kP;
+  float* sG = reinterpret_cast<float*>(sdOr + NB * L::kRaw);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -341,8 +346,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         R.dO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, mt);
         if (FUSE) R.P.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
         else R.dD.load(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, 64, mt);
-        if (GATE == LNX_GATE_SCALAR && mt < 64) R.G = wsp<float>(p, p.off.G)[slot * 64 + mt];
-        if (GATE == LNX_GATE_VECTOR && mt < DK) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + mt];
+        // every thread loads (clamped index): a load behind a branch cannot be counted
+        if (GATE == LNX_GATE_SCALAR) R.G = wsp<float>(p, p.off.G)[slot * 64 + (mt & 63)];
+        if (GATE == LNX_GATE_VECTOR) R.G = wsp<float>(p, p.off.G)[(slot * 64 + 63) * DK + min(mt, DK - 1)];
       }
       if (part < 0 || part == 2) {
         if (GATE == LNX_GATE_VECTOR) R.Q.load(wsp<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
@@ -355,12 +361,12 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         }
       }
     };
-    auto commit_rest = [&](const Tiles& R) {
-      R.Q.store(sQ, LDK, mt);
-      R.W.store(sW, LDK, mt);
+    auto commit_rest = [&](const Tiles& R, int pb) {
+      R.Q.store(sQ + pb * L::kRow, LDK, mt);
+      R.W.store(sW + pb * L::kRow, LDK, mt);
       if (FUSE) {
-        R.P.store(sP, LDC, mt);
-        R.dO.store(sdOr, LDU, mt);
+        R.P.store(sP + pb * L::kP, LDC, mt);
+        R.dO.store(sdOr + pb * L::kRaw, LDU, mt);
       } else {
         R.dD.store(sdDl, LDU, mt);
       }
@@ -373,9 +379,29 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
           for (int e = 0; e < Slab::N; ++e) o[e] = from_f32<T>(to_f32(o[e]) * os);
         }
-        if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + r * LDU + c) = o;
+        if (idx < Slab::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(sdO + pb * L::kSlab + r * LDU + c) = o;
       }
-      if (mt < L::kG) sG[mt] = R.G;
+      if (mt < L::kG) sG[pb * L::kG + mt] = R.G;
+    };
+    // Double-buffered form.  Chunk n - 1 goes to the buffers chunk n + 1 was read from, so no tile write waits for a
+    // reader: loads of chunk n - 2 in the first phase, dS', dD -> workspace and the tile writes in the second.
+    // `steady` (a std::bool_constant): chunks n - 1 and n - 2 exist, so nothing sits behind a branch and the compiler
+    // can count the loads in flight.
+    auto step_db = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
+      constexpr bool STEADY = decltype(steady)::value;
+      const int64_t slot = (int64_t)row * N + n;
+      const int pb = (c1 - 1 - n) & 1;
+      if (STEADY || n - 2 >= c0) fetch(cur, n - 2, -1);  // chunk n's registers are free again
+      if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
+      lds_barrier();  // B2
+      unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
+      unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+      if (STEADY || n - 1 >= c0) {
+        nxt.K.store(sK + (pb ^ 1) * L::kRow, LDK, mt);
+        commit_rest(nxt, pb ^ 1);
+      }
+      lds_barrier();  // B3
+      lds_barrier();  // B1 of the next chunk
     };
     auto step = [&](Tiles& cur, const Tiles& nxt, int n) {  // cur: chunk n (in LDS already), nxt: chunk n - 1
       const int64_t slot = (int64_t)row * N + n;
@@ -389,17 +415,27 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
       lds_barrier();  // B3
       if (more && AHEAD == 2) fetch(cur, n - AHEAD, 2);
-      if (n - 1 >= c0) commit_rest(nxt);
+      if (n - 1 >= c0) commit_rest(nxt, 0);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
       fetch(ta, c1 - 1, -1);
       ta.K.store(sK, LDK, mt);
-      commit_rest(ta);
+      commit_rest(ta, 0);
     }
     if (AHEAD == 2 && c1 - 2 >= c0) fetch(tb, c1 - 2, -1);
     lds_barrier();  // B1 of the first chunk
-    if (AHEAD == 2) {
+    if constexpr (L::DB) {
+      int n = c1 - 1;
+      for (; n - 3 >= c0; n -= 2) {  // chunks n - 2 and n - 3 exist
+        step_db(ta, tb, n, std::true_type{});
+        step_db(tb, ta, n - 1, std::true_type{});
+      }
+      for (; n >= c0; n -= 2) {
+        step_db(ta, tb, n, std::false_type{});
+        if (n - 1 >= c0) step_db(tb, ta, n - 1, std::false_type{});
+      }
+    } else if (AHEAD == 2) {
       for (int n = c1 - 1; n >= c0; n -= 2) {
         step(ta, tb, n);
         if (n - 1 >= c0) step(tb, ta, n - 1);
@@ -433,19 +469,27 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
   if (c0 < c1) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
   lds_barrier();  // B1 of the first chunk
   for (int n = c1 - 1; n >= c0; --n) {
-    const float gl = (GATE == LNX_GATE_SCALAR) ? sG[63] : 0.f;
+    const int pb = L::DB ? (c1 - 1 - n) & 1 : 0;  // buffer of this chunk's tiles
+    const T* cK = sK + pb * L::kRow;
+    const T* cQ = sQ + pb * L::kRow;
+    const T* cW = sW + pb * L::kRow;
+    const T* cdO = sdO + pb * L::kSlab;
+    const T* cP = sP + pb * L::kP;
+    const T* cdOr = sdOr + pb * L::kRaw;
+    const float* cG = sG + pb * L::kG;
+    const float gl = (GATE == LNX_GATE_SCALAR) ? cG[63] : 0.f;
     // dD = dD_loc + r_j (K dS)_j
     if (has_tile) {
       floatx16 d[1][1];
       frag_zero(d);
-      mma_nt<T, 1, 1>(d, sK + 32 * wi * LDK, LDK, sdST + 32 * wj * LDK, LDK, DK, lane);
+      mma_nt<T, 1, 1>(d, cK + 32 * wi * LDK, LDK, sdST + 32 * wj * LDK, LDK, DK, lane);
       // the complete dD replaces the local part in place (all reads first: interleaved with the
       // writes they would be serialised); the movers write it out
       float dl[16];
       if (FUSE) {  // dD_loc[j][v] = sum_i P[i][j] dO[i][v]: both operands contract along the rows of their tiles
         floatx16 l[1][1];
         frag_zero(l);
-        mma_x<T, 1, 1, true, true>(l, sP + 32 * wi, LDC, sdOr + 32 * wj, LDU, 64, lane);
+        mma_x<T, 1, 1, true, true>(l, cP + 32 * wi, LDC, cdOr + 32 * wj, LDU, 64, lane);
 #pragma unroll
         for (int e = 0; e < 16; ++e) dl[e] = l[0][0][e];
       } else {
@@ -454,7 +498,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - sG[32 * wi + frag_row(e, lane)], 0.f)) : 1.f;
+        const float rj = (GATE == LNX_GATE_SCALAR) ? __expf(fminf(gl - cG[32 * wi + frag_row(e, lane)], 0.f)) : 1.f;
         d[0][0][e] = dl[e] + rj * d[0][0][e];
       }
 #pragma unroll
@@ -482,20 +526,20 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 #pragma unroll
         for (int j = 0; j < NT; ++j)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) dS[i][j][e] *= __expf(sG[srow + 32 * i + frag_row(e, lane)]);
+          for (int e = 0; e < 16; ++e) dS[i][j][e] *= __expf(cG[srow + 32 * i + frag_row(e, lane)]);
     }
     if (L::SHAREK) {  // W first: Q is still on its way into the tile it shares with K
-      mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
+      mma_x<T, RT, NT, true, false>(dS, cW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
       lds_barrier();  // B2'
-      mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+      mma_x<T, RT, NT, true, true>(dS, cQ + srow, LDK, cdO + scol, LDU, 64, lane);
     } else {
       if (L::SHARE) lds_barrier();  // B2a: Q has replaced K in the shared tile
-      mma_x<T, RT, NT, true, true>(dS, sQ + srow, LDK, sdO + scol, LDU, 64, lane);
+      mma_x<T, RT, NT, true, true>(dS, cQ + srow, LDK, cdO + scol, LDU, 64, lane);
       if (L::SHARE) {
         lds_barrier();  // B2b
         lds_barrier();  // B2c: W has replaced Q
       }
-      mma_x<T, RT, NT, true, false>(dS, sW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
+      mma_x<T, RT, NT, true, false>(dS, cW + srow, LDK, sdDT + scol * LDC, LDC, 64, lane);
     }
     lds_barrier();  // B3
     if (n > c0) frag_store_t<T, RT, NT>(dS, sdST + scol * LDK + srow, LDK, lane);
