@@ -77,27 +77,30 @@ template <typename T, int DK> struct Prep2Cfg {
   static constexpr size_t r1 = sizeof(float) * 128;  // beta, G
   static constexpr size_t r2 = cmax(mat + scr, 2 * kTile * sizeof(T));
   static constexpr size_t bytes = r0 + r1 + r2;
+  // LITE: the slab tiles, then A inverted in place + merge scratch | beta, G, row factors | P   (31.5 KB, five per CU)
+  static constexpr size_t lite_bytes = mat + scr + sizeof(float) * 256 + kTile * sizeof(T);
 };
 
 // LITE: stop after the inverse and leave Tm itself (row-major) next to Pm and G -- all that the kernels of
 // chunk_direct.hip read; V is not touched.
 template <typename T, int DK, int GATE, bool LITE = false>
-__global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
+__global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdParams p) {
   typedef Prep2Cfg<T, DK> L;
   constexpr int LDC = L::LDC, NKS = DK / 64;
   extern __shared__ __align__(16) char smem[];
-  float* sA = reinterpret_cast<float*>(smem);      // region 0
+  float* sA = reinterpret_cast<float*>(smem);      // region 0 (LITE: over the slab tiles)
   T* sTw = reinterpret_cast<T*>(smem);             //   Tw, Tu once the inverse is done with A
   T* sTu = sTw + L::kTile;
-  float* sBeta = reinterpret_cast<float*>(smem + L::r0);
+  float* sBeta = reinterpret_cast<float*>(smem + (LITE ? L::mat + L::scr : L::r0));
   float* sG = sBeta + 64;
-  char* reg2 = smem + L::r0 + L::r1;               // region 2
+  char* reg2 = LITE ? smem : smem + L::r0 + L::r1;  // region 2
   T* sKa = reinterpret_cast<T*>(reg2);             //   K slab of the first loop, then P
   T* sQa = sKa + L::kTile;                         //   Q slab
   float* sT = reinterpret_cast<float*>(reg2);      //   Tm
   float* sX = reinterpret_cast<float*>(reg2 + L::mat);
   T* sIn = sKa;                                    //   second loop: slab in, result out
   T* sOut = sQa;
+  T* sPt = LITE ? reinterpret_cast<T*>(smem + L::mat + L::scr + sizeof(float) * 256) : sKa;  // P on its way out
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -155,9 +158,8 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
   }
   // LITE: per-row factors 1 / (|x| + eps) (1 without the normalisation), kept behind the slab tiles and written to the
   // workspace for the scans and the chunk-local backward, which scale the rows as they stage them
-  float* sNk = reinterpret_cast<float*>(reg2 + 2 * L::kTile * sizeof(T));
+  float* sNk = sBeta + 128;
   float* sNq = sNk + 64;
-  static_assert(!LITE || 2 * L::kTile * sizeof(T) + 512 <= L::r2, "room for the row factors behind the slab tiles");
   if constexpr (LITE) {
     nk2 = quad_sum(nk2);
     nq2 = quad_sum(nq2);
@@ -190,17 +192,21 @@ __global__ __launch_bounds__(256) void chunk_prepare2_kernel(FwdParams p) {
       sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * fx * ax[0][0][e] : 0.f;
       pe[0][0][e] = (i >= j) ? p.scale * dec * fp * ap[0][0][e] : 0.f;
     }
-    frag_store<T, 1, 1>(pe, sKa + 32 * wi * LDC + 32 * wj, LDC, lane);
+    frag_store<T, 1, 1>(pe, sPt + 32 * wi * LDC + 32 * wj, LDC, lane);
   }
   lds_barrier();
-  unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sKa, LDC, 64, tid);
-  lds_barrier();  // Tm is built over the P tile
-  tri_inverse_64(sA, sT, sX, tid);
+  unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sPt, LDC, 64, tid);
+  if constexpr (LITE) {
+    tri_inverse_64<true>(sA, sA, sX, tid);
+  } else {
+    lds_barrier();  // Tm is built over the P tile
+    tri_inverse_64(sA, sT, sX, tid);
+  }
   if constexpr (LITE) {
     T* Tm = ws_ptr<T>(p, p.off.Tm) + slot * 64 * 64;
     for (int idx = tid; idx < 64 * 16; idx += 256) {
       const int r = idx >> 4, c = (idx & 15) * 4;
-      store4(Tm + r * 64 + c, load4(sT + r * LNX_LDA + c));
+      store4(Tm + r * 64 + c, load4(sA + r * LNX_LDA + c));
     }
     return;
   }
@@ -1340,7 +1346,7 @@ template <int DK, int GATE>
 void launch_prepare_lite(const FwdParams& p, hipStream_t st) {
   auto k = chunk_prepare2_kernel<bf16_t, DK, GATE, true>;
   lnx_profile_mark("chunk_prepare", st);
-  const size_t b = Prep2Cfg<bf16_t, DK>::bytes;
+  const size_t b = Prep2Cfg<bf16_t, DK>::lite_bytes;
   hipLaunchKernelGGL(k, dim3((unsigned)((int64_t)p.geom.rows * p.geom.N)), dim3(256), b, st, p);
 }
 

@@ -379,10 +379,15 @@ __device__ __forceinline__ void mm16_store(float* dst, int ld, floatx4 c, int la
 // matrix (upper triangle zero); `sX` is a [32][36] fp32 scratch.  Must be called by all 256
 // threads.  Diagonal 16x16 blocks by forward substitution, then two levels of block merges
 //   [[L0, 0], [B, L1]]^-1 = [[L0^-1, 0], [-L1^-1 B L0^-1, L1^-1]].
+// In place (sT == sA, INPLACE): A's upper triangle and diagonal must hold zeros; every block of A is read for the last
+// time before the barrier that precedes the write of the same block of Tm.
+template <bool INPLACE = false>
 __device__ __forceinline__ void tri_inverse_64(const float* sA, float* sT, float* sX, int tid) {
   const int wave = tid >> 6, lane = tid & 63;
-  for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) sT[idx] = 0.f;
-  lds_barrier();
+  if (!INPLACE) {
+    for (int idx = tid; idx < 64 * LNX_LDA; idx += 256) sT[idx] = 0.f;
+    lds_barrier();
+  }
   if (lane < 16) {
     const int r0 = 16 * wave, c = lane;
     float d[16];
