@@ -136,6 +136,22 @@ def test_strong_decay_stays_finite(gate):
     assert max_rel(o.float().cpu().numpy(), o_ref) < 2e-2 and max_rel(S.cpu().numpy(), S_ref) < 2e-2
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 200, 128, 128), (1, 3, 330, 128, 64)])
+def test_vector_gate_two_byte_output_is_the_rounded_fp32_output(shape):
+    """The per-channel-gate scan stages its outputs through LDS in either precision; kda_chunkwise only ever asks for
+    fp32 (kda.py:655), so the 2-byte branch is reached through the internal entry: same arithmetic, one rounding at the
+    store, hence bit-equal to the rounded fp32 result.  Ragged lengths: the last chunk's rows past T are not written."""
+    from linearnexus_amd import linear_attn as la_int
+    B, H, T, dk, dv = shape
+    x, dt = _prep(make_inputs(46, B, H, T, dk, dv, gate="vector", with_state=True), True)
+    q, k, v = _t(x["q"], dt), _t(x["k"], dt), _t(x["v"], dt)
+    args = (q, k, v, _t(x["g"]), _t(x["beta"]), None, _t(x["S0"]), 64, False)
+    o32, S32 = la_int._chunk(*args, torch.float32, True, None)
+    o16, S16 = la_int._chunk(*args, torch.bfloat16, True, None)
+    assert o16.dtype == torch.bfloat16 and o32.dtype == torch.float32
+    assert torch.equal(o16, o32.to(torch.bfloat16)) and torch.equal(S16, S32)
+
+
 def test_chunk_equals_recurrent_kernel_at_full_config2_size():
     """Size-independent check at B8 H16 T4096 d128 bf16: the MFMA chunk path and the fp32
     token-by-token kernel (itself checked against the oracle) must agree."""
