@@ -377,15 +377,6 @@ __device__ __forceinline__ void pair_col(float* out, const float* M, const float
 // never leave the lane.  Not STRICT: the diagonal X[i][i] (E = 1) is added to both sums.
 // X [64][LNX_LDA] fp32, G [64][ldf] fp32, b / a [64][ld] bf16, all in LDS; results are per lane, index 4 t + e.
 // ---------------------------------------------------------------------------------------
-__device__ __forceinline__ bf16x4 pack_bf16x4(floatx4 v) {
-  // Two v_cvt_pk_bf16_f32, joined as integers: a four-element conversion is taken apart element by element and
-  // permuted back together.
-  typedef float floatx2_ __attribute__((ext_vector_type(2)));
-  typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
-  const uint2_ r = {__builtin_bit_cast(unsigned, __builtin_convertvector((floatx2_{v[0], v[1]}), bf16x2)),
-                    __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2_{v[2], v[3]}), bf16x2))};
-  return __builtin_bit_cast(bf16x4, r);
-}
 __device__ __forceinline__ floatx4 mfma16_bf16(bf16x4 a, bf16x4 b, floatx4 c) {
   typedef short short4_ __attribute__((ext_vector_type(4)));
   return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_, a), __builtin_bit_cast(short4_, b), c, 0, 0, 0);

@@ -45,11 +45,17 @@ __device__ __forceinline__ floatx4 load4(const bf16_t* p) {
   floatx4 r = {(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
   return r;
 }
-__device__ __forceinline__ void store4(float* p, floatx4 x) { *reinterpret_cast<floatx4*>(p) = x; }
-__device__ __forceinline__ void store4(bf16_t* p, floatx4 x) {
-  bf16x4 t = {(bf16_t)x[0], (bf16_t)x[1], (bf16_t)x[2], (bf16_t)x[3]};
-  *reinterpret_cast<bf16x4*>(p) = t;
+// Four fp32 -> four bf16 (round to nearest even) as two v_cvt_pk_bf16_f32 joined as integers: written as a four-element
+// conversion, or element by element, hipcc takes the vector apart -- one conversion per element and a v_perm_b32 per
+// pair to put them back together, three instructions where one does.
+__device__ __forceinline__ bf16x4 pack_bf16x4(floatx4 v) {
+  typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
+  const uint2_ r = {__builtin_bit_cast(unsigned, __builtin_convertvector((floatx2{v[0], v[1]}), bf16x2)),
+                    __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2{v[2], v[3]}), bf16x2))};
+  return __builtin_bit_cast(bf16x4, r);
 }
+__device__ __forceinline__ void store4(float* p, floatx4 x) { *reinterpret_cast<floatx4*>(p) = x; }
+__device__ __forceinline__ void store4(bf16_t* p, floatx4 x) { *reinterpret_cast<bf16x4*>(p) = pack_bf16x4(x); }
 
 // Token range [seq_first, seq_end) of packed sequence s, read defensively: cu_seqlens lives in device memory where the
 // host cannot check it, so entries are clamped to [0, T] and an end before its start reads as an empty sequence.  A

@@ -51,10 +51,11 @@ template <> struct Mma<bf16_t> {
   // only needs both operands to agree on which contraction index sits in which slot, so the A operand is loaded in
   // that same order ("chain order") with two 8-byte reads instead of one 16-byte read.
   static __device__ __forceinline__ Frag from_acc(const floatx16& c, int h) {
-    Frag b;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) b[t] = (bf16_t)c[8 * h + t];
-    return b;
+    typedef unsigned uint4_ __attribute__((ext_vector_type(4)));
+    typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
+    const uint2_ lo = __builtin_bit_cast(uint2_, pack_bf16x4(floatx4{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]}));
+    const uint2_ hi = __builtin_bit_cast(uint2_, pack_bf16x4(floatx4{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]}));
+    return __builtin_bit_cast(Frag, (uint4_{lo[0], lo[1], hi[0], hi[1]}));
   }
   // A operand in chain order from a [rows][k] tile: p points at (this lane's row, first k of the 16-wide step)
   static __device__ __forceinline__ Frag load_chain(const bf16_t* p, int lane) {
