@@ -152,6 +152,30 @@ def test_backward_packed_sequences(gate):
     check(got, ref, 2e-2)
 
 
+def test_backward_packed_sequences_of_four_to_eight_chunks():
+    """Per-channel gate, packed sequences of 4, 5, 7 and 8 chunks behind one another: the scans take two chunks per loop
+    round once a sequence has four, with an odd or even remainder, and start every sequence on the first of their two
+    tile buffers whatever the parity of its first chunk in the batch."""
+    H, d = 1, 128
+    lens = [256, 300, 448, 512]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    x = make_inputs(58, 1, H, T, d, d, gate="vector", with_grad=True)
+    rng = np.random.default_rng(8)
+    x["S0"] = (rng.standard_normal((4, H, d, d)) * 0.02).astype(np.float32)
+    x["dS"] = (rng.standard_normal((4, H, d, d)) * 0.1).astype(np.float32)
+    x, dt = _prep(x, True)
+    parts = []
+    for s in range(4):
+        a, b = cu[s], cu[s + 1]
+        sl = lambda n: x[n][:, :, a:b]
+        parts.append(delta_rule_adjoint(sl("q"), sl("k"), sl("v"), sl("beta"), sl("dO"), sl("g"), x["dS"][s:s + 1], None,
+                                        x["S0"][s:s + 1], False))
+    ref = {n: np.concatenate([p[n] for p in parts], 2) for n in ("dq", "dk", "dv", "dbeta", "dg")}
+    ref["dS0"] = np.concatenate([p["dS0"] for p in parts], 0)
+    check(gpu_grads(x, "vector", dt, cu=cu), ref, 2e-2)
+
+
 def test_backward_adjoint_identity_at_full_config2_size():
     """Size-independent check at B8 H16 T4096 d128 bf16 with S0 = 0: o is linear in v, so
     <dO, o(v)> == <dv, v> must hold for the dv the backward kernels return."""
