@@ -121,13 +121,15 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
 #pragma unroll
     for (int it = 0; it < ValTile::IT; ++it) ta.bv[it] = tb.bv[it] = 0.f;
-    auto fetch = [&](Tiles& R, int n) {
+    // part 0: K, 1: Q, 2: the rest; < 0: everything
+    auto fetch = [&](Tiles& R, int n, int part = -1) {
       const int64_t slot = (int64_t)row * N + n;
       int tok0;
       chunk_span(span, n, tok0, R.len);
       const int64_t tbase = tok_index(p.geom, row, tok0);
-      R.K.load(p.k + tbase * DK, tsk, R.len, mt);
-      R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      if (part < 0 || part == 0) R.K.load(p.k + tbase * DK, tsk, R.len, mt);
+      if (part < 0 || part == 1) R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      if (part == 0 || part == 1) return;
       R.V.load(p.v + tbase * p.vcols + v0, tsv, (v0 < p.vcols) ? R.len : 0, mt);  // columns v does not hold read as zero
       R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
       R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
@@ -148,21 +150,28 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       for (int it = 0; it < ValTile::IT; ++it)
         R.bv[it] = p.beta[tbase + (int64_t)min(min((mt + 256 * it) / ValTile::VPR, 63), R.len - 1) * p.geom.ts];
     };
-    auto commit = [&](const Tiles& R, int pb) {
+    auto commit = [&](const Tiles& R, int pb, int part = -1) {
       {  // K rows normalised; Q rows normalised and scaled by scale e^{G_i}: the outputs then need no scaling of their own
         T* dstk = sK + pb * L::kK;
         T* dst = sQ + pb * L::kK;
 #pragma unroll
         for (int it = 0; it < RowTile::IT; ++it) {
           const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
-          const float f = R.fq[it];
-          typename Vec16<T>::V x = R.Q.x[it], y = R.K.x[it];
+          if (part < 0 || part == 0) {
+            typename Vec16<T>::V y = R.K.x[it];
 #pragma unroll
-          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f), y[e] = (bf16_t)((float)y[e] * R.nk[it]);
-          *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
-          *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
+            for (int e = 0; e < RowTile::N; ++e) y[e] = (bf16_t)((float)y[e] * R.nk[it]);
+            *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
+          }
+          if (part < 0 || part == 1) {
+            typename Vec16<T>::V x = R.Q.x[it];
+#pragma unroll
+            for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * R.fq[it]);
+            *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+          }
         }
       }
+      if (part == 0 || part == 1) return;
       {  // V rows scaled by beta_i: R = beta V - (beta e^G) Y
         T* dst = sV + pb * L::kV;
 #pragma unroll
@@ -187,10 +196,22 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     // cur: the register set that held chunk n (in LDS since the last step) and now takes chunk n + 2; nxt: chunk n + 1.
     // `steady` (a std::bool_constant): chunks n + 1 and n + 2 exist, so nothing below sits behind a branch -- behind a
     // conditional fetch the compiler cannot count the younger loads in flight and would wait for all of them.
+    // The loads are admitted at the rate the memory path takes them, and a wave that has a load waiting for a slot
+    // issues nothing else: so the tile writes of chunk n + 1 sit between the loads of chunk n + 2, a tile at a time, and
+    // go out while the loads before them drain (issued one after the other: forward scan 237 -> 216 us).
     auto step = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
       constexpr bool STEADY = decltype(steady)::value;
-      if (STEADY || n + 2 < c1) fetch(cur, n + 2);
-      if (STEADY || n + 1 < c1) commit(nxt, (n + 1 - c0) & 1);
+      if constexpr (STEADY) {
+#pragma unroll
+        for (int part = 0; part < 3; ++part) {
+          fetch(cur, n + 2, part);
+          commit(nxt, (n + 1 - c0) & 1, part);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        if (n + 2 < c1) fetch(cur, n + 2);
+        if (n + 1 < c1) commit(nxt, (n + 1 - c0) & 1);
+      }
       lds_barrier();  // Bmid
       int tok0, len;
       chunk_span(span, n, tok0, len);
@@ -481,13 +502,14 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
     ta.len = tb.len = 0;
 #pragma unroll
     for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
-    auto fetch = [&](Tiles& R, int n) {
+    auto fetch = [&](Tiles& R, int n, int part = -1) {  // part 0: K, 1: Q, 2: the rest; < 0: everything
       const int64_t slot = (int64_t)row * N + n;
       int tok0;
       chunk_span(span, n, tok0, R.len);
       const int64_t tbase = tok_index(p.geom, row, tok0);
-      R.K.load(p.k + tbase * DK, tsk, R.len, mt);
-      R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      if (part < 0 || part == 0) R.K.load(p.k + tbase * DK, tsk, R.len, mt);
+      if (part < 0 || part == 1) R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
+      if (part == 0 || part == 1) return;
       R.dO.load(p.d_o + tbase * p.dv + v0, tsv, R.len, mt);
       R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
       R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
@@ -504,21 +526,28 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       }
       R.b = p.beta[tbase + (int64_t)min(t, R.len - 1) * p.geom.ts];
     };
-    auto commit = [&](const Tiles& R, int pb) {
+    auto commit = [&](const Tiles& R, int pb, int part = -1) {
       {  // K rows normalised; Q rows normalised and scaled by scale e^{G_i}: (scale diag(e^G) Q)^T dO needs no scaled copy of dO
         T* dstk = sK + pb * L::kK;
         T* dst = sQ + pb * L::kK;
 #pragma unroll
         for (int it = 0; it < RowTile::IT; ++it) {
           const int idx = mt + 256 * it, r = idx / RowTile::VPR, c = (idx - r * RowTile::VPR) * RowTile::N;
-          const float f = R.fq[it];
-          typename Vec16<T>::V x = R.Q.x[it], y = R.K.x[it];
+          if (part < 0 || part == 0) {
+            typename Vec16<T>::V y = R.K.x[it];
 #pragma unroll
-          for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * f), y[e] = (bf16_t)((float)y[e] * R.nk[it]);
-          *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
-          *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
+            for (int e = 0; e < RowTile::N; ++e) y[e] = (bf16_t)((float)y[e] * R.nk[it]);
+            *reinterpret_cast<typename Vec16<T>::V*>(dstk + r * LDK + c) = y;
+          }
+          if (part < 0 || part == 1) {
+            typename Vec16<T>::V x = R.Q.x[it];
+#pragma unroll
+            for (int e = 0; e < RowTile::N; ++e) x[e] = (bf16_t)((float)x[e] * R.fq[it]);
+            *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDK + c) = x;
+          }
         }
       }
+      if (part == 0 || part == 1) return;
       R.dO.store(sdO + pb * L::kV, LDV, mt);
       R.Tm.store(sTm + pb * L::kC, LDC, mt);
       R.P.store(sP + pb * L::kC, LDC, mt);
@@ -535,8 +564,18 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
     // cur: the register set that held chunk n and now takes chunk n - 2; nxt: chunk n - 1 (see scan_fwd)
     auto step = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
       constexpr bool STEADY = decltype(steady)::value;
-      if (STEADY || n - 2 >= c0) fetch(cur, n - 2);
-      if (STEADY || n - 1 >= c0) commit(nxt, (c1 - n) & 1);  // position of chunk n - 1 from the end: c1 - 1 - (n - 1)
+      const int pbn = (c1 - n) & 1;  // position of chunk n - 1 from the end: c1 - 1 - (n - 1)
+      if constexpr (STEADY) {  // tile writes between the loads, a tile at a time (see scan_fwd)
+#pragma unroll
+        for (int part = 0; part < 3; ++part) {
+          fetch(cur, n - 2, part);
+          commit(nxt, pbn, part);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        if (n - 2 >= c0) fetch(cur, n - 2);
+        if (n - 1 >= c0) commit(nxt, pbn);
+      }
       lds_barrier();  // Bmid
       const int64_t slot = (int64_t)row * N + n;
       unstage_tile<T, BV, DK, true>(at<T>(p.ws, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
