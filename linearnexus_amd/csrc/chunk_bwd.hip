@@ -361,9 +361,12 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
         }
       }
     };
-    auto commit_rest = [&](const Tiles& R, int pb) {
-      R.Q.store(sQ + pb * L::kRow, LDK, mt);
-      R.W.store(sW + pb * L::kRow, LDK, mt);
+    auto commit_rest = [&](const Tiles& R, int pb, int part = -1) {  // parts as in fetch (K is written by the caller)
+      if (part < 0 || part == 2) {
+        R.Q.store(sQ + pb * L::kRow, LDK, mt);
+        R.W.store(sW + pb * L::kRow, LDK, mt);
+      }
+      if (part == 0 || part == 2) return;
       if (FUSE) {
         R.P.store(sP + pb * L::kP, LDC, mt);
         R.dO.store(sdOr + pb * L::kRaw, LDU, mt);
@@ -384,22 +387,35 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       if (mt < L::kG) sG[pb * L::kG + mt] = R.G;
     };
     // Double-buffered form.  Chunk n - 1 goes to the buffers chunk n + 1 was read from, so no tile write waits for a
-    // reader: loads of chunk n - 2 in the first phase, dS', dD -> workspace and the tile writes in the second.
+    // reader: loads of chunk n - 2 and the tile writes in the first phase, dS', dD -> workspace in the second.
     // `steady` (a std::bool_constant): chunks n - 1 and n - 2 exist, so nothing sits behind a branch and the compiler
     // can count the loads in flight.
     auto step_db = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
       constexpr bool STEADY = decltype(steady)::value;
       const int64_t slot = (int64_t)row * N + n;
       const int pb = (c1 - 1 - n) & 1;
-      if (STEADY || n - 2 >= c0) fetch(cur, n - 2, -1);  // chunk n's registers are free again
+      if constexpr (STEADY) {
+        // chunk n's registers are free again and take chunk n - 2; the tile writes of chunk n - 1 sit between the loads,
+        // a part at a time: a wave whose load waits for a slot in the memory path issues nothing else, and the writes
+        // go out while the loads before them drain
+#pragma unroll
+        for (int part = 0; part < 3; ++part) {
+          fetch(cur, n - 2, part);
+          if (part == 0) nxt.K.store(sK + (pb ^ 1) * L::kRow, LDK, mt);
+          else commit_rest(nxt, pb ^ 1, part);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        if (n - 2 >= c0) fetch(cur, n - 2, -1);
+        if (n - 1 >= c0) {
+          nxt.K.store(sK + (pb ^ 1) * L::kRow, LDK, mt);
+          commit_rest(nxt, pb ^ 1);
+        }
+      }
       if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
       lds_barrier();  // B2
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
-      if (STEADY || n - 1 >= c0) {
-        nxt.K.store(sK + (pb ^ 1) * L::kRow, LDK, mt);
-        commit_rest(nxt, pb ^ 1);
-      }
       lds_barrier();  // B3
       lds_barrier();  // B1 of the next chunk
     };

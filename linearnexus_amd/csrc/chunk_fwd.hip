@@ -875,31 +875,34 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
     Tiles ta, tb;
     ta.G = tb.G = 0.f;
     ta.tok0 = ta.len = tb.tok0 = tb.len = 0;
-    auto fetch = [&](Tiles& R, int n) {
+    // part 0: W, 1: K, 2: Q, 3: the rest; < 0: everything
+    auto fetch = [&](Tiles& R, int n, int part = -1) {
       const int64_t slot = (int64_t)row * N + n;
       chunk_span(span, n, R.tok0, R.len);
       const int64_t tbase = tok_index(p.geom, row, R.tok0);
       const int64_t tsk = (int64_t)p.geom.ts * DK;
-      R.W.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
-      if (GATE == LNX_GATE_VECTOR) R.K.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
-      else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, R.len, mt);
-      R.U.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
-      if (FUSE) {
+      if (part < 0 || part == 0) R.W.load(ws_ptr<T>(p, p.off.W) + slot * 64 * DK, DK, 64, mt);
+      if (part < 0 || part == 1) {
+        if (GATE == LNX_GATE_VECTOR) R.K.load(ws_ptr<T>(p, p.off.Kr) + slot * 64 * DK, DK, 64, mt);
+        else R.K.load(reinterpret_cast<const T*>(p.k) + tbase * DK, tsk, R.len, mt);
+      }
+      if (FUSE && (part < 0 || part == 2)) {
         if (GATE == LNX_GATE_VECTOR) R.Q.load(ws_ptr<T>(p, p.off.Qg) + slot * 64 * DK, DK, 64, mt);
         else R.Q.load(reinterpret_cast<const T*>(p.q) + tbase * DK, tsk, R.len, mt);
-        R.P.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       }
+      if (part >= 0 && part < 3) return;
+      R.U.load(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + v0, p.dv, 64, mt);
+      if (FUSE) R.P.load(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, 64, mt);
       // every thread loads (clamped index): a load behind a branch cannot be counted
       if (GATE == LNX_GATE_SCALAR) R.G = ws_ptr<float>(p, p.off.G)[slot * 64 + (mt & 63)];
       if (GATE == LNX_GATE_VECTOR) R.G = ws_ptr<float>(p, p.off.G)[(slot * 64 + 63) * DK + min(mt, DK - 1)];  // G_last[c]
     };
-    auto commit_rest = [&](const Tiles& R, int pb) {
-      R.K.store(sK + pb * L::kKT, LDK, mt);
+    auto commit_rest = [&](const Tiles& R, int pb, int part = -1) {  // parts as in fetch (W is written by the caller)
+      if (part < 0 || part == 1) R.K.store(sK + pb * L::kKT, LDK, mt);
+      if (FUSE && (part < 0 || part == 2)) R.Q.store(sQ + pb * L::kQ, LDK, mt);
+      if (part >= 0 && part < 3) return;
       R.U.store(sU + pb * L::kU, LDU, mt);
-      if (FUSE) {
-        R.Q.store(sQ + pb * L::kQ, LDK, mt);
-        R.P.store(sP + pb * L::kP, LDC, mt);
-      }
+      if (FUSE) R.P.store(sP + pb * L::kP, LDC, mt);
       if (mt < L::kG) sG[pb * kGM + mt] = R.G;
       if (mt == 0) {
         sMeta[pb * kGM] = R.tok0;
@@ -917,18 +920,31 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       if constexpr (L::DB) {
         // Chunk n + 1 goes to the buffers chunk n - 1 was read from, so no tile write waits for a reader, and every
         // global store of the kernel is issued here: stores issued by the compute waves queued behind the movers'
-        // loads and held the chain up.  Loads in the first phase, the chunk's state and D and the next chunk's tile
-        // writes in the second (the compute waves' longest), the outputs in the third.
+        // loads and held the chain up.  Loads and the next chunk's tile writes in the first phase, the chunk's state
+        // and D in the second, the outputs in the third.
         const int pb = (n - c0) & 1;
-        if (STEADY || n + AHEAD < c1) fetch(cur, n + AHEAD);  // chunk n's registers are free again
+        if constexpr (STEADY) {
+          // chunk n's registers are free again and take chunk n + 2; the tile writes of chunk n + 1 sit between the
+          // loads, a tile at a time: a wave whose load waits for a slot in the memory path issues nothing else, and
+          // the writes go out while the loads before them drain
+#pragma unroll
+          for (int part = 0; part < 4; ++part) {
+            fetch(cur, n + AHEAD, part);
+            if (part == 0) nxt.W.store(sW + (pb ^ 1) * L::kW, LDK, mt);
+            else commit_rest(nxt, pb ^ 1, part);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
+          if (n + AHEAD < c1) fetch(cur, n + AHEAD);
+          if (n + 1 < c1) {
+            nxt.W.store(sW + (pb ^ 1) * L::kW, LDK, mt);
+            commit_rest(nxt, pb ^ 1);
+          }
+        }
         lds_barrier();  // B2
         if (p.save) {
           unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
           unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU + pb * L::kU, LDU, 64, mt);
-        }
-        if (STEADY || n + 1 < c1) {
-          nxt.W.store(sW + (pb ^ 1) * L::kW, LDK, mt);
-          commit_rest(nxt, pb ^ 1);
         }
         lds_barrier();  // B3
         if (p.o) {
