@@ -387,7 +387,7 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       if (mt < L::kG) sG[pb * L::kG + mt] = R.G;
     };
     // Double-buffered form.  Chunk n - 1 goes to the buffers chunk n + 1 was read from, so no tile write waits for a
-    // reader: loads of chunk n - 2 and the tile writes in the first phase, dS', dD -> workspace in the second.
+    // reader: loads of chunk n - 2 and the tile writes in the first two phases, dS', dD -> workspace in the second.
     // `steady` (a std::bool_constant): chunks n - 1 and n - 2 exist, so nothing sits behind a branch and the compiler
     // can count the loads in flight.
     auto step_db = [&](Tiles& cur, const Tiles& nxt, int n, auto steady) {
@@ -397,9 +397,9 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       if constexpr (STEADY) {
         // chunk n's registers are free again and take chunk n - 2; the tile writes of chunk n - 1 sit between the loads,
         // a part at a time: a wave whose load waits for a slot in the memory path issues nothing else, and the writes
-        // go out while the loads before them drain
+        // go out while the loads before them drain.  Q and W follow the stores of the second phase.
 #pragma unroll
-        for (int part = 0; part < 3; ++part) {
+        for (int part = 0; part < 2; ++part) {
           fetch(cur, n - 2, part);
           if (part == 0) nxt.K.store(sK + (pb ^ 1) * L::kRow, LDK, mt);
           else commit_rest(nxt, pb ^ 1, part);
@@ -416,6 +416,10 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       lds_barrier();  // B2
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
+      if constexpr (STEADY) {
+        fetch(cur, n - 2, 2);
+        commit_rest(nxt, pb ^ 1, 2);
+      }
       lds_barrier();  // B3
       lds_barrier();  // B1 of the next chunk
     };

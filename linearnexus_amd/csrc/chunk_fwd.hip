@@ -920,15 +920,16 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
       if constexpr (L::DB) {
         // Chunk n + 1 goes to the buffers chunk n - 1 was read from, so no tile write waits for a reader, and every
         // global store of the kernel is issued here: stores issued by the compute waves queued behind the movers'
-        // loads and held the chain up.  Loads and the next chunk's tile writes in the first phase, the chunk's state
-        // and D in the second, the outputs in the third.
+        // loads and held the chain up.  Loads and the next chunk's tile writes in the first two phases, the chunk's
+        // state and D in the second, the outputs in the third.
         const int pb = (n - c0) & 1;
         if constexpr (STEADY) {
           // chunk n's registers are free again and take chunk n + 2; the tile writes of chunk n + 1 sit between the
           // loads, a tile at a time: a wave whose load waits for a slot in the memory path issues nothing else, and
-          // the writes go out while the loads before them drain
+          // the writes go out while the loads before them drain.  W and K here, Q and the rest behind the stores of
+          // the second phase (all in this phase: 0.322 ms at B4 H16 T8192; split: 0.310)
 #pragma unroll
-          for (int part = 0; part < 4; ++part) {
+          for (int part = 0; part < 2; ++part) {
             fetch(cur, n + AHEAD, part);
             if (part == 0) nxt.W.store(sW + (pb ^ 1) * L::kW, LDK, mt);
             else commit_rest(nxt, pb ^ 1, part);
@@ -945,6 +946,14 @@ __global__ __launch_bounds__(512) void chunk_scan_kernel(FwdParams p) {
         if (p.save) {
           unstage_tile<T, BV, DK, true>(ws_ptr<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
           unstage_tile<T, 64, BV, true>(ws_ptr<T>(p, p.off.D) + slot * 64 * p.dv + v0, p.dv, sU + pb * L::kU, LDU, 64, mt);
+        }
+        if constexpr (STEADY) {
+#pragma unroll
+          for (int part = 2; part < 4; ++part) {
+            fetch(cur, n + AHEAD, part);
+            commit_rest(nxt, pb ^ 1, part);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
         lds_barrier();  // B3
         if (p.o) {
