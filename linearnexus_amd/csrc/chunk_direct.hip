@@ -46,6 +46,17 @@ __device__ __forceinline__ void store_frag_t(const floatx16& a, T* dst, int ld, 
   }
 }
 
+// Zeroes the 224 vectors above the diagonal (row r, columns 8 c .. 8 c + 7 with 8 c > r) of `ntile` consecutive
+// [64][ld] tiles of `stride` elements; 256 threads.  Group g of eight rows has 7 - g such vectors per row.
+__device__ __forceinline__ void zero_upper_triangles(T* tiles, int ntile, int stride, int ld, int tid) {
+  if (tid >= 512 - LNX_TRI_VECS) return;
+  int g = 0;
+  while (56 * (g + 1) - 4 * (g + 1) * g <= tid) ++g;  // vectors of the groups before g + 1
+  const int o = tid - (56 * g - 4 * g * (g - 1)), per = 7 - g;
+  const int r = 8 * g + o / per, c = g + 1 + (o - (o / per) * per);
+  for (int t = 0; t < ntile; ++t) *reinterpret_cast<Vec16<T>::V*>(tiles + t * stride + r * ld + 8 * c) = vec_zero<T>();
+}
+
 // Per-token scalars of one chunk in LDS, written by the movers when they commit a chunk
 struct Scal {
   enum { BETA = 0, GAM = 64, R = 128, SG = 192, DEC = 256, SIZE = 320 };  // beta, e^G, e^{G_C - G}, scale e^G, e^{G_C}
@@ -108,7 +119,7 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     struct Tiles {
       RowTile K, Q;
       ValTile V;
-      TileRegs<T, 64, 64> Tm, P;
+      TriRegs<T> Tm, P;  // lower-triangular tiles, packed in the workspace
       float g, gc, b;
       float fq[RowTile::IT], nk[RowTile::IT];  // factors of the token each of this thread's Q / K vectors belongs to
       float bv[ValTile::IT];  // beta of the token each of its V vectors belongs to
@@ -116,6 +127,8 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     };
     Tiles ta, tb;
     ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
+    ta.Tm.init(LDC, mt), ta.P.init(LDC, mt), tb.Tm.init(LDC, mt), tb.P.init(LDC, mt);
+    zero_upper_triangles(sTm, 4, L::kC, LDC, mt);  // both buffers of Tm and Pm: the packed tiles never write there
     ta.len = tb.len = 0;
 #pragma unroll
     for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
@@ -131,8 +144,8 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       if (part < 0 || part == 1) R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
       if (part == 0 || part == 1) return;
       R.V.load(p.v + tbase * p.vcols + v0, tsv, (v0 < p.vcols) ? R.len : 0, mt);  // columns v does not hold read as zero
-      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
-      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, mt);
+      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, mt);
       // every thread loads the scalars of token mt % 64 (no load behind a branch); tokens past the end are masked below
       const int t = mt & 63;
       if (GATE == LNX_GATE_SCALAR) {
@@ -183,8 +196,8 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
           if (idx < ValTile::TOTAL) *reinterpret_cast<typename Vec16<T>::V*>(dst + r * LDV + c) = x;
         }
       }
-      R.Tm.store(sTm + pb * L::kC, LDC, mt);
-      R.P.store(sP + pb * L::kC, LDC, mt);
+      R.Tm.store(sTm + pb * L::kC);
+      R.P.store(sP + pb * L::kC);
       if (mt < 64) {
         float* sc = sSc + pb * Scal::SIZE;
         const float gam = (GATE == LNX_GATE_SCALAR) ? __expf(R.g) : 1.f;
@@ -492,13 +505,15 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
     struct Tiles {
       RowTile K, Q;
       TileRegs<T, 64, BV> dO;
-      TileRegs<T, 64, 64> Tm, P;
+      TriRegs<T> Tm, P;  // lower-triangular tiles, packed in the workspace
       float g, gc, b;
       float fq[RowTile::IT], nk[RowTile::IT];  // factors of the token each of this thread's Q / K vectors belongs to
       int len;
     };
     Tiles ta, tb;
     ta.g = ta.gc = ta.b = tb.g = tb.gc = tb.b = 0.f;
+    ta.Tm.init(LDC, mt), ta.P.init(LDC, mt), tb.Tm.init(LDC, mt), tb.P.init(LDC, mt);
+    zero_upper_triangles(sTm, 4, L::kC, LDC, mt);  // both buffers of Tm and Pm: the packed tiles never write there
     ta.len = tb.len = 0;
 #pragma unroll
     for (int it = 0; it < RowTile::IT; ++it) ta.fq[it] = tb.fq[it] = ta.nk[it] = tb.nk[it] = 0.f;
@@ -511,8 +526,8 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       if (part < 0 || part == 1) R.Q.load(p.q + tbase * DK, tsk, R.len, mt);
       if (part == 0 || part == 1) return;
       R.dO.load(p.d_o + tbase * p.dv + v0, tsv, R.len, mt);
-      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, 64, 64, mt);
-      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, 64, 64, mt);
+      R.Tm.load(at<const T>(p.ws, p.off.Tm) + slot * 64 * 64, mt);
+      R.P.load(at<const T>(p.ws, p.off.P) + slot * 64 * 64, mt);
       const int t = mt & 63;
       if (GATE == LNX_GATE_SCALAR) {
         const float* G = at<const float>(p.ws, p.off.G) + slot * 64;
@@ -549,8 +564,8 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       }
       if (part == 0 || part == 1) return;
       R.dO.store(sdO + pb * L::kV, LDV, mt);
-      R.Tm.store(sTm + pb * L::kC, LDC, mt);
-      R.P.store(sP + pb * L::kC, LDC, mt);
+      R.Tm.store(sTm + pb * L::kC);
+      R.P.store(sP + pb * L::kC);
       if (mt < 64) {
         float* sc = sSc + pb * Scal::SIZE;
         const float gam = (GATE == LNX_GATE_SCALAR) ? __expf(R.g) : 1.f;

@@ -195,7 +195,20 @@ __global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdPa
     frag_store<T, 1, 1>(pe, sPt + 32 * wi * LDC + 32 * wj, LDC, lane);
   }
   lds_barrier();
-  unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sPt, LDC, 64, tid);
+  // LITE, 2-byte inputs: Pm and Tm leave packed (TriRegs in mma_tiles.h), only the vectors at or below the diagonal;
+  // this thread's vector tid and, for tid < 32, vector 256 + tid
+  int tr0 = 0, tc0 = 0, tr1 = 0, tc1 = 0;
+  const bool tri2 = tid < LNX_TRI_VECS - 256;
+  if constexpr (LITE && sizeof(T) == 2) {
+    tri_vec_pos(tid, tr0, tc0);
+    tri_vec_pos(tri2 ? 256 + tid : 0, tr1, tc1);
+    T* Pg = ws_ptr<T>(p, p.off.P) + slot * 64 * 64;
+    typedef typename Vec16<T>::V V;
+    *reinterpret_cast<V*>(Pg + 8 * tid) = *reinterpret_cast<const V*>(sPt + tr0 * LDC + 8 * tc0);
+    if (tri2) *reinterpret_cast<V*>(Pg + 8 * (256 + tid)) = *reinterpret_cast<const V*>(sPt + tr1 * LDC + 8 * tc1);
+  } else {
+    unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.P) + slot * 64 * 64, 64, sPt, LDC, 64, tid);
+  }
   if constexpr (LITE) {
     tri_inverse_64<true>(sA, sA, sX, tid);
   } else {
@@ -204,9 +217,21 @@ __global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdPa
   }
   if constexpr (LITE) {
     T* Tm = ws_ptr<T>(p, p.off.Tm) + slot * 64 * 64;
-    for (int idx = tid; idx < 64 * 16; idx += 256) {
-      const int r = idx >> 4, c = (idx & 15) * 4;
-      store4(Tm + r * 64 + c, load4(sA + r * LNX_LDA + c));
+    if constexpr (sizeof(T) == 2) {
+      typedef unsigned uint2_ __attribute__((ext_vector_type(2)));
+      typedef unsigned uint4_ __attribute__((ext_vector_type(4)));
+      auto put = [&](int idx, int r, int c) {
+        const float* src = sA + r * LNX_LDA + 8 * c;
+        const uint2_ lo = __builtin_bit_cast(uint2_, pack_bf16x4(load4(src))), hi = __builtin_bit_cast(uint2_, pack_bf16x4(load4(src + 4)));
+        *reinterpret_cast<uint4_*>(Tm + 8 * idx) = uint4_{lo[0], lo[1], hi[0], hi[1]};
+      };
+      put(tid, tr0, tc0);
+      if (tri2) put(256 + tid, tr1, tc1);
+    } else {
+      for (int idx = tid; idx < 64 * 16; idx += 256) {
+        const int r = idx >> 4, c = (idx & 15) * 4;
+        store4(Tm + r * 64 + c, load4(sA + r * LNX_LDA + c));
+      }
     }
     return;
   }

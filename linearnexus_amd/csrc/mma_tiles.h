@@ -258,6 +258,48 @@ template <typename T, int ROWS, int COLS> struct TileRegs {
   }
 };
 
+// A lower-triangular [64 x 64] 2-byte tile travels packed: of its 512 eight-element vectors (row r, columns 8 c .. 8 c + 7)
+// only the 288 with 8 c <= r can hold a non-zero.  Rows come in groups of eight; group g has g + 1 vectors per row and starts
+// at packed index 4 g (g + 1); a slot of the workspace keeps its 64 x 64 elements and uses the first 288 x 16 bytes.
+constexpr int LNX_TRI_VECS = 288;
+__device__ __forceinline__ void tri_vec_pos(int idx, int& r, int& c) {  // idx < LNX_TRI_VECS
+  int g = 0;
+#pragma unroll
+  for (int h = 1; h < 8; ++h) g += (4 * h * (h + 1) <= idx) ? 1 : 0;
+  const int o = idx - 4 * g * (g + 1);  // < 64
+  // o / (g + 1) without an integer division: (o + 0.5) / (g + 1) is at least 1/16 away from every integer
+  const int q = (int)(((float)o + 0.5f) * __builtin_amdgcn_rcpf((float)(g + 1)));
+  r = 8 * g + q;
+  c = o - q * (g + 1);
+}
+// The packed tile in the registers of 256 threads (vector tid, and vector 256 + tid for tid < 32) between its global
+// loads and its LDS stores, like TileRegs; the LDS tile's upper part is zeroed once by the caller and never written.
+template <typename T> struct TriRegs {
+  static_assert(sizeof(T) == 2, "packed triangles are a 2-byte format");
+  typename Vec16<T>::V x[2];
+  int o0, o1;  // LDS element offsets of this thread's two vectors for a leading dimension fixed at init
+  bool second;
+  __device__ __forceinline__ void init(int ld, int tid) {
+    int r, c;
+    tri_vec_pos(tid, r, c);
+    o0 = r * ld + 8 * c;
+    second = tid < LNX_TRI_VECS - 256;
+    tri_vec_pos(second ? 256 + tid : LNX_TRI_VECS - 1, r, c);
+    o1 = r * ld + 8 * c;
+  }
+  __device__ __forceinline__ void load(const T* src, int tid) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, LNX_TRI_VECS * 16, 0x00020000);
+    x[0] = __builtin_bit_cast(typename Vec16<T>::V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, 16 * tid, 0, 0));
+    // threads without a second vector read past the end: the range check returns zeros, nothing sits behind a branch
+    x[1] = __builtin_bit_cast(typename Vec16<T>::V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, 16 * (256 + tid), 0, 0));
+  }
+  __device__ __forceinline__ void store(T* dst) const {
+    *reinterpret_cast<typename Vec16<T>::V*>(dst + o0) = x[0];
+    if (second) *reinterpret_cast<typename Vec16<T>::V*>(dst + o1) = x[1];
+  }
+};
+
 // One-shot form (load, then store) for a single tile.
 template <typename T, int ROWS, int COLS>
 __device__ __forceinline__ void stage_tile(T* dst, int ld, const T* src, int64_t stride, int valid, int tid) {
