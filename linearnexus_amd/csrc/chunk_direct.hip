@@ -229,7 +229,7 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       int tok0, len;
       chunk_span(span, n, tok0, len);
       if (p.o)
-        unstage_tile<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
+        unstage_tile_checked<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
       if (p.save) {
         const int64_t slot = (int64_t)row * N + n;
         unstage_tile<T, BV, DK, true>(at<T>(p.ws, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
@@ -597,7 +597,7 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       unstage_tile<T, BV, 64, true>(at<T>(p.ws, p.off.dD) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, sdRT, LDC, BV, mt);
       int tok0, len;
       chunk_span(span, n, tok0, len);
-      unstage_tile<T, 64, BV>(p.dv_out + tok_index(p.geom, row, tok0) * p.dv + v0, tsv, sdV, LDV, len, mt);
+      unstage_tile_checked<T, 64, BV>(p.dv_out + tok_index(p.geom, row, tok0) * p.dv + v0, tsv, sdV, LDV, len, mt);
       lds_barrier();  // B1 of the next chunk
     };
     if (c0 < c1) {
