@@ -183,13 +183,25 @@ __global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdPa
   if (!LITE) fetch(0);
   lds_barrier();  // slab tiles dead
   {
+    // the per-row scalars of this lane's sixteen fragment rows (four runs of four) first, as vectors: read one by one
+    // between the stores below, each read waited for its own round trip to LDS (the stores might alias them)
+    floatx4 gi[4], bi[4], nki[4], nqi[4];
+    const int j = 32 * wj + frag_col(lane);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i0 = 32 * wi + 8 * q + 4 * (lane >> 5);
+      gi[q] = load4(sG + i0);
+      bi[q] = load4(sBeta + i0);
+      if (LITE) nki[q] = load4(sNk + i0), nqi[q] = load4(sNq + i0);
+    }
+    const float gj = sG[j], nkj = LITE ? sNk[j] : 1.f;
     floatx16 pe[1][1];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
-      const float fx = LITE ? sNk[i] * sNk[j] : 1.f, fp = LITE ? sNq[i] * sNk[j] : 1.f;
-      sA[i * LNX_LDA + j] = (i > j) ? sBeta[i] * dec * fx * ax[0][0][e] : 0.f;
+      const int i = 32 * wi + frag_row(e, lane), q = e >> 2, u = e & 3;
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gi[q][u] - gj, 0.f));
+      const float fx = LITE ? nki[q][u] * nkj : 1.f, fp = LITE ? nqi[q][u] * nkj : 1.f;
+      sA[i * LNX_LDA + j] = (i > j) ? bi[q][u] * dec * fx * ax[0][0][e] : 0.f;
       pe[0][0][e] = (i >= j) ? p.scale * dec * fp * ap[0][0][e] : 0.f;
     }
     frag_store<T, 1, 1>(pe, sPt + 32 * wi * LDC + 32 * wj, LDC, lane);
