@@ -116,9 +116,15 @@ __global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdPa
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.vcols;
   const int wi = wave >> 1, wj = wave & 1;
 
-  TileRegs<T, 64, 64> rK, rQ;
+  // LITE with two slabs: all four tiles are requested at once, so the latency of the loads is waited out once
+  constexpr bool AHEAD = LITE && NKS == 2;
+  TileRegs<T, 64, 64> rK, rQ, rK1, rQ1;
   rK.load(kg, tsk, len, tid);
   rQ.load(qg, tsk, len, tid);
+  if (AHEAD) {
+    rK1.load(kg + 64, tsk, len, tid);
+    rQ1.load(qg + 64, tsk, len, tid);
+  }
   if (wave == 0) {
     const bool ok = lane < len;
     sBeta[lane] = ok ? p.beta[tbase + (int64_t)lane * p.geom.ts] : 0.f;
@@ -132,13 +138,18 @@ __global__ __launch_bounds__(256, LITE ? 5 : 1) void chunk_prepare2_kernel(FwdPa
   frag_zero(ax);
   frag_zero(ap);
   float nk2 = 0.f, nq2 = 0.f;  // LITE: squared row norms, thread = (row tid / 4, 16 columns of the slab)
-#pragma unroll 1
+#pragma unroll(AHEAD ? 2 : 1)
   for (int s_ = 0; s_ < NKS; ++s_) {
     lds_barrier();
-    rK.store(sKa, LDC, tid);
-    rQ.store(sQa, LDC, tid);
+    if (AHEAD && s_ == 1) {
+      rK1.store(sKa, LDC, tid);
+      rQ1.store(sQa, LDC, tid);
+    } else {
+      rK.store(sKa, LDC, tid);
+      rQ.store(sQa, LDC, tid);
+    }
     lds_barrier();
-    if (s_ + 1 < NKS) {
+    if (!AHEAD && s_ + 1 < NKS) {
       rK.load(kg + 64 * (s_ + 1), tsk, len, tid);
       rQ.load(qg + 64 * (s_ + 1), tsk, len, tid);
     }
