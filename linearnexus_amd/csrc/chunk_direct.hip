@@ -270,6 +270,11 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     for (int ci = 0; ci < KT; ++ci)
 #pragma unroll
       for (int e = 0; e < 16; ++e) S[ci][e] = s0[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv + frag_col(lane)];
+    // the loads complete here: left pending into the loop, every iteration would count them down again
+#pragma unroll
+    for (int ci = 0; ci < KT; ++ci)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) asm volatile("" : "+v"(S[ci][e]));
   }
   lds_barrier();  // B1 of the first chunk
   // Every LDS read is issued well ahead of the product that consumes it (A fragments two steps ahead, the next
@@ -330,41 +335,45 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // first A fragments of D = Tm R
+    // Tm and Pm are lower-triangular: the first 32 rows of D and of the outputs take the first 32 tokens only, so the two
+    // products need 6 MFMAs each, not 8, and the work on the first half (R, D, scaling, conversions, stores) runs in the
+    // shadow of the second half's MFMAs.  tm[i][ks], pm[i][ks]: row tile i, 16-token step ks (i = 0: ks < 2).
+    M::Frag tm0[2], tm1[4], pm0[2], pm1[4];
 #pragma unroll
-    for (int s_ = 0; s_ < 2; ++s_)
-#pragma unroll
-      for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_chain(sTc + (32 * i + fr) * LDC + 16 * s_, lane);
+    for (int ks = 0; ks < 2; ++ks) {
+      tm0[ks] = M::load_chain(sTc + fr * LDC + 16 * ks, lane);
+      tm1[ks] = M::load_chain(sTc + (32 + fr) * LDC + 16 * ks, lane);
+    }
     __builtin_amdgcn_sched_barrier(0);
-    // ---- R = beta V - (beta e^G) Y, in place of Y ----
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
+    // ---- R = beta V - (beta e^G) Y, in place of Y: tokens 0 .. 31 ----
+    auto form_r = [&](int i) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int u = 0; u < 4; ++u) y[i][4 * q + u] = (float)vr[i][q][u] - sv[i][q][u] * y[i][4 * q + u];
+    };
+    form_r(0);
     M::Frag br[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(y[ks >> 1], ks & 1);
+    br[0] = M::from_acc(y[0], 0), br[1] = M::from_acc(y[0], 1);
     __builtin_amdgcn_sched_barrier(0);
-    // ---- D = Tm R ----
+    // ---- D = Tm R: the steps over tokens 0 .. 31, with R of tokens 32 .. 63 formed meanwhile ----
     floatx16 d[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) d[i][e] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      if (ks + 2 < 4) {
+    for (int ks = 2; ks < 4; ++ks) tm1[ks] = M::load_chain(sTc + (32 + fr) * LDC + 16 * ks, lane);
+    M::mma(d[0], tm0[0], br[0]);
+    M::mma(d[1], tm1[0], br[0]);
+    M::mma(d[0], tm0[1], br[1]);
+    M::mma(d[1], tm1[1], br[1]);
+    form_r(1);
+    br[2] = M::from_acc(y[1], 0), br[3] = M::from_acc(y[1], 1);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) fa[(ks + 2) % 3][i] = M::load_chain(sTc + (32 * i + fr) * LDC + 16 * (ks + 2), lane);
-      } else {  // first fragments of Pm for the outputs
-#pragma unroll
-        for (int i = 0; i < 2; ++i) fb[ks - 2][i] = M::load_chain(sPc + (32 * i + fr) * LDC + 16 * (ks - 2), lane);
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(d[i], fa[ks % 3][i], br[ks]);
-      __builtin_amdgcn_sched_barrier(0);
+    for (int ks = 0; ks < 2; ++ks) {
+      pm0[ks] = M::load_chain(sPc + fr * LDC + 16 * ks, lane);
+      pm1[ks] = M::load_chain(sPc + (32 + fr) * LDC + 16 * ks, lane);
     }
     if (GATE == LNX_GATE_SCALAR) {  // e^{G_C - G} for the state update
 #pragma unroll
@@ -372,28 +381,30 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
 #pragma unroll
         for (int q = 0; q < 4; ++q) sv[i][q] = load4(sc + Scal::R + 32 * i + 8 * q + 4 * (lane >> 5));
     }
-    if (p.save) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) store_frag_t(d[i], sDT + vs * LDC + 32 * i, LDC, lane);
-    }
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(d[ks >> 1], ks & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- the last two steps of D's second half; the first half goes on to the outputs ----
+    M::Frag fu[2][KT];  // K^T fragments of the state update, [step parity][row tile of the state]
+    M::Frag bd[4];      // D as the outputs' operand; br becomes the state update's operand (rows scaled by e^{G_C - G})
+    M::mma(d[1], tm1[2], br[2]);
+    M::mma(d[1], tm1[3], br[3]);
+    store_frag_t(d[0], sDT + vs * LDC, LDC, lane);  // also when nothing is saved: a branch here would split the schedule
+    bd[0] = M::from_acc(d[0], 0), bd[1] = M::from_acc(d[0], 1);
     __builtin_amdgcn_sched_barrier(0);
     // ---- O^T = (Q~ S)^T + D^T Pm^T ----
-    M::Frag fu[2][KT];  // K^T fragments of the state update, [step parity][row tile of the state]
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      if (ks + 2 < 4) {
+    for (int ks = 2; ks < 4; ++ks) pm1[ks] = M::load_chain(sPc + (32 + fr) * LDC + 16 * ks, lane);
+    M::mma(o[0], bd[0], pm0[0]);
+    M::mma(o[1], bd[0], pm1[0]);
+    M::mma(o[0], bd[1], pm0[1]);
+    M::mma(o[1], bd[1], pm1[1]);
+    store_frag_t(d[1], sDT + vs * LDC + 32, LDC, lane);
+    bd[2] = M::from_acc(d[1], 0), bd[3] = M::from_acc(d[1], 1);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) fb[(ks + 2) % 3][i] = M::load_chain(sPc + (32 * i + fr) * LDC + 16 * (ks + 2), lane);
-      } else if (ks == 2) {
-#pragma unroll
-        for (int ci = 0; ci < KT; ++ci) fu[0][ci] = M::load_t_chain(sKc, LDK, 0, 32 * ci, lane);
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(o[i], br[ks], fb[ks % 3][i]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    for (int ci = 0; ci < KT; ++ci) fu[0][ci] = M::load_t_chain(sKc, LDK, 0, 32 * ci, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    M::mma(o[1], bd[2], pm1[2]);
+    M::mma(o[1], bd[3], pm1[3]);
+    store_frag_t(o[0], sO + vs, LDV, lane);  // [token][value column]
     // the state update's operand while the last products finish: D rows scaled by e^{G_C - G}
     if (GATE == LNX_GATE_SCALAR) {
 #pragma unroll
@@ -404,11 +415,13 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
           for (int u = 0; u < 4; ++u) d[i][4 * q + u] *= sv[i][q][u];
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) br[ks] = M::from_acc(d[ks >> 1], ks & 1);
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) br[ks] = bd[ks];
     }
     const float dec = (GATE == LNX_GATE_SCALAR) ? sc[Scal::DEC] : 1.f;
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) store_frag_t(o[i], sO + 32 * i * LDV + vs, LDV, lane);  // [token][value column]
+    store_frag_t(o[1], sO + 32 * LDV + vs, LDV, lane);
     lds_barrier();  // Bmid
     // ---- S <- e^{G_C} S + K^T (e^{G_C - G} D) ----
     if (GATE == LNX_GATE_SCALAR) {
