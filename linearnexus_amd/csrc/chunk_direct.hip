@@ -664,8 +664,7 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
     for (int s_ = 0; s_ < 2; ++s_)
 #pragma unroll
       for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_chain(sKc + (32 * i + fr) * LDK + 16 * s_, lane);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) fp[0][i] = M::load_t(sPc, LDC, 0, 32 * i, lane);
+    fp[0][0] = M::load_t(sPc, LDC, 0, 0, lane);  // Pm^T and Tm^T are upper-triangular: row tile 1 takes steps 2, 3 only
     fo[0] = M::load_t(sOc, LDV, 0, vs, lane);
     // the state gradient as the B operand of Z = K dS'; its accumulators are then free to take the next dS
     M::Frag bs[NK];
@@ -689,7 +688,8 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       }
       if (ks + 1 < 4) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) fp[(ks + 1) & 1][i] = M::load_t(sPc, LDC, 16 * (ks + 1), 32 * i, lane);
+        for (int i = 0; i < 2; ++i)
+          if (i == 0 || ks + 1 >= 2) fp[(ks + 1) & 1][i] = M::load_t(sPc, LDC, 16 * (ks + 1), 32 * i, lane);
         fo[(ks + 1) & 1] = M::load_t(sOc, LDV, 16 * (ks + 1), vs, lane);
       }
       if (ks == NK - 2) {
@@ -702,16 +702,15 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
       for (int i = 0; i < 2; ++i) M::mma(z[i], fa[ks % 3][i], bs[ks]);
       if (ks < 4) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) M::mma(dd[i], fp[ks & 1][i], fo[ks & 1]);
+        for (int i = 0; i < 2; ++i)
+          if (i == 0 || ks >= 2) M::mma(dd[i], fp[ks & 1][i], fo[ks & 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     // first fragments of Tm^T, and of the (scale e^G Q)^T dO product that fills the wait for Z
     M::Frag fq[2][KT];
 #pragma unroll
-    for (int s_ = 0; s_ < 2; ++s_)
-#pragma unroll
-      for (int i = 0; i < 2; ++i) fa[s_][i] = M::load_t_chain(sTc, LDC, 16 * s_, 32 * i, lane);
+    for (int s_ = 0; s_ < 2; ++s_) fa[s_][0] = M::load_t_chain(sTc, LDC, 16 * s_, 0, lane);
 #pragma unroll
     for (int ci = 0; ci < KT; ++ci) fq[0][ci] = M::load_t(sQc, LDK, 0, 32 * ci, lane);
     fo[0] = M::load_t(sOc, LDV, 0, vs, lane);
@@ -767,9 +766,11 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
         for (int ci = 0; ci < KT; ++ci) fu[0][ci] = M::load_t_chain(sKc, LDK, 0, 32 * ci, lane);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(z[i], fa[ks % 3][i], bd[ks]);
+      for (int i = 0; i < 2; ++i)
+        if (i == 0 || ks >= 2) M::mma(z[i], fa[ks % 3][i], bd[ks]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) M::mma(dd[i], bd[ks], fa[ks % 3][i]);
+      for (int i = 0; i < 2; ++i)
+        if (i == 0 || ks >= 2) M::mma(dd[i], bd[ks], fa[ks % 3][i]);
       __builtin_amdgcn_sched_barrier(0);
     }
     const float bl0 = sc[Scal::BETA + fr], bl1 = sc[Scal::BETA + 32 + fr];
