@@ -90,9 +90,11 @@ __global__ __launch_bounds__(256) void kda_gate_bwd_kernel(GateParams p) {
   auto row = [&](float (&x)[N], float (&d)[N]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
+      // one exponential serves both: softplus(t) = max(t, 0) + log(1 + e), sigmoid(t) = (t >= 0 ? 1 : e) / (1 + e), e = e^-|t|
       const float t = x[i] + b[i];
       const bool lin = t > p.threshold;
-      const float sp = softplus_thr(t, p.threshold), ds = lin ? 1.f : 1.f / (1.f + __expf(-t));
+      const float e = __expf(-fabsf(t)), rc = __builtin_amdgcn_rcpf(1.f + e);
+      const float sp = lin ? t : fmaxf(t, 0.f) + __logf(1.f + e), ds = lin ? 1.f : (t >= 0.f ? rc : e * rc);
       sa[i] += d[i] * na * sp;
       x[i] = d[i] * na * ds;
       sb[i] += x[i];
