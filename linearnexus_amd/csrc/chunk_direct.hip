@@ -1015,12 +1015,24 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
       *reinterpret_cast<typename Vec16<T>::V*>(sQ + r * LDKT + c) = y;
     }
   }
+  // The cumulative gate and beta of this lane's sixteen accumulator rows (four runs of four), as vectors and once: read one
+  // by one between the tile stores below, each read would wait out its own round trip to LDS (the stores might alias it).
+  floatx4 gi[4], bi[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int i0 = 32 * wi + 8 * q + 4 * (lane >> 5);
+    gi[q] = load4(sG + i0);
+    bi[q] = load4(sBeta + i0);
+  }
+  const float gC = sG[63];
   {
     floatx16 pe[1][1];
+    const int j = 32 * wj + frag_col(lane);
+    const float gj = sG[j];
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int i = 32 * wi + frag_row(e, lane), j = 32 * wj + frag_col(lane);
-      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(sG[i] - sG[j], 0.f));
+      const int i = 32 * wi + frag_row(e, lane);
+      const float dec = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gi[e >> 2][e & 3] - gj, 0.f));
       pe[0][0][e] = (i >= j) ? p.scale * dec * aP[0][0][e] : 0.f;
       aA[0][0][e] = (i > j) ? -dec * aA[0][0][e] : 0.f;  // dXa
     }
@@ -1028,15 +1040,14 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     frag_store_t<T, 1, 1>(pe, sPeT + 32 * wj * LDC + 32 * wi, LDC, lane);
     frag_store<T, 1, 1>(aA, sXa + 32 * wi * LDC + 32 * wj, LDC, lane);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) aA[0][0][e] *= sBeta[32 * wi + frag_row(e, lane)];  // dXe
+    for (int e = 0; e < 16; ++e) aA[0][0][e] *= bi[e >> 2][e & 3];  // dXe
     frag_store_t<T, 1, 1>(aA, sXeT + 32 * wj * LDC + 32 * wi, LDC, lane);
   }
   lds_barrier();
-  const float gC = sG[63];
   // dq = scale e^G dQa + dPe K;   row = dXa K - e^G dK1 (in aK1)
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
-    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(sG[32 * wi + frag_row(e, lane)]);
+    const float gm = (GATE == LNX_GATE_NONE) ? 1.f : __expf(gi[e >> 2][e & 3]);
 #pragma unroll
     for (int c = 0; c < NKT; ++c) {
       aQ[0][c][e] *= p.scale * gm;
@@ -1057,15 +1068,19 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   // m_t = <k_t, row_t>;  chunk-end gate term sum_t r_t <k_t, dK2_t>;  dk <- beta row + r dK2 (in aK2)
   {
     float mv[16], tot = 0.f;
+    floatx4 kq[NKT][4];  // K at this lane's accumulator positions, one transposing read per run of four rows
+#pragma unroll
+    for (int c = 0; c < NKT; ++c)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) kq[c][q] = M::load_acc_rows(sK, LDKT, 32 * wi, q, 32 * (NKT * wj + c), lane);
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int r = 32 * wi + frag_row(e, lane);
-      const float rr = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gC - sG[r], 0.f));
-      const float bt = sBeta[r];
+      const float rr = (GATE == LNX_GATE_NONE) ? 1.f : __expf(fminf(gC - gi[e >> 2][e & 3], 0.f));
+      const float bt = bi[e >> 2][e & 3];
       mv[e] = 0.f;
 #pragma unroll
       for (int c = 0; c < NKT; ++c) {
-        const float kk = (float)sK[r * LDKT + 32 * (NKT * wj + c) + fr];
+        const float kk = kq[c][e >> 2][e & 3];
         mv[e] += kk * aK1[0][c][e];
         aK2[0][c][e] *= rr;
         tot += kk * aK2[0][c][e];
