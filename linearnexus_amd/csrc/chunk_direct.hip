@@ -890,7 +890,8 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   T* sXeT = sXa + L::kC;      // [j][i]
   T* sK = sXeT + L::kC;       // [token][dk]
   T* sQ = sK + L::kRow;
-  T* sSt = tiles;             // staging for dq, then dk, once the four small tiles are dead
+  T* sSt = tiles;             // staging for dq (over dPe, dPe^T) and dk (over dXa, dXe^T), once the four small tiles are dead
+  T* sSt2 = sXa;
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int N = p.geom.N;
@@ -1105,12 +1106,12 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     }
   }
   lds_barrier();  // the four small tiles are dead; sM and sMisc are complete
-  // dq, then dk, through the staging tile.  Thread = (token tid / 4, the 8-column groups tid % 4, tid % 4 + 4, ...): the
+  // dq and dk through their staging tiles.  Thread = (token tid / 4, the 8-column groups tid % 4, tid % 4 + 4, ...): the
   // row dots <q_t, dq_t> and <k_t, dk_t> give the gate gradient and carry the gradients through the normalisation,
   //   d/dx of x / (|x| + eps) applied to dy:  dy / (|x| + eps) - y <y, dy> / |x|.
   const int tr = tid >> 2, tq = 8 * (tid & 3);
   float dgp = 0.f;
-  auto emit = [&](const T* sIn, float fac, T* out, float sign) {
+  auto emit = [&](const T* sSt, const T* sIn, float fac, T* out, float sign) {
     float dot = 0.f;
 #pragma unroll
     for (int u = 0; u < DK; u += 32) {
@@ -1134,12 +1135,10 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     }
   };
   frag_store<T, 1, NKT>(aQ, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
+  frag_store<T, 1, NKT>(aK2, sSt2 + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
   lds_barrier();
-  emit(sQ, sNq[tr], p.dq, 1.f);
-  lds_barrier();  // dq has left the staging tile
-  frag_store<T, 1, NKT>(aK2, sSt + 32 * wi * LDK + 32 * NKT * wj, LDK, lane);
-  lds_barrier();
-  emit(sK, sNk[tr], p.dk, -1.f);
+  emit(sSt, sQ, sNq[tr], p.dq, 1.f);
+  emit(sSt2, sK, sNk[tr], p.dk, -1.f);
   if (GATE == LNX_GATE_SCALAR) {
     if ((tid & 3) == 0) {
       float d = dgp + 2.f * sBeta[tr] * sM[tr];
