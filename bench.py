@@ -8,6 +8,12 @@ bf16 q/k/v/dO, fp32 beta/g, chunk 64 (benchmark configuration 2).  One "step" is
 plus one backward pass through the public ops (``gated_delta_rule_chunkwise`` + autograd),
 inputs resident in HBM.  Prints ONE JSON line; ``value`` is tokens/s = B*T / step time.
 
+Before the W warm-up steps the workload runs untimed for ``--clock-warmup-seconds`` (default 2): the
+shader clock of an idle MI355X sits near 100 MHz and takes about two seconds of load to reach
+its 2.4 GHz, so W = 5 steps (5 ms) followed by 20 timed ones would time the ramp, not the
+kernels.  The JSON line says how long and how many steps that was (``clock_warmup``); the
+timed region is still exactly K steps.
+
 ``roofline`` describes the kernel with the largest share of the step, timed with HIP events
 recorded by the library on the launch stream during the timed steps; ``achieved`` is that
 kernel's algorithmic FLOP/s (or bytes/s).  ``cpu_baseline`` times the CPU restatement of the
@@ -29,6 +35,23 @@ C = 64
 PEAK_BF16 = 2500.0  # TFLOP/s, dense bf16 MFMA, MI355X
 PEAK_HBM = 8000.0   # GB/s
 PEAK_FP32_MFMA = 157.3  # TFLOP/s
+CLOCK_WARMUP_S = 2.0    # set from --clock-warmup-seconds
+
+
+def clock_warmup(torch, fn, seconds=None):
+    """Runs fn untimed until `seconds` of wall clock have passed (the GPU's clocks leave their idle state); returns
+    the number of calls."""
+    seconds = CLOCK_WARMUP_S if seconds is None else min(seconds, CLOCK_WARMUP_S)
+    n = 0
+    if seconds <= 0:
+        return n
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+        n += 8
+    return n
 
 def sources_sha256(files):
     """Hash of the named kernel sources, so that counter figures are only quoted for the code they were taken on."""
@@ -195,6 +218,7 @@ def bench_chunk(args, torch, la, _lib, name):
         if backward:
             o.backward(dO.to(o.dtype))
 
+    n_clock = clock_warmup(torch, step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -216,6 +240,7 @@ def bench_chunk(args, torch, la, _lib, name):
     fwd_only_ms = float("nan")
     if not args.no_forward_only:
         with torch.no_grad():
+            clock_warmup(torch, forward, 0.25)
             for _ in range(2):
                 forward()
             torch.cuda.synchronize()
@@ -245,6 +270,8 @@ def bench_chunk(args, torch, la, _lib, name):
         "value": B * T / dtm, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dtm * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if fp32 else "bf16", "data": "synthetic",
+        "clock_warmup": {"seconds": CLOCK_WARMUP_S, "steps": n_clock,
+                         "why": "untimed steps before the W warm-up steps: the idle shader clock (about 100 MHz) needs about 2 s of load to reach 2.4 GHz"},
         "config": {"workload": name + ("_fwd_bwd" if backward else "_fwd"), "variant": variant, "B": B, "H": H, "T": T,
                    "dk": d, "dv": dv, "chunk": C, "packed_sequences": nseq, "initial_state": s0 is not None,
                    "use_qk_l2norm": l2norm,
@@ -279,6 +306,7 @@ def bench_decode(args, torch, la, _lib, steps=None):
     steps = steps or 1000
 
     def timed(fn):
+        clock_warmup(torch, fn, 0.5)
         for _ in range(20):
             fn()
         torch.cuda.synchronize()
@@ -324,6 +352,7 @@ def bench_conv(torch, la, _lib, steps, warmup):
         y, _ = la.depthwise_conv1d_causal(x, w, None, activation="silu")
         y.backward(dy)
 
+    clock_warmup(torch, step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -360,6 +389,7 @@ def bench_dplr_step(torch, la, _lib, steps):
     q, k, v = (rn(B, H, d).to("cuda:0").bfloat16() for _ in range(3))
     a, b = ((rn(B, H, d) * 0.1).to("cuda:0").bfloat16() for _ in range(2))
     gk = (-rn(B, H, d).abs() * 0.1).to("cuda:0")
+    clock_warmup(torch, lambda: la.dplr_delta_rule_step(q, k, v, a, b, gk, S, inplace=True), 0.5)
     for _ in range(20):
         la.dplr_delta_rule_step(q, k, v, a, b, gk, S, inplace=True)
     torch.cuda.synchronize()
@@ -400,6 +430,7 @@ def bench_dplr_train(torch, la, _lib, steps, warmup):
             t.grad = None
         o, _ = la.dplr_delta_rule_recurrent(q, k, v, a, b, gk, d ** -0.5)
         o.backward(dO)
+    clock_warmup(torch, step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -439,6 +470,7 @@ def bench_rmsnorm_gated(torch, la, _lib, steps, warmup):
         x.grad = g.grad = w.grad = None
         la.rmsnorm_gated(x, g, w).backward(dy)
 
+    clock_warmup(torch, step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -479,6 +511,7 @@ def bench_kda_gate(torch, la, _lib, steps, warmup):
         g, _ = la.kda_gate(raw, A, dk, bias, out_dtype=torch.float32)
         g.backward(dy)
 
+    clock_warmup(torch, step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -570,12 +603,17 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "dplr_train", "rmsnorm_gated", "kda_gate", "prefill_long"])
+    ap.add_argument("--clock-warmup-seconds", type=float, default=2.0,
+                    help="untimed run of the workload before the W warm-up steps, so that the timed steps see the GPU's "
+                         "clocks at their loaded level and not on the way up from idle (0: none; counter runs use that)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-forward-only", action="store_true",
                     help="skip the extra forward-without-gradients timing (profiler runs: keeps the per-kernel averages to the differentiable step)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 512 MiB device copy (known traffic) so that a counter run can be scaled")
     args = ap.parse_args()
+    global CLOCK_WARMUP_S
+    CLOCK_WARMUP_S = max(0.0, args.clock_warmup_seconds)
     if args.gpus != 1:
         print("bench.py measures one GPU only: the scan needs no collective and every figure here is "
               "single-GPU; run with --gpus 1", file=sys.stderr)

@@ -438,10 +438,12 @@ class _ChunkScan(torch.autograd.Function):
     """Pairs lnx_chunk_fwd with lnx_chunk_bwd (the role ``jax.custom_vjp`` plays for a JAX caller)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens):
-        # nothing to differentiate (inference, torch.no_grad()): the kernels skip what only the backward reads
+    def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, grad_mode=True):
+        # nothing to differentiate (inference): the kernels skip what only the backward reads.  `grad_mode` is the
+        # caller's torch.is_grad_enabled() -- inside forward() it is always off, and needs_input_grad alone is still set
+        # for leaves that require grad under torch.no_grad()
         o, sT, saved, meta = _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens,
-                                            forward_only=not any(ctx.needs_input_grad))
+                                            forward_only=not (grad_mode and any(ctx.needs_input_grad)))
         ctx.save_for_backward(*saved)
         ctx.meta = meta
         return o, sT
@@ -475,7 +477,7 @@ class _ChunkScan(torch.autograd.Function):
         dbeta = dbeta.to(beta_dt)
         if dg is not None:
             dg = dg.to(g_dt)
-        return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None
+        return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None, None
 
 
 _CHUNK_DK = (64, 128, 256)  # key head dimensions the chunk kernels are built for
@@ -527,7 +529,7 @@ def _segmented_forward(q, k, v, g, beta, scale, initial_state, l2norm, o_dtype, 
         s_in[i] = cur
         if i + 1 < nseg:
             cur = torch.baddbmm(Bs[i], As[i], cur)
-    o, sT = _ChunkScan.apply(q1, k1, v1, g1, beta1, s_in, scale, l2norm, o_dtype, cu)
+    o, sT = _ChunkScan.apply(q1, k1, v1, g1, beta1, s_in, scale, l2norm, o_dtype, cu, torch.is_grad_enabled())
     return o.reshape(B, H, T, dv), sT[nseg - 1].reshape(B, H, dk, dv)
 
 
@@ -551,7 +553,7 @@ def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, 
             nseg = _prefill_segments(q.shape[0], q.shape[1], q.shape[2], dv)
             if nseg > 1:
                 return _segmented_forward(q, k, v, g, beta, scale, initial_state, l2norm, o_dtype, nseg)
-        return _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+        return _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, torch.is_grad_enabled())
     # Head dimensions between the kernels' sizes (the reference's own tests use dk = 8, 16, dv = 8, 32):
     # zero channels are exact.  A zero key/query channel adds nothing to any <q,k>, <k,k> or |x|_2, the state rows
     # and columns it would feed stay zero, and the padded value columns are independent of the others; autograd
@@ -562,7 +564,7 @@ def _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, l2norm, o_dtype, 
         g = pad(g, (0, dkp - dk))
     if initial_state is not None:
         initial_state = pad(initial_state, (0, dvp - dv, 0, dkp - dk))
-    o, sT = _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens)
+    o, sT = _ChunkScan.apply(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, torch.is_grad_enabled())
     return o[..., :dv], sT[..., :dk, :dv]
 
 
