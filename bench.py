@@ -677,6 +677,13 @@ def main():
         del a, b
     out, (B, H, T, d) = bench_chunk(args, torch, la, _lib, args.workload)
     if args.workload == "gdn_chunk":
+        if not args.no_forward_only:
+            # the same step through the reference's default use_qk_l2norm=True, on rows that are not normalised
+            torch.cuda.empty_cache()
+            l2, _ = bench_chunk(args, torch, la, _lib, "gdn_chunk_l2norm")
+            out["use_qk_l2norm_true"] = {k_: l2[k_] for k_ in ("ms_per_step", "value", "unit", "kernel_ms", "forward_only_ms")}
+            del l2
+            torch.cuda.empty_cache()
         out["decode_step"] = bench_decode(args, torch, la, _lib)
     if not args.no_cpu_baseline and args.workload == "gdn_chunk":
         out["cpu_baseline"] = cpu_baseline_chunk(torch, B, H, T, d, 2)
