@@ -176,3 +176,38 @@ def test_unsupported_dims_raise_runtime_error():
     q = torch.randn(1, 1, 64, 272, device=DEV)  # key heads wider than 256 (narrower ones are embedded with zero channels)
     with pytest.raises(RuntimeError):
         la.delta_rule_chunkwise(q, q, torch.randn(1, 1, 64, 64, device=DEV), torch.ones(1, 1, 64, device=DEV))
+
+
+@pytest.mark.parametrize("gate", ["none", "scalar", "vector"])
+def test_no_grad_with_leaves_that_require_grad_is_the_forward_only_path(gate, monkeypatch):
+    """Evaluation of a model whose parameters require grad, under torch.no_grad(): the op must not save for a backward
+    pass (it used to, going by the leaves alone) and must return what the differentiable call returns, bit for bit."""
+    import linearnexus_amd as la
+    from linearnexus_amd import linear_attn
+    x, dt = _prep(make_inputs(31, 2, 2, 200, 128, 128, gate=gate, with_state=True), True)
+    q, k, v = _t(x["q"], dt), _t(x["k"], dt), _t(x["v"], dt)
+    beta, s0 = _t(x["beta"]), _t(x["S0"])
+    g = _t(x["g"]) if gate != "none" else None
+    for t in (q, k, v, beta, s0) + ((g,) if g is not None else ()):
+        t.requires_grad_(True)
+
+    def call():
+        if gate == "none":
+            return la.delta_rule_chunkwise(q, k, v, beta, s0)
+        fn = la.gated_delta_rule_chunkwise if gate == "scalar" else la.kda_chunkwise
+        return fn(q, k, v, g, beta, None, s0, 64, False)
+
+    seen = []
+    inner = linear_attn._chunk_forward
+
+    def spy(*a, forward_only, **kw):
+        seen.append(forward_only)
+        return inner(*a, forward_only=forward_only, **kw)
+
+    monkeypatch.setattr(linear_attn, "_chunk_forward", spy)
+    o1, s1 = call()
+    with torch.no_grad():
+        o2, s2 = call()
+    assert seen == [False, True]
+    assert o1.requires_grad and not o2.requires_grad
+    assert torch.equal(o1.detach(), o2) and torch.equal(s1.detach(), s2)
