@@ -675,6 +675,11 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
+    cpu = None
+    if not args.no_cpu_baseline and args.workload == "gdn_chunk":
+        # the CPU leg first: the GPU legs then run back to back up to the end of the process
+        _, cB, cH, cT, cd = CHUNK_CONFIGS["gdn_chunk"][:5]
+        cpu = cpu_baseline_chunk(torch, cB, cH, cT, cd, 2)
     out, (B, H, T, d) = bench_chunk(args, torch, la, _lib, args.workload)
     if args.workload == "gdn_chunk":
         if not args.no_forward_only:
@@ -685,8 +690,8 @@ def main():
             del l2
             torch.cuda.empty_cache()
         out["decode_step"] = bench_decode(args, torch, la, _lib)
-    if not args.no_cpu_baseline and args.workload == "gdn_chunk":
-        out["cpu_baseline"] = cpu_baseline_chunk(torch, B, H, T, d, 2)
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 

@@ -92,6 +92,11 @@ typedef struct lnx_scan_args {
                                    are not read.  0 = all dv.  With forward_only, o may also be NULL: only the final
                                    states are wanted.  (Transition matrices of sequence segments: value columns
                                    [v | 0], initial states [0 | I].) */
+
+  /* Test hooks (ABI version 8); a binding leaves both 0 = the library's choice.  Neither changes results or the
+     workspace layout, only which of two tilings of the same kernel runs, so that tests reach both at small shapes. */
+  int32_t test_scan_slab;       /* 32 or 64: value columns per workgroup of the sequential kernels */
+  int32_t test_out_slabs;       /* > 0: value slabs per workgroup of the fp32 output kernel */
 } lnx_scan_args;
 
 /* Library identification; also the symbol a loader probes first. */
@@ -118,7 +123,9 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  * Chunked (WY) forward on MFMA.  Replaces delta_rule_chunkwise (delta_net.py:216-354),
  * gated_delta_rule_chunkwise (gated_deltanet.py:232-534), kda_chunkwise (kda.py:350-655).
  * The workspace keeps the per-chunk tensors the backward pass re-uses; pass the same
- * workspace, unchanged, to lnx_chunk_bwd (unless forward_only was set).
+ * workspace, unchanged, to lnx_chunk_bwd (unless forward_only was set), with the same shape, dtype, gate, nseq,
+ * token_first, scale and use_qk_l2norm fields: the layout of the workspace follows from B, H, T, dk, dv, dtype, gate
+ * and nseq alone (o_dtype does not enter it), and there is exactly one set of kernels per such shape.
  * Shapes: dk in {64, 128, 256} (256 is the head_dim of the reference's Gated DeltaNet presets,
  * models.py:142-143), dv a multiple of 64.
  */
@@ -127,7 +134,7 @@ int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);
 /*
  * 1 when lnx_chunk_fwd / lnx_chunk_bwd apply the in-op normalisation of q and k themselves for these arguments
  * (use_qk_l2norm = 1: gated_deltanet.py:273-275, kda.py:379-381 normalise inside the op, and it is their default):
- * element types bf16, dk <= 128, no per-channel gate.  The rows are scaled where the kernels stage them and the
+ * q, k, v in bf16, dk <= 128, no per-channel gate.  The rows are scaled where the kernels stage them and the
  * backward pass carries d_q, d_k through the normalisation, so no normalised copies of q and k exist.  0: the chunk
  * entry points refuse use_qk_l2norm for these arguments; normalise with lnx_l2norm_fwd first.
  */
@@ -142,8 +149,15 @@ int lnx_chunk_fuses_l2norm(const lnx_scan_args* a);
  * or other allocating routine.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
  * (two streams, two threads) race and must be serialised by the caller.  No counterpart in the reference, whose
  * JAX ops leave allocation to XLA.
+ * For bf16 inputs with dk <= 128 and no per-channel gate the scratch takes 17 KiB per 64-token chunk of every
+ * (batch, head) row, so B * H * ceil(T / 64) <= 3855 chunks fit (8 heads of 30720 tokens; a packed batch counts
+ * T / 64 + nseq chunks per head); the other shapes also keep W and U there, (dk + dv) * 128 bytes more per chunk (twice
+ * that for fp32); lnx_chunk_workspace_bytes with forward_only = 1 gives the exact figure.  The address of the array on the current device is looked up on the first call on
+ * that device; a caller that will make its first call while its stream is capturing calls lnx_chunk_fwd_static_init()
+ * once per device beforehand, outside the capture (it launches nothing).
  */
 #define LNX_STATIC_SCRATCH_BYTES (64u << 20)
+int lnx_chunk_fwd_static_init(void);
 int lnx_chunk_fwd_static(const lnx_scan_args* a, void* hip_stream);
 
 /*
@@ -301,7 +315,9 @@ int lnx_sigmoid_bwd(const float* y, const float* dy, float* dx, int64_t n, void*
  * every entry point records HIP events around each kernel it launches, on the caller's stream.
  * lnx_profile_read waits for them, returns the number of kernels timed since the last read and
  * fills up to `capacity` (name, milliseconds) pairs.  At most 8192 marks (one per kernel plus one
- * per entry-point call) are kept between reads.
+ * per entry-point call) are kept between reads.  This is the one piece of process-wide mutable state in the
+ * library (a mutex-guarded list of events, created on first use); it is off unless enabled, and calls on a
+ * stream that is being captured into a graph take no marks, so the compute entry points stay capturable.
  */
 int lnx_profile_enable(int on);
 int lnx_profile_read(int capacity, const char** names, float* ms);

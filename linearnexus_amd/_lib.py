@@ -16,7 +16,7 @@ GATE_NONE, GATE_SCALAR, GATE_VECTOR = 0, 1, 2
 
 EXPORTS = (
     "lnx_abi_version", "lnx_last_error", "lnx_decode_step", "lnx_recurrent_fwd",
-    "lnx_chunk_workspace_bytes", "lnx_chunk_fuses_l2norm", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
+    "lnx_chunk_workspace_bytes", "lnx_chunk_fuses_l2norm", "lnx_chunk_fwd", "lnx_chunk_fwd_static", "lnx_chunk_fwd_static_init", "lnx_chunk_bwd", "lnx_l2norm_fwd", "lnx_l2norm_bwd",
     "lnx_conv1d_fwd", "lnx_conv1d_bwd", "lnx_conv1d_cache_bwd", "lnx_conv1d_packed_fwd", "lnx_conv1d_packed_bwd", "lnx_dplr_recurrent_fwd", "lnx_dplr_step", "lnx_dplr_recurrent_bwd", "lnx_dplr_recurrent_bwd_workspace_bytes", "lnx_rmsnorm_gated_fwd", "lnx_rmsnorm_gated_bwd", "lnx_rmsnorm_gated_bwd_workspace_bytes",
     "lnx_gdn_gate_fwd", "lnx_gdn_gate_bwd", "lnx_gdn_gate_bwd_workspace_bytes", "lnx_kda_gate_fwd", "lnx_kda_gate_bwd", "lnx_kda_gate_bwd_workspace_bytes", "lnx_sigmoid_fwd", "lnx_sigmoid_bwd",
     "lnx_profile_enable", "lnx_profile_read",
@@ -38,6 +38,7 @@ class ScanArgs(C.Structure):
         ("d_v", C.c_void_p), ("d_beta", C.c_void_p), ("d_g", C.c_void_p), ("d_initial_state", C.c_void_p),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
         ("value_cols", C.c_int32),
+        ("test_scan_slab", C.c_int32), ("test_out_slabs", C.c_int32),
     ]
 
 
@@ -82,6 +83,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(ScanArgs), C.c_void_p]
+    lib.lnx_chunk_fwd_static_init.restype = C.c_int
+    lib.lnx_chunk_fwd_static_init.argtypes = []
     lib.lnx_chunk_workspace_bytes.restype = C.c_uint64
     lib.lnx_chunk_workspace_bytes.argtypes = [C.POINTER(ScanArgs)]
     lib.lnx_chunk_fuses_l2norm.restype = C.c_int

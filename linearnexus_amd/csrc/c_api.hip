@@ -20,7 +20,7 @@ int lnx_set_error(int code, const char* fmt, ...) {
 }
 
 extern "C" const char* lnx_last_error(void) { return g_error; }
-extern "C" int lnx_abi_version(void) { return 7; }
+extern "C" int lnx_abi_version(void) { return 8; }
 
 // ---- optional per-kernel timing with HIP events on the caller's stream.  Process-wide (one
 // mutex-guarded list) because a framework may run the backward entry point on another thread. ----
@@ -41,6 +41,9 @@ void lnx_profile_mark(const char* kernel_name, hipStream_t st) {
   if (!P.on) return;  // unguarded fast path: timing is off in normal use
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   if (!P.on || P.n > LNX_PROFILE_MAX) return;
+  // a capturing stream takes no marks: an event created or recorded here would become part of the caller's graph
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return;
   if (kernel_name != nullptr && P.n == LNX_PROFILE_MAX) return;  // keep one slot for the closing mark
   if (P.created <= P.n) {
     if (hipEventCreate(&P.ev[P.created]) != hipSuccess) return;

@@ -30,6 +30,7 @@ struct BwdParams {
   float* dg;
   float* ds0;
   int dv, gate;
+  int slab;  // lnx_scan_args.test_scan_slab
   float scale;
   char* ws;
   ChunkWs off;
@@ -58,7 +59,6 @@ __global__ __launch_bounds__(256) void bwd_local_kernel(BwdParams p) {
   chunk_span(p.geom, n, tok0, len);
   if (len <= 0) return;
   const int64_t tbase = tok_index(p.geom, row, tok0);
-  if (v0 == 0 && tid < 64 && p.gate == LNX_GATE_SCALAR) wsp<float>(p, p.off.dG)[slot * 64 + tid] = 0.f;  // accumulated by bwd_dqk
   TileRegs<T, 64, 64> rP, rdO;
   rP.load(wsp<T>(p, p.off.P) + slot * 64 * 64, 64, 64, tid);
   rdO.load(reinterpret_cast<const T*>(p.d_o) + tbase * p.dv + v0, (int64_t)p.geom.ts * p.dv, len, tid);
@@ -301,7 +301,6 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       for (int n = c1 - 1; n >= c0; --n) {
         const int64_t slot = (int64_t)row * N + n;
         if (n - 1 >= c0) fetch_main(n - 1);
-        if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
         unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
         lds_barrier();  // B2
         rQ.store(sQ, LDK, mt);
@@ -412,7 +411,6 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
           commit_rest(nxt, pb ^ 1);
         }
       }
-      if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
       lds_barrier();  // B2
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       unstage_tile<T, 64, BV, true>(wsp<T>(p, p.off.dD) + slot * 64 * p.dv + v0, p.dv, sdDl, LDU, 64, mt);
@@ -427,7 +425,6 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
       const int64_t slot = (int64_t)row * N + n;
       const bool more = n - AHEAD >= c0;  // chunk n's registers are free again: they take chunk n - AHEAD
       if (more) fetch(cur, n - AHEAD, AHEAD == 2 ? 0 : -1);
-      if (FUSE && GATE == LNX_GATE_SCALAR && v0 == 0 && mt < 64) wsp<float>(p, p.off.dG)[slot * 64 + mt] = 0.f;  // accumulated by bwd_dqk
       unstage_tile<T, BV, DK, true>(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sdST, LDK, BV, mt);
       lds_barrier();  // B2
       if (n - 1 >= c0) nxt.K.store(sK, LDK, mt);
@@ -606,7 +603,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
   extern __shared__ __align__(16) char smem[];
   float* sG = reinterpret_cast<float*>(smem);
   float* sSS = sG + 64;     // vector gate: per key channel sum_v dS_n[c][v] S_n[c][v]
-  float* sMisc = sSS + 64;  // [0] = sum_j r_j <dKr_j, k_j>, [1] = <dS_n, S_n>
+  float* sMisc = sSS + 64;  // scalar gate: [4 + wave] = the wave's share of sum_j r_j <dKr_j, k_j>, [8 + wave] = of <dS_n, S_n>
   float* sR = sMisc + 64;   // vector gate only: dP [64][LNX_LDA]
   T* sdO = reinterpret_cast<T*>(sMisc + 64 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0));
   T* sD = sdO + L::kLoop;
@@ -690,7 +687,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     if ((tid & 3) == 0) sSS[tid >> 2] = ss;
   } else if (GATE == LNX_GATE_SCALAR) {
     ss = wave_sum(ss);
-    if (lane == 0) atomicAdd(&sMisc[1], ss);
+    if (lane == 0) sMisc[8 + wave] = ss;  // one slot per wave, added in a fixed order where the sum is used
   }
   lds_barrier();  // slab tiles are dead from here on
 
@@ -755,12 +752,15 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
       sOut[r * LDF + c] = aK[0][0][e] * __expf(fminf(sAl[63 * LDF + c] - sAl[r * LDF + c], 0.f));
     }
     lds_barrier();
-    {  // chunk-end gate term per channel: sum_r out[r][c] k[r][c], sixteen rows per wave (sMisc is zero: unused here)
-      const int c = tid & 63, r0 = 16 * (tid >> 6);
+    {  // chunk-end gate term per channel: sum_r out[r][c] k[r][c].  A wave owns sixteen channels, lane group lane / 16
+       // the rows congruent to it mod 4, and the four groups meet through two shuffles: no atomics, one order of addition
+      const int c = 16 * wave + (lane & 15), rq = lane >> 4;
       float part = 0.f;
 #pragma unroll
-      for (int r = r0; r < r0 + 16; ++r) part += sOut[r * LDF + c] * to_f32(sKr[r * LDC + c]);
-      atomicAdd(&sMisc[c], part);
+      for (int j = 0; j < 16; ++j) part += sOut[(4 * j + rq) * LDF + c] * to_f32(sKr[(4 * j + rq) * LDC + c]);
+      part += __shfl_xor(part, 16, LNX_WAVE);
+      part += __shfl_xor(part, 32, LNX_WAVE);
+      if (lane < 16) sMisc[c] = part;
     }
     lds_barrier();
     if (tid < 64) sSS[tid] = sMisc[tid] + __expf(sAl[63 * LDF + tid]) * sSS[tid];  // added to row 63 below
@@ -825,7 +825,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     mma_x<T, 1, 1, true, true>(aK, sPe + 32 * wi, LDC, sQr + 32 * wj, LDC, 64, lane);
     if (GATE != LNX_GATE_NONE) {
       tot = wave_sum(tot);
-      if (lane == 0) atomicAdd(&sMisc[0], tot);
+      if (lane == 0) sMisc[4 + wave] = tot;
     }
     lds_barrier();  // all reads of sPe / sOut done
     frag_store<T, 1, 1>(aQ, sPe + 32 * wi * LDC + 32 * wj, LDC, lane);
@@ -848,8 +848,9 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
       d += __shfl_xor(d, 1, LNX_WAVE);
       d += __shfl_xor(d, 2, LNX_WAVE);
       if ((tid & 3) == 0) {
-        if (r == 63) d += sMisc[0] + __expf(gl) * sMisc[1];
-        unsafeAtomicAdd(&wsp<float>(p, p.off.dG)[slot * 64 + r], d);  // hardware fp32 atomic: the two channel halves share dG
+        if (r == 63) d += ((sMisc[4] + sMisc[5]) + (sMisc[6] + sMisc[7])) + __expf(gl) * ((sMisc[8] + sMisc[9]) + (sMisc[10] + sMisc[11]));
+        // one slot per 64-channel part; bwd_wy2 adds the parts in order (no atomics: the same bits from run to run)
+        wsp<float>(p, p.off.dG)[((int64_t)part * p.geom.rows * N + slot) * 64 + r] = d;
       }
     }
   }
@@ -995,7 +996,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       }
       t += __shfl_xor(t, 1, LNX_WAVE);
       t += __shfl_xor(t, 2, LNX_WAVE);
-      if ((tid & 3) == 0) atomicAdd(&(is_k ? sdGk : sdB)[r], t);
+      if ((tid & 3) == 0) (is_k ? sdGk : sdB)[r] += t;  // row r has this one writer in every phase
     }
     if (!is_k) {  // dv = beta dBu, 16-byte stores
       constexpr int VN = Vec16<T>::N;
@@ -1045,7 +1046,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       }
       rs += __shfl_xor(rs, 1, LNX_WAVE);
       rs += __shfl_xor(rs, 2, LNX_WAVE);
-      if ((tid & 3) == 0) atomicAdd(&sdB[r], rs);
+      if ((tid & 3) == 0) sdB[r] += rs;
     }
 #pragma unroll 1
     for (int h = 0; h < DK / 64; ++h) {
@@ -1103,7 +1104,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         }
         t += __shfl_xor(t, 1, LNX_WAVE);
         t += __shfl_xor(t, 2, LNX_WAVE);
-        if ((tid & 3) == 0) atomicAdd(&sdB[r], t);
+        if ((tid & 3) == 0) sdB[r] += t;
       }
       lds_barrier();
       float pr[16], pc[16];
@@ -1198,6 +1199,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       y[0][0][e] = sBeta[i] * da;
     }
     frag_store<T, 1, 1>(y, sYa + 32 * wi * LDC + 32 * wj, LDC, lane);
+    // two waves add to each entry of sRow (wj = 0, 1) and of sCol (wi = 0, 1), both zeroed above: 0 + a + b is the same
+    // number in either order, so these sums do not depend on which wave arrives first
     rows_reduce_add<1>(v, 32 * wi, lane, sRow);
     cs += __shfl_xor(cs, 32, LNX_WAVE);
     if (lane < 32) atomicAdd(&sCol[32 * wj + lane], cs);
@@ -1245,7 +1248,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
     const float w = gm * sdGk[t], rs = sRow[t];
     if (t < len) p.dbeta[tbase + t * ts] = sdB[t] + w + rs;
     if (GATE != LNX_GATE_NONE) {
-      float d = wsp<float>(p, p.off.dG)[slot * 64 + t] + sBeta[t] * (w + rs) - sCol[t];
+      float d = 0.f;  // bwd_dqk's share, one slot per 64-channel part
+#pragma unroll
+      for (int part = 0; part < DK / 64; ++part) d += wsp<float>(p, p.off.dG)[((int64_t)part * p.geom.rows * p.geom.N + slot) * 64 + t];
+      d += sBeta[t] * (w + rs) - sCol[t];
 #pragma unroll
       for (int s_ = 1; s_ < 64; s_ <<= 1) {
         const float y = __shfl_down(d, s_, LNX_WAVE);
@@ -1264,7 +1270,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   // dk >= 128, 4-byte inputs with dk = 128; 4-byte inputs with dk = 256 always get 32 columns from BScanCfg)
   constexpr bool can_narrow = (DK >= 128 && sizeof(T) == 2) || (DK == 128 && sizeof(T) == 4);
   constexpr int WIDE = 64, NARROW = can_narrow ? 32 : WIDE;
-  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64), p.slab);
   auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, NARROW> : bwd_scan_kernel<T, DK, GATE, WIDE>;
   const int bv = narrow ? BScanCfg<T, DK, NARROW>::BV : BScanCfg<T, DK, WIDE>::BV;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
@@ -1334,14 +1340,14 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.geom.tab = packed ? reinterpret_cast<const int32_t*>(reinterpret_cast<char*>(a->workspace) + w.tab) : nullptr;
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.d_o = a->d_o; p.d_sT = a->d_final_state;
   p.dq = a->d_q; p.dk = a->d_k; p.dv_out = a->d_v; p.dbeta = a->d_beta; p.dg = a->d_g; p.ds0 = a->d_initial_state;
-  p.dv = a->dv; p.gate = a->gate; p.scale = a->scale;
+  p.dv = a->dv; p.gate = a->gate; p.scale = a->scale; p.slab = a->test_scan_slab;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (lnx_chunk_direct(a)) {
     DirectParams d = {};
     d.geom = p.geom;
     d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
     d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.dv = a->dv; d.vcols = a->dv; d.gate = a->gate;
-    d.l2norm = a->use_qk_l2norm;
+    d.l2norm = a->use_qk_l2norm; d.slab = a->test_scan_slab;
     d.scale = a->scale; d.ws = p.ws; d.off = w;
     d.d_o = reinterpret_cast<const bf16_t*>(a->d_o); d.d_sT = a->d_final_state;
     d.dq = reinterpret_cast<bf16_t*>(a->d_q); d.dk = reinterpret_cast<bf16_t*>(a->d_k);
@@ -1352,10 +1358,10 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
     if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk backward launch: %s", hipGetErrorString(e));
     return LNX_OK;
   }
-  if (a->dtype == LNX_BF16)
+  if (a->dtype == LNX_BF16)  // dk <= 128 without a per-channel gate went to the direct-solve kernels above
     rc = (a->dk == 256)   ? launch_bwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
-         : (a->dk == 128) ? launch_bwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
-                          : launch_bwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+         : (a->dk == 128) ? launch_bwd<bf16_t, 128, LNX_GATE_VECTOR>(p, nstate, st)
+                          : launch_bwd<bf16_t, 64, LNX_GATE_VECTOR>(p, nstate, st);
   else
     rc = (a->dk == 256)   ? launch_bwd_gate<float, 256>(a->gate, p, nstate, st)
          : (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st)

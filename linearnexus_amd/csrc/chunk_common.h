@@ -22,8 +22,6 @@
 // and dG (fp32 partial gradient of the cumulative gate).
 #pragma once
 
-#include <stdlib.h>
-
 #include "mma_tiles.h"
 
 struct ChunkGeom {
@@ -108,13 +106,12 @@ struct ChunkWs {
   uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, Nq, Nk, Fq, TmT, D, SnT, dD, dSn, dW, dG, total;
 };
 
-// 2-byte inputs and outputs with dk <= 128 and no per-channel gate take the kernels of chunk_direct.hip, which keep G, Pm,
-// Tm, the per-chunk states and state gradients, D and dR in the workspace (no W, U, dW).  LNX_CHUNK_DIRECT=0 in the environment sends them through the
-// general kernels instead (used by the tests to keep those covered at small shapes).
+// 2-byte inputs with dk <= 128 and no per-channel gate take the kernels of chunk_direct.hip, which keep G, Pm, Tm, the
+// per-chunk states and state gradients, D and dR in the workspace (no W, U, dW); every other shape takes the WY-split
+// kernels.  The choice reads only fields that the forward and the backward call of one step necessarily share (element
+// type, dk, gate kind), so both calls lay the workspace out the same way; there is one set of kernels per shape.
 inline bool lnx_chunk_direct(const lnx_scan_args* a) {
-  if (a->dtype != LNX_BF16 || a->o_dtype != LNX_BF16 || a->dk > 128 || a->gate == LNX_GATE_VECTOR) return false;
-  const char* e = getenv("LNX_CHUNK_DIRECT");
-  return !(e && e[0] == '0');
+  return a->dtype == LNX_BF16 && a->dk <= 128 && a->gate != LNX_GATE_VECTOR;
 }
 
 inline uint64_t lnx_align256(uint64_t x) { return (x + 255) & ~uint64_t(255); }
@@ -166,18 +163,17 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.dD = take(bwd ? slots * C * dv * es : 0);
   w.dSn = take(bwd ? slots * dk * dv * es : 0);
   w.dW = take(bwd ? slots * C * dk * es : 0);
-  w.dG = take(bwd ? (vec ? slots * C * dk * 4 : slots * C * 4) : 0);
+  w.dG = take(bwd ? (vec ? slots * C * dk * 4 : slots * C * 4 * (dk / 64)) : 0);  // scalar gate: one slot per 64-channel part
   w.total = off;
   return w;
 }
 
 // Slab width of the two sequential kernels: 32 columns when 64-column slabs would give workgroups to at
-// most half of the 256 CUs.  LNX_SCAN_SLAB=32 or 64 in the environment overrides the choice (used by the
-// tests to cover both variants at small shapes).
-inline bool lnx_narrow_slabs(int64_t wide_workgroups) {
-  const char* e = getenv("LNX_SCAN_SLAB");
-  if (e && e[0] == '3') return true;
-  if (e && e[0] == '6') return false;
+// most half of the 256 CUs.  `forced` is lnx_scan_args.test_scan_slab: 32 or 64 overrides the choice (the
+// tests cover both variants at small shapes with it; the workspace layout does not depend on the width).
+inline bool lnx_narrow_slabs(int64_t wide_workgroups, int forced) {
+  if (forced == 32) return true;
+  if (forced == 64) return false;
   return wide_workgroups <= 128;
 }
 
@@ -196,6 +192,7 @@ struct DirectParams {
   int vcols;  // leading value columns present in v (its row length); the rest of the dv columns are zero
   int gate;
   int l2norm;  // q and k rows are normalised inside the kernels (factors from the prepare kernel in Nq, Nk)
+  int slab;    // lnx_scan_args.test_scan_slab
   float scale;
   char* ws;
   ChunkWs off;

@@ -1,8 +1,8 @@
 // Chunked delta-rule forward and backward for 2-byte inputs with dk <= 128 and no / a scalar gate, in the
 // "direct solve" split: the only per-chunk tensors that cross kernels are Tm = (I + A)^-1, Pm = scale tril(E * Q K^T)
-// and the cumulative gate G from the chunk-parallel prepare kernel, the states entering the chunks (forward scan ->
-// chunk-local backward) and the state gradients leaving them (reverse scan -> chunk-local backward).  W, U, D, dD, dW
-// of the WY form are never materialised: with S the state entering a chunk,
+// and the cumulative gate G from the chunk-parallel prepare kernel, the states entering the chunks and D (forward scan
+// -> chunk-local backward) and the state gradients leaving them and dR (reverse scan -> chunk-local backward).  W, U,
+// dD, dW of the WY form are never materialised: with S the state entering a chunk,
 //
 //   Y = K S          R = diag(beta) (V - diag(e^G) Y)      D = Tm R                     (forward substitution applied
 //   O = scale diag(e^G) (Q S) + Pm D                                                     to the chunk's right-hand
@@ -18,8 +18,8 @@
 //
 //   scan_fwd   (one workgroup per (state, slab of dv), sequential over chunks)   O, the entering states, S_T
 //   scan_bwd   (same grid, reverse)                                              the leaving state gradients, dS_0
-//   bwd_chunk  (one workgroup per chunk, all in parallel)                         dq, dk, dv, dbeta, dg -- recomputes
-//              Y, D, dD, dR of its chunk from q, k, v, dO and the two saved states
+//   bwd_chunk  (one workgroup per chunk, all in parallel)                         dq, dk, dbeta, dg from q, k, v, dO, the
+//              two saved states and D, dR as the scans left them (dv leaves the reverse scan)
 //
 // Both scans split their 512 threads into four compute waves (matrix work on the tiles in LDS, the fp32 state in MFMA
 // accumulators for the whole sequence) and four mover waves (global loads two chunks ahead into registers, tile
@@ -81,7 +81,7 @@ template <int DK, int BVW> struct FScanL {
   static constexpr int threads = 64 * NCW + 256;
 };
 
-template <int DK, int GATE, int BVW>
+template <int DK, int GATE, int BVW, typename OT>
 __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(DirectParams p) {
   typedef FScanL<DK, BVW> L;
   constexpr int LDK = L::LDK, LDC = L::LDC, BV = L::BV, LDV = L::LDV, NCW = L::NCW;
@@ -228,8 +228,12 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
       lds_barrier();  // Bmid
       int tok0, len;
       chunk_span(span, n, tok0, len);
-      if (p.o)
-        unstage_tile_checked<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
+      if (p.o) {
+        if constexpr (std::is_same<OT, float>::value)
+          unstage_tile_checked_widen<64, BV>(reinterpret_cast<float*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
+        else
+          unstage_tile_checked<bf16_t, 64, BV>(reinterpret_cast<bf16_t*>(p.o) + tok_index(p.geom, row, tok0) * p.dv + v0, tso, sO, LDV, len, mt);
+      }
       if (p.save) {
         const int64_t slot = (int64_t)row * N + n;
         unstage_tile<T, BV, DK, true>(at<T>(p.ws, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, sST, LDK, BV, mt);
@@ -449,11 +453,11 @@ __global__ __launch_bounds__((FScanL<DK, BVW>::threads)) void scan_fwd_kernel(Di
     for (int e = 0; e < 16; ++e) out[(int64_t)(32 * ci + frag_row(e, lane)) * p.dv] = S[ci][e];
 }
 
-template <int DK, int GATE>
+template <int DK, int GATE, typename OT>
 int launch_scan_fwd(const DirectParams& p, int nstate, hipStream_t st) {
   // 32-column slabs (one compute wave) when 64-column ones would occupy at most half of the chip
-  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
-  auto k = narrow ? scan_fwd_kernel<DK, GATE, 32> : scan_fwd_kernel<DK, GATE, 64>;
+  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64), p.slab);
+  auto k = narrow ? scan_fwd_kernel<DK, GATE, 32, OT> : scan_fwd_kernel<DK, GATE, 64, OT>;
   const size_t b = narrow ? FScanL<DK, 32>::bytes : FScanL<DK, 64>::bytes;
   const int bv = narrow ? 32 : 64, threads = narrow ? FScanL<DK, 32>::threads : FScanL<DK, 64>::threads;
   hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)b);
@@ -819,7 +823,7 @@ __global__ __launch_bounds__((BScanL<DK, BVW>::threads)) void scan_bwd_kernel(Di
 
 template <int DK, int GATE>
 int launch_scan_bwd(const DirectParams& p, int nstate, hipStream_t st) {
-  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  const bool narrow = lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64), p.slab);
   auto k = narrow ? scan_bwd_kernel<DK, GATE, 32> : scan_bwd_kernel<DK, GATE, 64>;
   const size_t b = narrow ? BScanL<DK, 32>::bytes : BScanL<DK, 64>::bytes;
   const int bv = narrow ? 32 : 64, threads = narrow ? BScanL<DK, 32>::threads : BScanL<DK, 64>::threads;
@@ -872,7 +876,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   float* sRdv = sBeta + 64;   // <dR_t, v_t>
   float* sM = sRdv + 64;      // m_t
   float* sdG = sM + 64;
-  float* sMisc = sdG + 64;    // [0] = sum_t r_t <k_t, dK2_t>, [1] = <dS', S>
+  float* sMisc = sdG + 64;    // [4 + wave] = the wave's share of sum_t r_t <k_t, dK2_t>, [8 + wave] = of <dS', S>
   float* sNq = sMisc + 64;    // normalisation factors of the q and k rows (1 when the inputs come normalised)
   float* sNk = sNq + 64;
   T* tiles = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
@@ -998,7 +1002,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   if ((tid & 3) == 0) sRdv[tid >> 2] = rdv;
   if (GATE == LNX_GATE_SCALAR) {
     ss = wave_sum(ss);
-    if (lane == 0) atomicAdd(&sMisc[1], ss);
+    if (lane == 0) sMisc[8 + wave] = ss;  // one slot per wave, added in a fixed order below
   }
   lds_barrier();  // slab tiles are dead from here on
 
@@ -1088,10 +1092,10 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
         aK2[0][c][e] += bt * aK1[0][c][e];
       }
     }
-    rows_reduce_add<1>(mv, 32 * wi, lane, sM);
+    rows_reduce_add<1>(mv, 32 * wi, lane, sM);  // two waves (wj = 0, 1) add to a zeroed entry: order-independent
     if (GATE == LNX_GATE_SCALAR) {
       tot = wave_sum(tot);
-      if (lane == 0) atomicAdd(&sMisc[0], tot);
+      if (lane == 0) sMisc[4 + wave] = tot;
     }
   }
   // dk += dPe^T Q + dXe^T K
@@ -1142,7 +1146,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   if (GATE == LNX_GATE_SCALAR) {
     if ((tid & 3) == 0) {
       float d = dgp + 2.f * sBeta[tr] * sM[tr];
-      if (tr == 63) d += sMisc[0] + __expf(gC) * sMisc[1];
+      if (tr == 63) d += ((sMisc[4] + sMisc[5]) + (sMisc[6] + sMisc[7])) + __expf(gC) * ((sMisc[8] + sMisc[9]) + (sMisc[10] + sMisc[11]));
       sdG[tr] = d;
     }
     lds_barrier();
@@ -1183,10 +1187,17 @@ int launch_bwd(const DirectParams& p, int nstate, hipStream_t st) {
 
 }  // namespace
 
-int lnx_direct_scan_fwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {
+namespace {
+template <typename OT>
+int scan_fwd_by_shape(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {
   if (dk == 128)
-    return gate == LNX_GATE_SCALAR ? launch_scan_fwd<128, LNX_GATE_SCALAR>(p, nstate, st) : launch_scan_fwd<128, LNX_GATE_NONE>(p, nstate, st);
-  return gate == LNX_GATE_SCALAR ? launch_scan_fwd<64, LNX_GATE_SCALAR>(p, nstate, st) : launch_scan_fwd<64, LNX_GATE_NONE>(p, nstate, st);
+    return gate == LNX_GATE_SCALAR ? launch_scan_fwd<128, LNX_GATE_SCALAR, OT>(p, nstate, st) : launch_scan_fwd<128, LNX_GATE_NONE, OT>(p, nstate, st);
+  return gate == LNX_GATE_SCALAR ? launch_scan_fwd<64, LNX_GATE_SCALAR, OT>(p, nstate, st) : launch_scan_fwd<64, LNX_GATE_NONE, OT>(p, nstate, st);
+}
+}  // namespace
+
+int lnx_direct_scan_fwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {
+  return p.o_dtype == LNX_F32 ? scan_fwd_by_shape<float>(p, dk, gate, nstate, st) : scan_fwd_by_shape<bf16_t>(p, dk, gate, nstate, st);
 }
 
 int lnx_direct_bwd(const DirectParams& p, int dk, int gate, int nstate, hipStream_t st) {

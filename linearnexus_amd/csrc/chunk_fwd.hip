@@ -38,6 +38,7 @@ struct FwdParams {
   int out_spw;  // chunk_output: value slabs per workgroup
   int vcols;    // leading value columns present in v (its row length); the rest of the dv columns are zero
   int l2norm;   // chunk_prepare2<LITE>: q and k rows are normalised as x / (|x| + 1e-6) inside the kernels
+  int slab;     // lnx_scan_args.test_scan_slab
   float scale;
   char* ws;
   ChunkWs off;
@@ -1340,7 +1341,7 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   // with dk = 256, whose tiles leave no room in LDS for a wider slab
   constexpr bool can_narrow = (DK >= 128 && sizeof(T) == 2) || (DK == 128 && sizeof(T) == 4);
   constexpr int WIDE = (DK > 128 && sizeof(T) == 4) ? 32 : 64, NARROW = can_narrow ? 32 : WIDE;
-  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64));
+  const bool narrow = can_narrow && lnx_narrow_slabs((int64_t)nstate * p.geom.H * (p.dv / 64), p.slab);
   auto k2 = narrow ? chunk_scan_kernel<T, DK, GATE, NARROW> : chunk_scan_kernel<T, DK, GATE, WIDE>;
   auto k3 = chunk_output_kernel<T, DK, GATE>;
   const int bv = narrow ? NARROW : WIDE;
@@ -1357,11 +1358,11 @@ int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   hipLaunchKernelGGL(k2, dim3(lnx_xcd_grid((int64_t)nstate * p.geom.H, p.dv / bv)), dim3(512), b2, st, p);
   if (!ScanSmem<T, DK>::FUSE_OUT && p.o) {  // otherwise the scan has written the outputs
     lnx_profile_mark("chunk_output", st);
-    // value slabs per workgroup: as many as leave about two thousand workgroups (LNX_OUT_SLABS overrides, for tests)
+    // value slabs per workgroup: as many as leave about two thousand workgroups (p.out_spw > 0: the tests' override)
     const int nslab = p.dv / OutSmem<T, DK>::BV;
     FwdParams po = p;
     po.out_spw = (int)std::max<int64_t>(1, std::min<int64_t>(nslab, slots * nslab / 2048));
-    if (const char* e = getenv("LNX_OUT_SLABS")) po.out_spw = std::max(1, std::min(nslab, atoi(e)));
+    if (p.out_spw > 0) po.out_spw = std::min(nslab, p.out_spw);
     hipLaunchKernelGGL(k3, dim3(lnx_xcd_grid(slots, (nslab + po.out_spw - 1) / po.out_spw)), dim3(256), b3, st, po);
   }
   lnx_profile_mark(nullptr, st);
@@ -1402,9 +1403,11 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (a->dtype != LNX_F32 && a->dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "dtype %d", a->dtype);
   if (a->o_dtype != LNX_F32 && a->o_dtype != LNX_BF16) return lnx_set_error(LNX_ERR_DTYPE, "o_dtype %d", a->o_dtype);
   if (a->use_qk_l2norm && !lnx_chunk_direct(a))
-    return lnx_set_error(LNX_ERR_SHAPE, "use_qk_l2norm inside the chunk kernels needs 2-byte inputs and outputs, dk <= 128 and no per-channel gate; "
+    return lnx_set_error(LNX_ERR_SHAPE, "use_qk_l2norm inside the chunk kernels needs 2-byte inputs, dk <= 128 and no per-channel gate; "
                                         "normalise with lnx_l2norm_fwd first");
   if (a->token_first != 0 && a->token_first != 1) return lnx_set_error(LNX_ERR_SHAPE, "token_first must be 0 or 1");
+  if ((a->test_scan_slab != 0 && a->test_scan_slab != 32 && a->test_scan_slab != 64) || a->test_out_slabs < 0)
+    return lnx_set_error(LNX_ERR_SHAPE, "test_scan_slab must be 0, 32 or 64 and test_out_slabs >= 0");
   if (backward && a->forward_only) return lnx_set_error(LNX_ERR_SHAPE, "forward_only is set: the workspace holds nothing for a backward pass");
   if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
     return lnx_set_error(LNX_ERR_SHAPE, "packed batches need B == 1 and nseq > 0 (B=%d nseq=%d)", a->B, a->nseq);
@@ -1436,7 +1439,7 @@ int launch_direct_fwd(const lnx_scan_args* a, const FwdParams& p, int nstate, hi
   d.q = reinterpret_cast<const bf16_t*>(a->q); d.k = reinterpret_cast<const bf16_t*>(a->k);
   d.v = reinterpret_cast<const bf16_t*>(a->v); d.beta = a->beta; d.s0 = a->initial_state; d.sT_out = a->final_state;
   d.o = a->o; d.dv = a->dv; d.o_dtype = a->o_dtype; d.save = !a->forward_only; d.vcols = p.vcols; d.gate = a->gate;
-  d.l2norm = a->use_qk_l2norm;
+  d.l2norm = a->use_qk_l2norm; d.slab = a->test_scan_slab;
   d.scale = a->scale; d.ws = p.ws; d.off = p.off;
   int rc = lnx_direct_scan_fwd(d, a->dk, a->gate, nstate, st);
   if (rc != LNX_OK) return rc;
@@ -1474,16 +1477,17 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
   p.sT_out = a->final_state; p.o = a->o; p.dv = a->dv; p.o_dtype = a->o_dtype; p.scale = a->scale;
   // 4-byte inputs form the outputs in a separate kernel that reads the state and D back
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
-  p.out_spw = 1;
+  p.out_spw = a->test_out_slabs;
+  p.slab = a->test_scan_slab;
   p.vcols = a->value_cols ? a->value_cols : a->dv;
   p.l2norm = a->use_qk_l2norm;
   p.ws = ws; p.off = w;
   int rc;
   if (lnx_chunk_direct(a)) return launch_direct_fwd(a, p, nstate, st);
-  if (a->dtype == LNX_BF16)
+  if (a->dtype == LNX_BF16)  // dk <= 128 without a per-channel gate went to the direct-solve kernels above
     rc = (a->dk == 256)   ? launch_fwd_gate<bf16_t, 256>(a->gate, p, nstate, st)
-         : (a->dk == 128) ? launch_fwd_gate<bf16_t, 128>(a->gate, p, nstate, st)
-                          : launch_fwd_gate<bf16_t, 64>(a->gate, p, nstate, st);
+         : (a->dk == 128) ? launch_fwd<bf16_t, 128, LNX_GATE_VECTOR>(p, nstate, st)
+                          : launch_fwd<bf16_t, 64, LNX_GATE_VECTOR>(p, nstate, st);
   else
     rc = (a->dk == 256)   ? launch_fwd_gate<float, 256>(a->gate, p, nstate, st)
          : (a->dk == 128) ? launch_fwd_gate<float, 128>(a->gate, p, nstate, st)
@@ -1536,6 +1540,11 @@ extern "C" int lnx_chunk_fwd(const lnx_scan_args* a, void* stream) {
   int rc = lnx_chunk_check(a, false);
   if (rc != LNX_OK) return rc;
   return chunk_fwd_on(a, a->workspace, a->workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int lnx_chunk_fwd_static_init(void) {
+  void* ws = nullptr;
+  return static_scratch(&ws);
 }
 
 extern "C" int lnx_chunk_fwd_static(const lnx_scan_args* a, void* stream) {

@@ -159,6 +159,13 @@ __global__ __launch_bounds__(256) void conv1d_fwd_kernel(ConvParams p) {
   if (p.new_cache && t1 == p.T) {  // this thread saw the end of the (last) sequence: the window holds its last 3 rows
     const int keep = p.K - 1;
     T* cp = static_cast<T*>(p.new_cache) + (size_t)b * keep * p.D + c;
+    if (PACKED && seq_end(p.cu, p.nseq - 1, p.T) <= seq_first(p.cu, p.nseq - 1, p.T)) {
+      // the last sequence has no tokens: the window still holds the tail of the one before it, the carry is zero
+#pragma unroll
+      for (int j = 0; j < KMAX; ++j)
+#pragma unroll
+        for (int i = 0; i < N; ++i) win[j][i] = 0.f;
+    }
     for (int i = 0; i < keep; ++i) store_vec<T, N>(cp + (size_t)i * p.D, win[KMAX - 1 - keep + i]);
   }
 }

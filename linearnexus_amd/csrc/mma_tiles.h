@@ -360,9 +360,37 @@ __device__ __forceinline__ void unstage_tile_checked(T* dst, int64_t stride, con
   }
 }
 
+// A bf16 LDS tile written out as fp32 rows (same range check): the direct-solve forward scan stages its outputs in
+// bf16 -- the precision the reference returns them in for bf16 inputs -- and widens them here when the caller asked
+// for fp32 outputs.
+template <int ROWS, int COLS>
+__device__ __forceinline__ void unstage_tile_checked_widen(float* dst, int64_t stride, const bf16_t* src, int ld, int valid, int tid) {
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int VPR = COLS / 8, TOTAL = ROWS * VPR, IT = TOTAL / 256;
+  static_assert(TOTAL % 256 == 0, "whole passes only");
+  const int bytes = valid > 0 ? (int)(valid * stride * (int64_t)sizeof(float)) : 0;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(dst, 0, bytes, 0x00020000);
+  bf16x8 x[IT];
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * 8;
+    x[it] = *reinterpret_cast<const bf16x8*>(src + r * ld + c);
+  }
+#pragma unroll
+  for (int it = 0; it < IT; ++it) {
+    const int idx = tid + 256 * it, r = idx / VPR, c = (idx - r * VPR) * 8;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const floatx4 y = {(float)x[it][4 * h], (float)x[it][4 * h + 1], (float)x[it][4 * h + 2], (float)x[it][4 * h + 3]};
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, y), rsrc, (int)((r * stride + c + 4 * h) * (int64_t)sizeof(float)), 0, 0);
+    }
+  }
+}
+
 // Sums f(e) * acc[i][0][e] over the 32 lanes that share rows, for all 16*MT rows of a wave's
 // fragments at once, by a transpose-reduce (31 shuffles per 32 values instead of 160), then adds
-// the row totals into rows[] (LDS) with one atomic per row and wave.
+// the row totals into rows[] (LDS) with one atomic per row and wave.  Callers zero rows[] and have at most two waves
+// per row, so the result does not depend on the order of arrival (0 + a + b = 0 + b + a in floating point).
 template <int MT>
 __device__ __forceinline__ void rows_reduce_add(float (&v)[16 * MT], int row0, int lane, float* rows) {
   // after the step with mask m, v[t] (t < n/2) holds the partial for value index t + (lane & m ? n/2 : 0)

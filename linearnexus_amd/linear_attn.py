@@ -128,8 +128,14 @@ def _gate_kind(g: Optional[Tensor], lead_shape, dk: int) -> int:
     raise RuntimeError(f"gate shape {tuple(g.shape)} matches neither {tuple(lead_shape)} nor {tuple(lead_shape) + (dk,)}")
 
 
+# Test hooks: the tiling overrides of ``lnx_scan_args`` (0 = the library's choice).  The GPU tests set them to reach both
+# slab widths of the sequential kernels, and the grouped form of the fp32 output kernel, at small shapes.
+_test_hooks = {"scan_slab": 0, "out_slabs": 0}
+
+
 def _base_args(B, H, T, dk, dv, dtype, o_dtype, gate, l2norm, scale) -> ScanArgs:
     a = ScanArgs()
+    a.test_scan_slab, a.test_out_slabs = _test_hooks["scan_slab"], _test_hooks["out_slabs"]
     a.B, a.H, a.T, a.dk, a.dv = B, H, T, dk, dv
     a.chunk = CHUNK
     a.dtype, a.o_dtype, a.gate = dtype, o_dtype, gate

@@ -26,14 +26,46 @@ def test_library_exports_every_declared_symbol():
     assert set(names) >= set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.lnx_abi_version() == 7
+    assert lib.lnx_abi_version() == 8
 
 
 def test_struct_layout_matches_header():
-    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size, value_cols (+ tail padding)
-    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8 + 8
+    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size, value_cols and the two test hooks
+    # (+ tail padding)
+    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8 + 16
     assert _lib.ScanArgs.q.offset == 56
     assert _lib.ScanArgs.value_cols.offset == 56 + 18 * 8 + 8
+    assert _lib.ScanArgs.test_out_slabs.offset == 56 + 18 * 8 + 8 + 8
+
+
+def test_one_kernel_set_per_shape_and_no_environment_dispatch():
+    """The split between the direct-solve and the WY kernels follows from fields the forward and the backward call
+    share (dtype, dk, gate) -- not from o_dtype, which the backward does not use, and not from the environment: the
+    workspace size (whose layout differs between the splits) does not react to either, and no source under csrc/
+    reads the environment."""
+    lib = _lib.load()
+    a = _lib.ScanArgs()
+    a.B, a.H, a.T, a.dk, a.dv, a.chunk = 2, 2, 256, 128, 128, 64
+    a.dtype, a.gate = _lib.LNX_BF16, _lib.GATE_SCALAR
+    a.o_dtype = _lib.LNX_BF16
+    n_bf16 = int(lib.lnx_chunk_workspace_bytes(a))
+    a.o_dtype = _lib.LNX_F32
+    assert int(lib.lnx_chunk_workspace_bytes(a)) == n_bf16 and lib.lnx_chunk_fuses_l2norm(a) == 1
+    os.environ["LNX_CHUNK_DIRECT"] = "0"
+    try:
+        assert int(lib.lnx_chunk_workspace_bytes(a)) == n_bf16
+    finally:
+        del os.environ["LNX_CHUNK_DIRECT"]
+    a.gate = _lib.GATE_VECTOR
+    assert int(lib.lnx_chunk_workspace_bytes(a)) > n_bf16 and lib.lnx_chunk_fuses_l2norm(a) == 0
+    a.gate, a.test_scan_slab = _lib.GATE_SCALAR, 48
+    one = ctypes.c_float(0)
+    a.q = a.k = a.v = a.beta = a.o = a.final_state = a.g = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"test_scan_slab" in lib.lnx_last_error()
+    csrc = os.path.join(ROOT, "linearnexus_amd", "csrc")
+    for f in os.listdir(csrc):
+        if f.endswith((".hip", ".h")):
+            assert "getenv" not in open(os.path.join(csrc, f)).read(), f
 
 
 def test_argument_validation_without_gpu():

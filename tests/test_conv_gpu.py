@@ -128,7 +128,10 @@ def test_full_size_linearity_and_shift():
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("act", [None, "silu"])
 @pytest.mark.parametrize("case", [(300, 64, 4, [0, 64, 65, 65, 200, 300]), (40, 32, 3, [0, 1, 2, 3, 40]),
-                                  (1000, 520, 4, [0, 31, 33, 500, 1000]), (130, 16, 2, [0, 130])])
+                                  (1000, 520, 4, [0, 31, 33, 500, 1000]), (130, 16, 2, [0, 130]),
+                                  (100, 32, 4, [0, 100, 100]),      # empty last sequence: the carry out is zero
+                                  (100, 32, 4, [0, 98, 98, 100]),   # last sequence shorter than K - 1, behind an empty one
+                                  (66, 16, 3, [0, 65, 66])])
 def test_packed_batch_equals_one_call_per_sequence(case, act, bf16):
     """Packed batches: the taps stop at sequence boundaries -- outputs and all gradients equal the oracle applied to
     every sequence on its own with a zero cache (sequences of 0, 1 and 2 tokens, boundaries inside a thread's run)."""

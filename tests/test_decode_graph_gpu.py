@@ -77,9 +77,9 @@ def test_graph_rejects_bad_states():
 @pytest.mark.parametrize("variant", ["gated", "kda"])
 def test_chunk_forward_backward_under_graph_capture(variant):
     """A whole differentiable chunk step (forward kernels, autograd, backward kernels) captured in one HIP graph:
-    every replay must reproduce the eager results -- o, S, dq, dk, dv bit for bit; dg and dbeta, whose row sums go
-    through LDS atomics in varying order, within 2e-5 of their largest entry -- with new inputs copied into the
-    captured buffers and eager work between the replays."""
+    every replay must reproduce the eager results bit for bit -- o, S and all five gradients (the row and chunk sums
+    behind dg and dbeta are added in a fixed order) -- with new inputs copied into the captured buffers and eager work
+    between the replays."""
     import linearnexus_amd as la
     B, H, T, d = 2, 4, 200, 128
     gate = "scalar" if variant == "gated" else "vector"
@@ -114,7 +114,4 @@ def test_chunk_forward_backward_under_graph_capture(variant):
         ref = run(*fresh)  # eager work between the replays
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, ref)):
-            if i < 5:
-                assert torch.equal(a, b), (seed, i)
-            else:
-                assert (a - b).abs().max() <= 2e-5 * b.abs().max(), (seed, i)
+            assert torch.equal(a, b), (seed, i)

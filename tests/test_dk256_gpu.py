@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from linearnexus_amd import linear_attn
 from oracle import recurrent as rc
 from oracle.adjoint import delta_rule_adjoint
 from oracle.inputs import make_inputs
@@ -19,7 +20,7 @@ GATES = ["none", "scalar", "vector"]
 
 
 # 2-byte inputs have a 32-column variant of the two sequential kernels and a 64-column one in which two operand tiles
-# share LDS space (chosen by the number of workgroups); LNX_SCAN_SLAB forces either.
+# share LDS space (chosen by the number of workgroups); the test_scan_slab field of the argument block forces either.
 SLABS = ["32", "64"]
 
 
@@ -28,7 +29,7 @@ SLABS = ["32", "64"]
 @pytest.mark.parametrize("shape", [(1, 2, 200, 256, 128), (2, 1, 64, 256, 64), (1, 1, 130, 256, 512)])
 @pytest.mark.parametrize("with_state", [False, True])
 def test_forward_dk256(gate, shape, with_state, slab, monkeypatch):
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     B, H, T, dk, dv = shape
     x = make_inputs(81, B, H, T, dk, dv, gate=gate, with_state=with_state, with_grad=True)
     x, dt = _prep(x, True)
@@ -42,7 +43,7 @@ def test_forward_dk256(gate, shape, with_state, slab, monkeypatch):
 @pytest.mark.parametrize("gate", GATES)
 @pytest.mark.parametrize("shape", [(1, 2, 200, 256, 128), (2, 1, 70, 256, 64), (1, 1, 128, 256, 512)])
 def test_backward_dk256(gate, shape, slab, monkeypatch):
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     B, H, T, dk, dv = shape
     x = make_inputs(82, B, H, T, dk, dv, gate=gate, with_state=True, with_grad=True)
     x, dt = _prep(x, True)
@@ -53,7 +54,7 @@ def test_backward_dk256(gate, shape, slab, monkeypatch):
 @pytest.mark.parametrize("slab", SLABS)
 @pytest.mark.parametrize("gate", ["scalar", "vector"])
 def test_packed_dk256(gate, slab, monkeypatch):
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     H, T, dk, dv = 2, 300, 256, 128
     x = make_inputs(83, 1, H, T, dk, dv, gate=gate, with_grad=True)
     cu = np.array([0, 64, 70, 200, 300], np.int32)
@@ -75,7 +76,7 @@ def test_packed_dk256(gate, slab, monkeypatch):
 @pytest.mark.parametrize("slab", SLABS)
 def test_token_first_dk256(slab, monkeypatch):
     """[B, T, H, d] memory (the layout the reference's blocks hold before their transpose) through the same kernels."""
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     import linearnexus_amd as la
     B, H, T, dk, dv = 2, 3, 150, 256, 128
     x = make_inputs(84, B, H, T, dk, dv, gate="scalar", with_state=True)
@@ -124,7 +125,7 @@ def test_reference_preset_shape_against_token_kernel(slab, monkeypatch):
     """The presets' head shape (dk 256, dv 512) at a few thousand tokens: the chunk path and the fp32
     token-by-token kernel (itself checked against the oracle) must agree."""
     import linearnexus_amd as la
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     torch.manual_seed(3)
     B, H, T, dk, dv = 2, 4, 2048, 256, 512
     q = torch.nn.functional.normalize(torch.randn(B, H, T, dk, device=DEV), dim=-1).bfloat16()

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from linearnexus_amd import linear_attn
 from oracle import recurrent as rc
 from oracle.adjoint import delta_rule_adjoint
 from oracle.inputs import make_inputs, to_bf16_grid
@@ -159,9 +160,9 @@ def test_forward_without_gradients_skips_nothing_visible(gate, bf16):
 @pytest.mark.parametrize("bf16", [True, False])
 def test_both_slab_widths_of_the_sequential_kernels(gate, slab, bf16, monkeypatch):
     """dk = 128 has 32- and 64-column variants of the two scans (chosen by the number of workgroups; the 64-column
-    backward scan of 4-byte inputs lets K and Q share an LDS tile); LNX_SCAN_SLAB forces either so that both meet
+    backward scan of 4-byte inputs lets K and Q share an LDS tile); the test_scan_slab field of the argument block forces either so that both meet
     the oracle at a small shape."""
-    monkeypatch.setenv("LNX_SCAN_SLAB", slab)
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", int(slab))
     x = make_inputs(67, 1, 2, 200, 128, 128, gate=gate, with_state=True, with_grad=True)
     tol = 2e-2 if bf16 else 1e-4
     xf, dt = _prep(x, bf16)
@@ -178,8 +179,8 @@ def test_both_slab_widths_of_the_sequential_kernels(gate, slab, bf16, monkeypatc
 @pytest.mark.parametrize("dk,dv", [(128, 320), (256, 160), (64, 192)])
 def test_output_kernel_slabs_per_workgroup(gate, spw, dk, dv, monkeypatch):
     """4-byte inputs form the outputs in a kernel of their own, which takes several value slabs per workgroup at
-    large shapes (Q and P staged once); LNX_OUT_SLABS forces the count, here with a ragged last group."""
-    monkeypatch.setenv("LNX_OUT_SLABS", spw)
+    large shapes (Q and P staged once); the test_out_slabs field of the argument block forces the count, here with a ragged last group."""
+    monkeypatch.setitem(linear_attn._test_hooks, "out_slabs", int(spw))
     x = make_inputs(68, 1, 2, 150, dk, dv, gate=gate, with_state=True)
     o_ref, S_ref = oracle_fwd(x, gate)
     o, S = gpu_chunk_fwd(x, gate, torch.float32)
@@ -338,3 +339,30 @@ def test_packed_batch_with_hundreds_of_short_sequences(gate):
     ref = {n: np.concatenate([p[n] for p in parts], 2) for n in names}
     ref["dS0"] = np.concatenate([p["dS0"] for p in parts], 0)
     check(gpu_grads(x, gate, torch.float32, cu=cu), ref, 1e-4)
+
+
+@pytest.mark.parametrize("gate", ["none", "scalar"])
+@pytest.mark.parametrize("slab", [32, 64])
+def test_bf16_inputs_with_fp32_outputs_take_the_same_kernels(gate, slab, monkeypatch):
+    """o_dtype does not select kernels: bf16 q, k, v with an fp32 output tensor run the direct-solve kernels like the
+    bf16-output call (the outputs are formed in fp32, rounded to bf16 -- the precision the reference returns for such
+    inputs, gated_deltanet.py:534 -- and widened on their way out), the backward pass reads the same workspace layout,
+    and values and gradients equal the bf16-output call's exactly."""
+    monkeypatch.setitem(linear_attn._test_hooks, "scan_slab", slab)
+    x = make_inputs(91, 2, 3, 150, 128, 128, gate=gate, with_state=True, with_grad=True)
+    xb, dt = _prep_bwd(x, True)
+    g = None if gate == "none" else torch.from_numpy(xb["g"]).to(DEV)
+    res = []
+    for o_dtype in (torch.bfloat16, torch.float32):
+        leaves = [torch.from_numpy(xb[n]).to(DEV).to(torch.bfloat16).requires_grad_(True) for n in ("q", "k", "v")]
+        beta = torch.from_numpy(xb["beta"]).to(DEV).requires_grad_(True)
+        s0 = torch.from_numpy(xb["S0"]).to(DEV).requires_grad_(True)
+        o, S = linear_attn._chunk(*leaves, g, beta, None, s0, 64, False, o_dtype, True, None)
+        assert o.dtype == o_dtype
+        dO = torch.from_numpy(xb["dO"]).to(DEV).to(torch.bfloat16)
+        grads = torch.autograd.grad([o, S], leaves + [beta, s0], [dO.to(o_dtype), torch.from_numpy(xb["dS"]).to(DEV)])
+        res.append([o.detach().float(), S.detach(), *[t.float() for t in grads]])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    o_ref, S_ref = oracle_fwd(xb, gate)
+    assert max_rel(res[1][0].cpu().numpy(), o_ref) < 2e-2 and max_rel(res[1][1].cpu().numpy(), S_ref) < 2e-2

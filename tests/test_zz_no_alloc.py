@@ -89,3 +89,42 @@ def test_static_scratch_forward_refuses_what_does_not_fit():
     a.forward_only = 1
     assert int(lib.lnx_chunk_workspace_bytes(a)) > _lib.STATIC_SCRATCH_BYTES
     assert lib.lnx_chunk_fwd_static(a, None) == -4 and b"scratch" in lib.lnx_last_error()
+
+
+def test_static_scratch_forward_under_graph_capture():
+    """The entry point exists for callers under HIP graph capture: captured on a stream after
+    lnx_chunk_fwd_static_init() (the symbol lookup stays outside the capture), replayed three times with eager work and
+    synchronisations in between, every replay bit-identical to lnx_chunk_fwd on a caller-owned workspace."""
+    lib = _lib.load()
+    assert lib.lnx_chunk_fwd_static_init() == 0
+    B, H, T, d = 2, 3, 200, 128
+    xn = make_inputs(75, B, H, T, d, d, gate="scalar")
+    xn["S0"] = (np.random.default_rng(75).standard_normal((B, H, d, d)) * 0.02).astype(np.float32)
+    x = {n: torch.from_numpy(a).to(DEV) for n, a in xn.items()}
+    for n in ("q", "k", "v"):
+        x[n] = x[n].to(torch.bfloat16).contiguous()
+    o = torch.zeros(B, H, T, d, dtype=torch.bfloat16, device=DEV)
+    sT = torch.zeros(B, H, d, d, dtype=torch.float32, device=DEV)
+    a = _args(x, B, H, T, d, d)
+    a.o, a.final_state = o.data_ptr(), sT.data_ptr()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.lnx_chunk_fwd_static(a, torch.cuda.current_stream().cuda_stream), "lnx_chunk_fwd_static (capturing)")
+    for rep in range(3):
+        # new inputs in the captured buffers; the reference result through the workspace entry point, eagerly
+        x["v"].copy_(torch.randn(B, H, T, d, device=DEV).to(torch.bfloat16))
+        x["S0"].mul_(0.5)
+        o_ref = torch.empty_like(o)
+        s_ref = torch.empty_like(sT)
+        b = _args(x, B, H, T, d, d)
+        b.o, b.final_state = o_ref.data_ptr(), s_ref.data_ptr()
+        n = int(lib.lnx_chunk_workspace_bytes(b))
+        ws = torch.empty(n, dtype=torch.uint8, device=DEV)
+        b.workspace, b.workspace_bytes = ws.data_ptr(), n
+        _lib.check(lib.lnx_chunk_fwd(b, torch.cuda.current_stream().cuda_stream), "lnx_chunk_fwd")
+        torch.cuda.synchronize()
+        o.fill_(float("nan"))
+        sT.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref) and torch.equal(sT, s_ref), f"replay {rep}"
