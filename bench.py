@@ -163,6 +163,10 @@ CHUNK_CONFIGS = {
     # configuration 2 through the reference's default, use_qk_l2norm=True, on q and k that are not normalised
     "gdn_chunk_l2norm": ("gated", 8, 16, 4096, 128, 0, False, True),
     "kda_chunk": ("kda", 4, 16, 8192, 128, 0, True, True),           # configuration 3
+    # configuration 3 from the block's raw gate projection: kda_gate's activation inside the chunk kernels
+    # (kda_chunkwise_raw_gate), against the same step behind the stand-alone gate kernels (kda_chunk_gate_kernels)
+    "kda_chunk_raw_gate": ("kda", 4, 16, 8192, 128, 0, True, True),
+    "kda_chunk_gate_kernels": ("kda", 4, 16, 8192, 128, 0, True, True),
     "deltanet_varlen": ("delta", 1, 32, 32768, 128, 8, False, True),  # configuration 5
     "deltanet_fp32": ("delta32", 2, 4, 512, 64, 0, False, False),     # configuration 1 (forward only)
     # head shape of the reference's Gated DeltaNet presets (models.py:142-143: head_dim 256, expand_v 2), 2048 wide
@@ -178,7 +182,8 @@ def bench_chunk(args, torch, la, _lib, name):
     variant, B, H, T, d, nseq, with_s0, backward = CHUNK_CONFIGS[name]
     dev = "cuda:0"
     l2norm = name.endswith("_l2norm")
-    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "gdn_chunk_l2norm": 2, "kda_chunk": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
+    seed = {"deltanet_fp32": 1, "gdn_chunk": 2, "gdn_chunk_l2norm": 2, "kda_chunk": 3, "kda_chunk_raw_gate": 3,
+            "kda_chunk_gate_kernels": 3, "deltanet_varlen": 5, "gdn_dk256": 6,
             "gdn_chunk_fp32": 2, "gdn_dk256_fp32": 6, "kda_chunk_fp32": 3}[name]
     fp32 = variant.endswith("32")
     variant = variant[:-2] if fp32 else variant
@@ -190,8 +195,15 @@ def bench_chunk(args, torch, la, _lib, name):
     q, k, v, dO = (x[n].to(dt) for n in ("q", "k", "v", "dO"))
     beta, g = x["beta"], x["g"]
     gen = torch.Generator(device="cpu").manual_seed(seed + 100)
+    raw_gate = name in ("kda_chunk_raw_gate", "kda_chunk_gate_kernels")
     if variant == "kda":
         g = (-torch.nn.functional.softplus(torch.randn(B, H, T, d, generator=gen)) * 0.05).to(dev)
+    if raw_gate:  # g = -exp(A_log) softplus(raw + bias) with A_log = log 0.05, bias = 0: the same decays as configuration 3
+        import math
+        g = None
+        raw = torch.randn(B, H, T, d, generator=gen).to(dev).to(dt)  # head-first like q, k, v here: no layout copies in either form
+        A_log = torch.full((H,), math.log(0.05), device=dev)
+        g_bias = torch.zeros(H * d, device=dev)
     cu = None
     nstate = B
     if nseq:
@@ -199,7 +211,9 @@ def bench_chunk(args, torch, la, _lib, name):
         cu = torch.from_numpy(cu_np).to(dev)
         nstate = nseq
     s0 = (torch.randn(nstate, H, d, dv, generator=gen) * 0.02).to(dev) if (with_s0 or nseq) else None
-    leaves = [q, k, v, beta] + ([g] if variant in ("gated", "kda") else []) + ([s0] if s0 is not None else [])
+    leaves = [q, k, v, beta] + ([g] if variant in ("gated", "kda") and not raw_gate else []) + ([s0] if s0 is not None else [])
+    if raw_gate:
+        leaves += [raw, A_log, g_bias]
     if backward:
         for t in leaves:
             t.requires_grad_(True)
@@ -207,6 +221,11 @@ def bench_chunk(args, torch, la, _lib, name):
     def forward():
         if variant == "gated":
             return la.gated_delta_rule_chunkwise(q, k, v, g, beta, None, s0, 64, l2norm)
+        if name == "kda_chunk_raw_gate":
+            return la.kda_chunkwise_raw_gate(q, k, v, raw, beta, A_log, g_bias, None, s0, 64, False)
+        if name == "kda_chunk_gate_kernels":  # every (batch, head) as a one-head batch row of the gate kernel (A_log is uniform here)
+            ga, _ = la.kda_gate(raw.view(B * H, T, d), A_log[:1], d, g_bias[:d], out_dtype=torch.float32)
+            return la.kda_chunkwise(q, k, v, ga.view(B, H, T, d), beta, None, s0, 64, False)
         if variant == "kda":
             return la.kda_chunkwise(q, k, v, g, beta, None, s0, 64, False)
         return la.delta_rule_chunkwise(q, k, v, beta, s0, cu_seqlens=cu)

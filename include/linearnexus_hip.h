@@ -93,6 +93,22 @@ typedef struct lnx_scan_args {
                                    states are wanted.  (Transition matrices of sequence segments: value columns
                                    [v | 0], initial states [0 | I].) */
 
+  /* The per-channel gate's activation inside the chunk op (ABI version 8; gate == LNX_GATE_VECTOR only).  With
+     gate_raw != NULL, g is ignored and lnx_chunk_fwd forms the log-decay itself from the block's raw gate projection,
+       g[b, h, t, c] = -exp(gate_A_log[h]) * softplus(gate_raw[b, h, t, c] + gate_bias[h * dk + c])
+     (kda_gate, kda.py:153-165; softplus(x) = x above gate_threshold), in the prepare kernel's gate load: the fp32
+     log-decay tensor never exists in memory.  gate_raw has the layout and element type of q ([B,H,T,dk] or, with
+     token_first, [B,T,H,dk] = the projection's [B,T,H*dk]).  lnx_chunk_bwd then needs the same fields again, writes
+     d_gate_raw (element type of q) in place of d_g and returns the parameter gradients d_gate_A_log [H] and
+     d_gate_bias [H*dk] (either may be NULL), summed without atomics through partial rows in the workspace. */
+  const void* gate_raw;
+  const float* gate_A_log;
+  const float* gate_bias;       /* NULL = no bias */
+  float gate_threshold;
+  void* d_gate_raw;
+  float* d_gate_A_log;
+  float* d_gate_bias;
+
   /* Test hooks (ABI version 8); a binding leaves both 0 = the library's choice.  Neither changes results or the
      workspace layout, only which of two tilings of the same kernel runs, so that tests reach both at small shapes. */
   int32_t test_scan_slab;       /* 32 or 64: value columns per workgroup of the sequential kernels */

@@ -15,6 +15,7 @@ from .linear_attn import (
     gated_delta_rule_recurrent,
     gated_delta_rule_step,
     kda_chunkwise,
+    kda_chunkwise_raw_gate,
     kda_recurrent,
     kda_step,
     l2norm_rows,
@@ -25,6 +26,6 @@ __all__ = [
     "DeltaNetState", "GatedDeltaNetState", "KDAState",
     "delta_rule_recurrent", "delta_rule_chunkwise", "delta_rule_step",
     "gated_delta_rule_recurrent", "gated_delta_rule_chunkwise", "gated_delta_rule_step",
-    "kda_recurrent", "kda_chunkwise", "kda_step", "l2norm_rows", "depthwise_conv1d_causal",
+    "kda_recurrent", "kda_chunkwise", "kda_chunkwise_raw_gate", "kda_step", "l2norm_rows", "depthwise_conv1d_causal",
     "dplr_delta_rule_recurrent", "dplr_delta_rule_step", "rmsnorm_gated", "kda_gate", "gated_deltanet_gate",
 ]

@@ -38,6 +38,8 @@ class ScanArgs(C.Structure):
         ("d_v", C.c_void_p), ("d_beta", C.c_void_p), ("d_g", C.c_void_p), ("d_initial_state", C.c_void_p),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
         ("value_cols", C.c_int32),
+        ("gate_raw", C.c_void_p), ("gate_A_log", C.c_void_p), ("gate_bias", C.c_void_p), ("gate_threshold", C.c_float),
+        ("d_gate_raw", C.c_void_p), ("d_gate_A_log", C.c_void_p), ("d_gate_bias", C.c_void_p),
         ("test_scan_slab", C.c_int32), ("test_out_slabs", C.c_int32),
     ]
 

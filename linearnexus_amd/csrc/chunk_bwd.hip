@@ -12,6 +12,7 @@
 // with r_j = exp(G_last - G_j), G the cumulative log-decay inside the chunk.
 
 #include "chunk_common.h"
+#include "reduce_rows.h"
 
 namespace {
 
@@ -31,6 +32,14 @@ struct BwdParams {
   float* ds0;
   int dv, gate;
   int slab;  // lnx_scan_args.test_scan_slab
+  // per-channel gate activated inside the op (lnx_scan_args.gate_raw): bwd_wy2 carries dg through the activation
+  const void* graw;
+  const float* gA;
+  const float* gbias;
+  float gthr;
+  void* dgraw;
+  float* gpart;       // [2][prows + LNX_SUM_SLICES][H * dk]: per-chunk partial sums of d_bias and of dg * g
+  int64_t gprows;     // partial rows: chunk slots per head
   float scale;
   char* ws;
   ChunkWs off;
@@ -883,7 +892,9 @@ template <typename T, int DK, int GATE> struct Wy2Cfg {
   static constexpr size_t bytes = stash_off + (STASH ? sizeof(float) * 16 * 256 : 0);
 };
 
-template <typename T, int DK, int GATE>
+// GRAW (per-channel gate only): the gate was activated inside the op from the raw projection; dg goes on through the
+// activation to d_gate_raw and to the per-chunk partial sums of the parameter gradients.
+template <typename T, int DK, int GATE, bool GRAW = false>
 __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || DK > 128 ? 2 : 3) : (GATE == LNX_GATE_VECTOR || DK > 128 ? 1 : 2))) void bwd_wy2_kernel(BwdParams p) {
   typedef Wy2Cfg<T, DK, GATE> L;
   constexpr int LDC = L::LDC, LDF = L::LDF, NKS = DK / 64;
@@ -908,7 +919,16 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   const int row = (int)(slot / N), n = (int)(slot % N);
   int tok0, len;
   chunk_span(p.geom, n, tok0, len);
-  if (len <= 0) return;
+  // fused gate activation: this chunk's row of the parameter-gradient partial sums, columns of this head
+  auto gate_part = [&](int which) {
+    const int64_t gD = (int64_t)p.geom.H * DK;
+    return p.gpart + (which * (p.gprows + LNX_SUM_SLICES) + (int64_t)(row / p.geom.H) * N + n) * gD + (row % p.geom.H) * DK;
+  };
+  if (len <= 0) {  // an unused slot of a packed batch: its partial sums are zero
+    if constexpr (GRAW)
+      for (int c = tid; c < DK; c += 256) gate_part(0)[c] = gate_part(1)[c] = 0.f;
+    return;
+  }
   const int64_t tbase = tok_index(p.geom, row, tok0);
   const int64_t ts = p.geom.ts, tsk = ts * DK, tsv = ts * p.dv;  // token stride, row strides of the token tiles
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
@@ -1154,8 +1174,63 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         float off = 0.f;
         for (int s_ = seg + 1; s_ < 4; ++s_) off += sSeg[s_ * 64 + c];
 #pragma unroll 4
-        for (int i = 0; i < 16; ++i)
-          if (16 * seg + i < len) p.dg[(tbase + (16 * seg + i) * ts) * DK + ch0 + c] = sOut[(16 * seg + i) * LDF + c] + off;
+        for (int i = 0; i < 16; ++i) sOut[(16 * seg + i) * LDF + c] += off;
+      }
+      // dg leaves by rows: thread = (row tid / 16 + 16 it, four channels), 16-byte accesses (one channel per lane and
+      // token, as in the pass above, makes four times as many memory instructions).  With the gate activated inside
+      // the op, g = -e^{A_log} softplus(x), x = raw + bias (kda.py:153-165), the gradient goes on to the raw projection,
+      // d_raw = dg (-e^{A_log}) softplus'(x), and the rows add to the channel's sums of d_raw (-> d_bias) and of dg g
+      // (-> d_A_log).  One exponential serves softplus and its derivative: softplus(x) = max(x, 0) + log(1 + e),
+      // sigmoid(x) = (x >= 0 ? 1 : e) / (1 + e), e = e^-|x|.
+      typedef typename Mma<T>::Quad Quad;  // four elements of T
+      Quad rq[4];
+      if constexpr (GRAW) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+          rq[it] = *reinterpret_cast<const Quad*>(reinterpret_cast<const T*>(p.graw) + (tbase + (int64_t)min(r, len - 1) * ts) * DK + ch0 + c);
+        }
+      }
+      lds_barrier();
+      if constexpr (!GRAW) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+          if (r < len) store4(p.dg + (tbase + (int64_t)r * ts) * DK + ch0 + c, load4(sOut + r * LDF + c));
+        }
+      } else {
+        const int c = (tid & 15) * 4;
+        const float na = -__expf(p.gA[row % p.geom.H]);
+        floatx4 bias = {0.f, 0.f, 0.f, 0.f}, sb = bias, sa = bias;
+        if (p.gbias) bias = load4(p.gbias + (row % p.geom.H) * DK + ch0 + c);
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int r = (tid >> 4) + 16 * it;
+          const floatx4 dgv = load4(sOut + r * LDF + c);
+          floatx4 dr;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float x = to_f32(rq[it][e]) + bias[e];
+            const bool lin = x > p.gthr;
+            const float ex = __expf(-fabsf(x)), rc = __builtin_amdgcn_rcpf(1.f + ex);
+            const float sp = lin ? x : fmaxf(x, 0.f) + __logf(1.f + ex), ds = lin ? 1.f : (x >= 0.f ? rc : ex * rc);
+            dr[e] = r < len ? dgv[e] * na * ds : 0.f;
+            sb[e] += dr[e];
+            sa[e] += r < len ? dgv[e] * na * sp : 0.f;
+          }
+          if (r < len) store4(reinterpret_cast<T*>(p.dgraw) + (tbase + (int64_t)r * ts) * DK + ch0 + c, dr);
+        }
+        float* sPart = reinterpret_cast<float*>(sKr);  // [2][16 row groups][64]: the K tile is dead, the segment totals read
+        store4(sPart + (tid >> 4) * 64 + c, sb);
+        store4(sPart + 1024 + (tid >> 4) * 64 + c, sa);
+        lds_barrier();
+        if (tid < 128) {  // the sixteen row groups in a fixed order
+          const float* src = sPart + (tid >> 6) * 1024 + (tid & 63);
+          float t = 0.f;
+#pragma unroll
+          for (int q = 0; q < 16; ++q) t += src[64 * q];
+          gate_part(tid >> 6)[ch0 + (tid & 63)] = t;
+        }
       }
     }
     if (tid < 64 && tid < len) p.dbeta[tbase + tid * ts] = sdB[tid];
@@ -1274,7 +1349,7 @@ int launch_bwd(const BwdParams& p, int nstate, hipStream_t st) {
   auto k1 = narrow ? bwd_scan_kernel<T, DK, GATE, NARROW> : bwd_scan_kernel<T, DK, GATE, WIDE>;
   const int bv = narrow ? BScanCfg<T, DK, NARROW>::BV : BScanCfg<T, DK, WIDE>::BV;
   auto k2 = bwd_dqk_kernel<T, DK, GATE>;
-  auto k3 = bwd_wy2_kernel<T, DK, GATE>;
+  auto k3 = (GATE == LNX_GATE_VECTOR && p.graw) ? bwd_wy2_kernel<T, DK, GATE, GATE == LNX_GATE_VECTOR> : bwd_wy2_kernel<T, DK, GATE>;
   const size_t b1 = narrow ? BScanCfg<T, DK, NARROW>::bytes : BScanCfg<T, DK, WIDE>::bytes;
   const size_t b2 = DqkCfg<T, DK, GATE>::bytes, b3 = Wy2Cfg<T, DK, GATE>::bytes;
   hipError_t e;
@@ -1341,6 +1416,11 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.q = a->q; p.k = a->k; p.v = a->v; p.beta = a->beta; p.d_o = a->d_o; p.d_sT = a->d_final_state;
   p.dq = a->d_q; p.dk = a->d_k; p.dv_out = a->d_v; p.dbeta = a->d_beta; p.dg = a->d_g; p.ds0 = a->d_initial_state;
   p.dv = a->dv; p.gate = a->gate; p.scale = a->scale; p.slab = a->test_scan_slab;
+  const bool raw_gate = a->gate == LNX_GATE_VECTOR && a->gate_raw != nullptr;
+  p.graw = raw_gate ? a->gate_raw : nullptr; p.gA = a->gate_A_log; p.gbias = a->gate_bias; p.gthr = a->gate_threshold;
+  p.dgraw = a->d_gate_raw;
+  p.gprows = (int64_t)(packed ? 1 : a->B) * lnx_chunk_slots(a);
+  p.gpart = raw_gate ? reinterpret_cast<float*>(reinterpret_cast<char*>(a->workspace) + w.gpart) : nullptr;
   p.ws = reinterpret_cast<char*>(a->workspace); p.off = w;
   if (lnx_chunk_direct(a)) {
     DirectParams d = {};
@@ -1367,6 +1447,10 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
          : (a->dk == 128) ? launch_bwd_gate<float, 128>(a->gate, p, nstate, st)
                           : launch_bwd_gate<float, 64>(a->gate, p, nstate, st);
   if (rc != LNX_OK) return rc;
+  if (raw_gate && (a->d_gate_A_log || a->d_gate_bias)) {
+    lnx_gate_finish_sums(p.gpart, p.gprows, a->H, a->dk, a->d_gate_A_log, a->d_gate_bias, st);
+    lnx_profile_mark(nullptr, st);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return lnx_set_error(LNX_ERR_LAUNCH, "chunk backward launch: %s", hipGetErrorString(e));
   return LNX_OK;

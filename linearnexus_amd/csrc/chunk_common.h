@@ -103,8 +103,17 @@ __device__ __forceinline__ bool xcd_slot_part(int64_t slots, int parts, int64_t&
 inline unsigned lnx_xcd_grid(int64_t slots, int parts) { return (unsigned)(((slots + 7) / 8) * 8 * parts); }
 
 struct ChunkWs {
-  uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, Nq, Nk, Fq, TmT, D, SnT, dD, dSn, dW, dG, total;
+  uint64_t tab, G, P, X, W, U, Kr, Qg, Tm, Nq, Nk, Fq, TmT, D, SnT, dD, dSn, dW, dG, gpart, total;
 };
+
+// kda_gate.hip: partial rows of the fused gate activation's parameter gradients and their reduction
+uint64_t lnx_gate_part_bytes(int64_t nrows, int D);
+void lnx_gate_finish_sums(float* part, int64_t nrows, int H, int dk, float* d_A_log, float* d_bias, hipStream_t st);
+
+// log(1 + e^x) in the overflow-free form max(x, 0) + log1p(e^-|x|); x itself above the threshold (kda.py:157-163)
+__device__ __forceinline__ float lnx_softplus_thr(float x, float thr) {
+  return x > thr ? x : fmaxf(x, 0.f) + __logf(1.f + __expf(-fabsf(x)));
+}
 
 // 2-byte inputs with dk <= 128 and no per-channel gate take the kernels of chunk_direct.hip, which keep G, Pm, Tm, the
 // per-chunk states and state gradients, D and dR in the workspace (no W, U, dW); every other shape takes the WY-split
@@ -135,7 +144,7 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   auto take = [&](uint64_t bytes) { uint64_t o = off; off = lnx_align256(off + bytes); return o; };
   w.tab = take(a->cu_seqlens ? (2 * N + 2 * (uint64_t)a->nseq + 1) * 4 : 0);
   if (lnx_chunk_direct(a)) {
-    w.X = w.W = w.U = w.Kr = w.Qg = w.TmT = w.dW = w.dG = 0;
+    w.X = w.W = w.U = w.Kr = w.Qg = w.TmT = w.dW = w.dG = w.gpart = 0;
     w.G = take(slots * C * 4);
     w.Nq = take(slots * C * 4);  // 1 / (|q_t| + eps), or 1 when the inputs come normalised
     w.Nk = take(slots * C * 4);
@@ -164,6 +173,8 @@ inline ChunkWs lnx_chunk_ws_layout(const lnx_scan_args* a) {
   w.dSn = take(bwd ? slots * dk * dv * es : 0);
   w.dW = take(bwd ? slots * C * dk * es : 0);
   w.dG = take(bwd ? (vec ? slots * C * dk * 4 : slots * C * 4 * (dk / 64)) : 0);  // scalar gate: one slot per 64-channel part
+  // fused gate activation: one partial row of its parameter gradients per chunk slot of a (batch element, head)
+  w.gpart = take(bwd && vec && a->gate_raw ? lnx_gate_part_bytes((int64_t)(slots / a->H), a->H * a->dk) : 0);
   w.total = off;
   return w;
 }

@@ -39,6 +39,11 @@ struct FwdParams {
   int vcols;    // leading value columns present in v (its row length); the rest of the dv columns are zero
   int l2norm;   // chunk_prepare2<LITE>: q and k rows are normalised as x / (|x| + 1e-6) inside the kernels
   int slab;     // lnx_scan_args.test_scan_slab
+  // per-channel gate formed inside kda_prepare from the raw projection (lnx_scan_args.gate_raw): element type of q
+  const void* graw;
+  const float* gA;
+  const float* gbias;
+  float gthr;
   float scale;
   char* ws;
   ChunkWs off;
@@ -431,7 +436,9 @@ template <typename T, int DK> struct KdaPrepSmem {
   static constexpr size_t bytes = sizeof(T) * 2 * kTile + sizeof(float) * (64 * LDF + 2 * 64 * LNX_LDA + 32 * 36 + 64);
 };
 
-template <typename T, int DK>
+// GRAW: the gate arrives as the block's raw projection and is activated here, g = -exp(A_log[h]) softplus(raw + bias)
+// (kda.py:153-165), on its way into LDS: the activated fp32 gate tensor is never written or read.
+template <typename T, int DK, bool GRAW>
 __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_kernel(FwdParams p) {
   typedef KdaPrepSmem<T, DK> L;
   constexpr int LDC = L::LDC, LDF = L::LDF, NH = DK / 64;
@@ -461,11 +468,37 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
 
   // ---- phase A: per 64-channel half ----
   TileRegs<T, 64, 64> rK, rQ;
-  TileRegs<float, 64, 64> rG;
+  TileRegs<typename std::conditional<GRAW, T, float>::type, 64, 64> rG;
+  const float gna = GRAW ? -__expf(p.gA[row % p.geom.H]) : 0.f;
   auto fetch_half = [&](int h) {
     rK.load(kg + 64 * h, tsk, len, tid);
     rQ.load(qg + 64 * h, tsk, len, tid);
-    rG.load(p.g + tbase * DK + 64 * h, tsk, len, tid);
+    if constexpr (GRAW) rG.load(reinterpret_cast<const T*>(p.graw) + tbase * DK + 64 * h, tsk, len, tid);
+    else rG.load(p.g + tbase * DK + 64 * h, tsk, len, tid);
+  };
+  // the raw gate tile -> activated fp32 gate in LDS; rows past the chunk's end stay zero (they read as raw zeros,
+  // whose activation is not zero)
+  auto store_gate = [&](int h) {
+    if constexpr (GRAW) {
+      typedef TileRegs<T, 64, 64> GT;
+      const int c = (tid % GT::VPR) * GT::N;  // a thread keeps its channel group in every pass (256 % VPR == 0)
+      float bias[GT::N];
+#pragma unroll
+      for (int e = 0; e < GT::N; ++e) bias[e] = p.gbias ? p.gbias[(row % p.geom.H) * DK + 64 * h + c + e] : 0.f;
+#pragma unroll
+      for (int it = 0; it < GT::IT; ++it) {
+        const int r = (tid + 256 * it) / GT::VPR;
+#pragma unroll
+        for (int e0 = 0; e0 < GT::N; e0 += 4) {
+          floatx4 g4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) g4[e] = r < len ? gna * lnx_softplus_thr(to_f32(rG.x[it][e0 + e]) + bias[e0 + e], p.gthr) : 0.f;
+          store4(sG + r * LDF + c + e0, g4);
+        }
+      }
+    } else {
+      rG.store(sG, LDF, tid);
+    }
   };
   fetch_half(0);
   if (tid < 64) sBeta[tid] = (tid < len) ? p.beta[tbase + (int64_t)tid * p.geom.ts] : 0.f;
@@ -491,7 +524,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
     lds_barrier();  // the previous half's tiles are dead
     rK.store(sK, LDC, tid);
     rQ.store(sQ, LDC, tid);
-    rG.store(sG, LDF, tid);
+    store_gate(h);
     lds_barrier();
     if (h + 1 < NH) fetch_half(h + 1);
     {  // cumulative gate along the tokens, per channel: 16-row segments in parallel, then their offsets
@@ -1326,17 +1359,17 @@ __global__ void build_table_kernel(const int32_t* cu, int nseq, int N, int T, in
 
 template <typename T, int DK, int GATE> struct PrepSelect {
   static constexpr size_t bytes = Prep2Cfg<T, DK>::bytes;
-  static auto kernel() { return chunk_prepare2_kernel<T, DK, GATE>; }
+  static auto kernel(bool) { return chunk_prepare2_kernel<T, DK, GATE>; }
 };
 template <typename T, int DK> struct PrepSelect<T, DK, LNX_GATE_VECTOR> {
   static constexpr size_t bytes = KdaPrepSmem<T, DK>::bytes;
-  static auto kernel() { return kda_prepare_kernel<T, DK>; }
+  static auto kernel(bool raw_gate) { return raw_gate ? kda_prepare_kernel<T, DK, true> : kda_prepare_kernel<T, DK, false>; }
 };
 
 template <typename T, int DK, int GATE>
 int launch_fwd(const FwdParams& p, int nstate, hipStream_t st) {
   const int64_t slots = (int64_t)p.geom.rows * p.geom.N;
-  auto k1 = PrepSelect<T, DK, GATE>::kernel();
+  auto k1 = PrepSelect<T, DK, GATE>::kernel(p.graw != nullptr);
   // 32-column slabs when 64-column ones would occupy at most half of the chip (256 CUs); always for 4-byte inputs
   // with dk = 256, whose tiles leave no room in LDS for a wider slab
   constexpr bool can_narrow = (DK >= 128 && sizeof(T) == 2) || (DK == 128 && sizeof(T) == 4);
@@ -1393,8 +1426,12 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
     return lnx_set_error(LNX_ERR_SHAPE, "value_cols = %d needs forward_only and a multiple of 64 up to dv = %d", a->value_cols, a->dv);
   if (backward && tokens && (!a->d_o || !a->d_q || !a->d_k || !a->d_v || !a->d_beta))
     return lnx_set_error(LNX_ERR_NULL, "d_o, d_q, d_k, d_v and d_beta are required");
-  if (tokens && a->gate != LNX_GATE_NONE && !a->g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
-  if (backward && tokens && a->gate != LNX_GATE_NONE && !a->d_g) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs d_g", a->gate);
+  const bool raw_gate = a->gate_raw != nullptr;
+  if (raw_gate && a->gate != LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "gate_raw is the per-channel gate's raw projection: gate must be LNX_GATE_VECTOR");
+  if (raw_gate && !a->gate_A_log) return lnx_set_error(LNX_ERR_NULL, "gate_raw needs gate_A_log");
+  if (tokens && a->gate != LNX_GATE_NONE && !a->g && !raw_gate) return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs g", a->gate);
+  if (backward && tokens && a->gate != LNX_GATE_NONE && !(raw_gate ? a->d_gate_raw : (void*)a->d_g))
+    return lnx_set_error(LNX_ERR_NULL, "gate kind %d needs %s", a->gate, raw_gate ? "d_gate_raw" : "d_g");
   if (a->gate < LNX_GATE_NONE || a->gate > LNX_GATE_VECTOR) return lnx_set_error(LNX_ERR_SHAPE, "unknown gate kind %d", a->gate);
   if (a->dk != 64 && a->dk != 128 && a->dk != 256)
     return lnx_set_error(LNX_ERR_SHAPE, "chunk kernels need dk in {64, 128, 256}, got %d", a->dk);
@@ -1479,6 +1516,7 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
   p.save = !(a->forward_only && a->dtype == LNX_BF16);
   p.out_spw = a->test_out_slabs;
   p.slab = a->test_scan_slab;
+  p.graw = a->gate == LNX_GATE_VECTOR ? a->gate_raw : nullptr; p.gA = a->gate_A_log; p.gbias = a->gate_bias; p.gthr = a->gate_threshold;
   p.vcols = a->value_cols ? a->value_cols : a->dv;
   p.l2norm = a->use_qk_l2norm;
   p.ws = ws; p.off = w;

@@ -231,6 +231,23 @@ extern "C" int lnx_kda_gate_bwd(const void* g, const float* A_log, const float* 
   return e == hipSuccess ? LNX_OK : lnx_set_error(LNX_ERR_LAUNCH, "kda_gate_bwd: %s", hipGetErrorString(e));
 }
 
+// Parameter gradients of the gate activation fused into the chunk kernels: `part` holds two [nrows x H*dk] matrices of
+// per-chunk partial sums (d_bias parts, then d_out * out parts), each followed by its first-level sums, and H*dk floats
+// of per-channel scratch -- lnx_gate_part_bytes(nrows, H * dk) bytes in all.
+uint64_t lnx_gate_part_bytes(int64_t nrows, int D) { return 2 * lnx_sum_rows_bytes(nrows, D) + (uint64_t)D * sizeof(float); }
+
+void lnx_gate_finish_sums(float* part, int64_t nrows, int H, int dk, float* d_A_log, float* d_bias, hipStream_t st) {
+  const int D = H * dk;
+  float* part_a = part + (nrows + LNX_SUM_SLICES) * D;
+  float* chan = part_a + (nrows + LNX_SUM_SLICES) * D;
+  lnx_profile_mark("kda_gate_sums", st);
+  if (d_bias) lnx_sum_rows(part, nrows, D, d_bias, st);
+  if (d_A_log) {
+    lnx_sum_rows(part_a, nrows, D, chan, st);
+    sum_heads_kernel<<<H, 64, 0, st>>>(chan, dk, d_A_log);
+  }
+}
+
 extern "C" int lnx_sigmoid_fwd(const float* x, float* y, int64_t n, void* hip_stream) {
   if (n < 0) return lnx_set_error(LNX_ERR_SHAPE, "sigmoid: n=%lld", (long long)n);
   if (n == 0) return LNX_OK;

@@ -397,9 +397,11 @@ class _L2Norm(torch.autograd.Function):
 
 
 def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, forward_only,
-                   dv_total=None, want_o=True):
+                   dv_total=None, want_o=True, raw_gate=None):
     """One lnx_chunk_fwd call.  ``dv_total`` > v's columns: the state has dv_total value columns of which v holds the
-    first ones and the others are zero (``value_cols``); ``want_o=False``: final states only.  Both forward-only."""
+    first ones and the others are zero (``value_cols``); ``want_o=False``: final states only.  Both forward-only.
+    ``raw_gate = (A_log, g_bias or None, threshold)``: ``g`` is the raw per-channel gate projection in q's dtype and the
+    kernels apply kda_gate's activation themselves."""
     dt, B, H, T, dk, dv_in, beta, gate, nseq, nstate, cu = _seq_setup(q, k, v, g, beta, None, cu_seqlens)
     dv = dv_in if dv_total is None else dv_total
     if initial_state is not None and tuple(initial_state.shape) != (nstate, H, dk, dv):
@@ -408,7 +410,7 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
     q_in, k_in = _as_layout(q, tf), _as_layout(k, tf)
     v = _as_layout(v, tf)
     beta_f = _as_layout(beta.to(torch.float32), tf)
-    g_f = None if g is None else _as_layout(g.to(torch.float32), tf)
+    g_f = None if g is None else _as_layout(g if raw_gate is not None else g.to(torch.float32), tf)
     s0 = None if initial_state is None else _f32(initial_state)
     o = _empty_layout(B, H, T, (dv,), o_dtype, q.device, tf) if want_o else None
     sT = torch.empty(nstate, H, dk, dv, dtype=torch.float32, device=q.device)
@@ -427,6 +429,12 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
     a.value_cols = 0 if dv == dv_in else dv_in
     a.q, a.k, a.v, a.beta, a.g = _ptr(qn), _ptr(kn), _ptr(v), _ptr(beta_f), _ptr(g_f)
     a.initial_state, a.final_state, a.o, a.cu_seqlens = _ptr(s0), _ptr(sT), _ptr(o), _ptr(cu)
+    gate_keep = ()
+    if raw_gate is not None:
+        A32 = raw_gate[0].detach().to(torch.float32).contiguous()
+        b32 = None if raw_gate[1] is None else raw_gate[1].detach().to(torch.float32).contiguous()
+        a.g, a.gate_raw, a.gate_A_log, a.gate_bias, a.gate_threshold = None, _ptr(g_f), _ptr(A32), _ptr(b32), float(raw_gate[2])
+        gate_keep = (A32, b32)
     lib = _lib.load()
     nbytes = int(lib.lnx_chunk_workspace_bytes(a))
     if nbytes == 0 and T > 0 and B > 0:
@@ -434,7 +442,7 @@ def _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_s
     ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q.device)
     a.workspace, a.workspace_bytes = _ptr(ws), nbytes
     _lib.check(lib.lnx_chunk_fwd(a, _stream(q)), "lnx_chunk_fwd")
-    saved = (q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws)
+    saved = (q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws) + gate_keep
     meta = (dt, B, H, T, dk, dv, gate, nseq, float(scale), bool(l2norm), o_dtype, beta.dtype,
             None if g is None else g.dtype, initial_state is not None, tf, fused)
     return o, sT, saved, meta
@@ -444,19 +452,22 @@ class _ChunkScan(torch.autograd.Function):
     """Pairs lnx_chunk_fwd with lnx_chunk_bwd (the role ``jax.custom_vjp`` plays for a JAX caller)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, grad_mode=True):
+    def forward(ctx, q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, grad_mode=True,
+                A_log=None, g_bias=None, threshold=None):
         # nothing to differentiate (inference): the kernels skip what only the backward reads.  `grad_mode` is the
         # caller's torch.is_grad_enabled() -- inside forward() it is always off, and needs_input_grad alone is still set
         # for leaves that require grad under torch.no_grad()
+        raw_gate = None if A_log is None else (A_log, g_bias, threshold)
         o, sT, saved, meta = _chunk_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens,
-                                            forward_only=not (grad_mode and any(ctx.needs_input_grad)))
+                                            forward_only=not (grad_mode and any(ctx.needs_input_grad)), raw_gate=raw_gate)
         ctx.save_for_backward(*saved)
         ctx.meta = meta
+        ctx.raw_gate = None if A_log is None else (float(threshold), A_log.dtype, None if g_bias is None else g_bias.dtype)
         return o, sT
 
     @staticmethod
     def backward(ctx, d_o, d_sT):
-        q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws = ctx.saved_tensors
+        q_in, k_in, qn, kn, v, beta_f, g_f, s0, cu, ws = ctx.saved_tensors[:10]
         dt, B, H, T, dk, dv, gate, nseq, scale, l2norm, o_dtype, beta_dt, g_dt, has_s0, tf, fused = ctx.meta
         dev = qn.device
         d_o = torch.zeros(B, H, T, dv, dtype=qn.dtype, device=dev) if d_o is None else d_o.to(qn.dtype)
@@ -476,6 +487,14 @@ class _ChunkScan(torch.autograd.Function):
         a.d_q, a.d_k, a.d_v, a.d_beta, a.d_g, a.d_initial_state = (_ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(dbeta),
                                                                    _ptr(dg), _ptr(ds0))
         a.workspace, a.workspace_bytes = _ptr(ws), ws.numel()
+        dA = dbias = None
+        if ctx.raw_gate is not None:  # g is the raw gate projection: its gradient and the activation's parameter gradients
+            A32, b32 = ctx.saved_tensors[10:12]
+            dA = torch.empty_like(A32)
+            dbias = None if b32 is None else torch.empty_like(b32)
+            a.g, a.d_g = None, None
+            a.gate_raw, a.gate_A_log, a.gate_bias, a.gate_threshold = _ptr(g_f), _ptr(A32), _ptr(b32), ctx.raw_gate[0]
+            a.d_gate_raw, a.d_gate_A_log, a.d_gate_bias = _ptr(dg), _ptr(dA), _ptr(dbias)
         _lib.check(_lib.load().lnx_chunk_bwd(a, _stream(qn)), "lnx_chunk_bwd")
         if l2norm and not fused:
             dq = _l2norm_rows_bwd(q_in, dq)
@@ -483,7 +502,10 @@ class _ChunkScan(torch.autograd.Function):
         dbeta = dbeta.to(beta_dt)
         if dg is not None:
             dg = dg.to(g_dt)
-        return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None, None
+        if ctx.raw_gate is not None:
+            dA = dA.to(ctx.raw_gate[1])
+            dbias = None if dbias is None else dbias.to(ctx.raw_gate[2])
+        return dq, dk_, dv_, dg, dbeta, ds0, None, None, None, None, None, dA, dbias, None
 
 
 _CHUNK_DK = (64, 128, 256)  # key head dimensions the chunk kernels are built for
@@ -592,3 +614,31 @@ def kda_chunkwise(q, k, v, g, beta, scale=None, initial_state=None, chunk_size=6
     """Chunked KDA scan, ``g [B,H,T,dk]`` (kda.py:350-655).  Like the reference, the output is
     float32 whatever the input dtype (kda.py:416, :655); pass ``output_dtype`` to change that."""
     return _chunk(q, k, v, g, beta, scale, initial_state, chunk_size, use_qk_l2norm, output_dtype, True, cu_seqlens)
+
+
+def kda_chunkwise_raw_gate(q, k, v, g_raw, beta, A_log, g_bias=None, scale=None, initial_state=None, chunk_size=64,
+                           use_qk_l2norm=True, *, threshold=20.0, cu_seqlens=None, output_dtype=torch.float32):
+    """``kda_gate`` (kda.py:120-172) and ``kda_chunkwise`` (kda.py:350-655) as one op: the KDA block's two steps between
+    its projections and its output norm without the fp32 log-decay tensor in between.
+
+    ``g_raw [B,H,T,dk]`` is the raw gate projection in q's dtype -- the block's ``[B,T,H*dk]`` viewed as
+    ``[B,T,H,dk].transpose(1, 2)`` is used in place, like q, k, v; ``A_log [H]``, ``g_bias [H*dk]`` as in ``kda_gate``.
+    Equal to ``kda_chunkwise(q, k, v, kda_gate(g_raw, A_log, dk, g_bias, out_dtype=float32)[0], beta, ...)`` with the
+    activation computed in fp32 inside the chunk kernels; differentiable with respect to q, k, v, g_raw, beta,
+    initial_state, A_log and g_bias.  dk must be 64, 128 or 256 and dv a multiple of 64."""
+    if chunk_size % 16 != 0:
+        raise ValueError(f"chunk_size (BT={chunk_size}) must be divisible by BC=16.")  # kda.py:438-440
+    if q.dim() != 4 or q.shape[-1] not in _CHUNK_DK or v.shape[-1] % 64 != 0:
+        raise RuntimeError(f"kda_chunkwise_raw_gate needs [B,H,T,d] inputs with dk in {_CHUNK_DK} and dv % 64 == 0, "
+                           f"got q {tuple(q.shape)}, v {tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype == g_raw.dtype) or q.dtype not in _DT:
+        raise RuntimeError("q, k, v and g_raw must share one of the dtypes float32 / bfloat16")
+    if tuple(g_raw.shape) != tuple(q.shape):
+        raise RuntimeError(f"g_raw {tuple(g_raw.shape)} must have q's shape {tuple(q.shape)}")
+    H, dk = q.shape[1], q.shape[-1]
+    if tuple(A_log.shape) != (H,) or (g_bias is not None and tuple(g_bias.shape) != (H * dk,)):
+        raise RuntimeError(f"A_log must be [{H}] and g_bias [{H * dk}]")
+    if scale is None:
+        scale = dk ** -0.5
+    return _ChunkScan.apply(q, k, v, g_raw, beta, initial_state, scale, use_qk_l2norm, output_dtype, cu_seqlens,
+                            torch.is_grad_enabled(), A_log, g_bias, float(threshold))

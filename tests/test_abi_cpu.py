@@ -30,12 +30,13 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layout_matches_header():
-    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size, value_cols and the two test hooks
-    # (+ tail padding)
-    assert ctypes.sizeof(_lib.ScanArgs) == 56 + 18 * 8 + 8 + 16
+    # 14 four-byte scalars, then 17 pointers, the workspace pointer and its size, value_cols (+ padding), the fused
+    # gate's three pointers, its threshold (+ padding) and three gradient pointers, and the two test hooks
     assert _lib.ScanArgs.q.offset == 56
-    assert _lib.ScanArgs.value_cols.offset == 56 + 18 * 8 + 8
-    assert _lib.ScanArgs.test_out_slabs.offset == 56 + 18 * 8 + 8 + 8
+    assert _lib.ScanArgs.value_cols.offset == 56 + 18 * 8 + 8 == 208
+    assert _lib.ScanArgs.gate_raw.offset == 216 and _lib.ScanArgs.gate_threshold.offset == 240
+    assert _lib.ScanArgs.d_gate_raw.offset == 248 and _lib.ScanArgs.test_out_slabs.offset == 276
+    assert ctypes.sizeof(_lib.ScanArgs) == 280
 
 
 def test_one_kernel_set_per_shape_and_no_environment_dispatch():

@@ -8,7 +8,7 @@ from linearnexus_amd import linear_attn as la
 def _run(monkeypatch, grad_mode, requires_grad):
     seen = []
 
-    def fake_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, forward_only):
+    def fake_forward(q, k, v, g, beta, initial_state, scale, l2norm, o_dtype, cu_seqlens, forward_only, raw_gate=None):
         seen.append(forward_only)
         B, H, T, dk = q.shape
         return q.new_zeros(B, H, T, v.shape[-1]), q.new_zeros(B, H, dk, v.shape[-1]), (), None
