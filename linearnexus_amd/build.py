@@ -44,7 +44,46 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(f"built {LIB} from {', '.join(srcs)}")
     build_c_abi_smoke(verbose)
+    build_xla_ffi(verbose)
     return LIB
+
+
+def xla_ffi_include_dir():
+    """Directory that holds ``xla/ffi/api/ffi.h``: ``XLA_FFI_INCLUDE_DIR`` if set, else what an installed JAX reports
+    (``jax.ffi.include_dir()``; ``jax.extend.ffi`` in older releases); None when neither is there."""
+    cands = [os.environ.get("XLA_FFI_INCLUDE_DIR")]
+    try:
+        import jax  # noqa: F401
+        try:
+            from jax import ffi as jffi
+        except ImportError:
+            from jax.extend import ffi as jffi
+        cands.append(jffi.include_dir())
+    except Exception:
+        pass
+    for d in cands:
+        if d and os.path.exists(os.path.join(d, "xla", "ffi", "api", "ffi.h")):
+            return d
+    return None
+
+
+def build_xla_ffi(verbose: bool = True) -> str:
+    """Compiles csrc/lnx_xla_ffi.cc (the XLA FFI handlers a JAX caller registers) into liblinearnexus_xla_ffi.so next to
+    the main library, where the XLA FFI headers exist; skipped with a message otherwise."""
+    inc = xla_ffi_include_dir()
+    if inc is None:
+        if verbose:
+            print("XLA FFI headers not found (no JAX installed, XLA_FFI_INCLUDE_DIR unset): csrc/lnx_xla_ffi.cc not built")
+        return ""
+    out = os.path.join(HERE, "liblinearnexus_xla_ffi.so")
+    cmd = ["hipcc", "-O2", "-std=c++17", "-fPIC", "-shared", f"-I{inc}", os.path.join(CSRC, "lnx_xla_ffi.cc"), "-o", out,
+           f"-L{HERE}", "-llinearnexus_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the XLA FFI handlers failed:\n" + r.stderr)
+    if verbose:
+        print(f"built {out}")
+    return out
 
 
 def build_c_abi_smoke(verbose: bool = True) -> str:
