@@ -34,6 +34,11 @@ namespace {
 
 using T = bf16_t;
 typedef Mma<T> M;
+struct Mma16Types {
+  typedef short short4_ __attribute__((ext_vector_type(4)));
+  typedef short short8_ __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) short4_ lds_short4;
+};
 
 template <typename X> __device__ __forceinline__ X* at(char* ws, uint64_t off) { return reinterpret_cast<X*>(ws + off); }
 
@@ -838,7 +843,7 @@ int launch_scan_bwd(const DirectParams& p, int nstate, hipStream_t st) {
 // bwd_chunk: the chunk-local gradients, one workgroup per chunk, all chunks in parallel.  Reads q, k, v, dO of the
 // chunk, the states S (entering) and dS' (leaving) and D, dR from the two scans; writes dq, dk, dbeta, dg (dv left
 // the reverse scan).  A loop over 32-column slabs of the value dimension accumulates every product that contracts
-// over value columns (next slab's tiles prefetched into registers):
+// over value columns; the slabs arrive in two LDS buffers through loads that bypass the registers, two slabs ahead:
 //   dQa = dO S^T     dK1 = dR S^T     dK2 = D dS'^T     dPm = dO D^T     dAm = dR D^T     <dR_t, v_t>     <dS', S>
 // then an epilogue over the chunk's tokens:
 //   dPe = scale tril(E * dPm)          dXa = -tril(E * dAm, -1)          dXe = diag(beta) dXa
@@ -847,28 +852,86 @@ int launch_scan_bwd(const DirectParams& p, int nstate, hipStream_t st) {
 //   dk  = beta row + e^{G_C - G} dK2 + dPe^T Q + dXe^T K
 //   dG  = <q, dq> - <k, dk> + 2 beta m;   dG_C += sum_t e^{G_C - G_t} <k_t, dK2_t> + e^{G_C} <dS', S>;   dg = reverse cumsum(dG)
 // Wave (wi, wj) owns the token-row tile wi and the key-column tiles NKT wj .. of the [64 x dk] accumulators and the
-// (wi, wj) tile of the [64 x 64] ones.  Tiles that are only read through transposing LDS loads get a row stride of
-// 64 bytes mod 256, which spreads the four rows a 16-lane group reads over all banks.
+// (wi, wj) tile of the [64 x 64] ones.  The epilogue's tiles that are only read through transposing LDS loads get a row
+// stride of 64 bytes mod 256, which spreads the four rows that half a wave reads over all banks.
+// Measured per workgroup at B8 H16 T4096 d128 (wall clock of wave 0, 2 workgroups per CU): 4.3 us until the first slab
+// is there, 6.2 us for the loop, 2.1 us staging K, Q and the four small tiles, 1.8 us for the epilogue's products and
+// 3.4 us until dq, dk have left -- memory latency at every step; the kernel moves 4.9 TB/s.
 // ---------------------------------------------------------------------------------------
+// ---- loads that go straight to LDS (global_load_lds_dwordx4): one wave instruction fetches 16 bytes per lane from
+// per-lane global addresses and writes them to 1 KB of consecutive LDS, lane l at `dst` + 16 l; no registers hold the
+// data, so a whole slab can be in flight behind the one being multiplied.  The LDS layout of a tile is therefore
+// unpadded; which 16-byte granule a lane fetches is free, so the granules of a row are permuted by an XOR of the row
+// index instead (SwzTile) -- rows that an access pattern reads together land in different banks.  The compiler does
+// not know that these instructions write LDS or count towards vmcnt: the callers wait with dma_wait<N>() (all but the N
+// youngest of this wave's loads have landed) and a workgroup barrier before reading.
+typedef __attribute__((address_space(3))) char lds_char_t;
+__device__ __forceinline__ unsigned lds_byte_addr(const void* p) { return (unsigned)(uintptr_t)(lds_char_t*)p; }
+__device__ __forceinline__ void dma16(const void* src, unsigned dst) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(dst)) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// A [ROWS][COLS] 2-byte tile in LDS without padding, COLS * 2 bytes per row, granule g (16 bytes) of row r at granule
+// position g ^ x(r):  256-byte rows x = 4 (r % 4), 128-byte rows x = 4 (r / 2 % 2), 64-byte rows x = r / 4 % 4.  With these
+// the four rows times 64 bytes that half a wave touches in a transposing read, and the sixteen rows times 16 bytes that
+// a 16-lane group touches in a row read of the 64-byte tiles, each cover all 256 bytes of bank space once.
+template <int ROWS, int COLS> struct SwzTile {
+  static constexpr int G = COLS / 8, BYTES = ROWS * COLS * 2, NINSTR = BYTES / 1024;
+  static_assert(G == 16 || G == 8 || G == 4, "rows of 256, 128 or 64 bytes");
+  static __device__ __forceinline__ int x(int r) { return G == 16 ? (r & 3) << 2 : G == 8 ? ((r >> 1) & 1) << 2 : (r >> 2) & 3; }
+  // element offset of (row r, column c)
+  static __device__ __forceinline__ int at(int r, int c) { return r * COLS + ((((c >> 3) ^ x(r)) << 3) | (c & 7)); }
+  // instruction j of the tile's DMA: the row and the column of the granule this lane fetches
+  static __device__ __forceinline__ void src(int j, int lane, int& r, int& c) {
+    const int p = 64 * j + lane;
+    r = p / G;
+    c = ((p % G) ^ x(r)) << 3;
+  }
+  // the four consecutive rows r0 .. r0 + 3 (r0 % 4 == 0) of column c0 + (this lane's column): one transposing read
+  static __device__ __forceinline__ typename Mma16Types::short4_ tr4(const T* tile, int r0, int c0, int lane) {
+    const int s = lane & 15;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((typename Mma16Types::lds_short4*)(tile + at(r0 + (s >> 2), c0 + 4 * (s & 3))));
+  }
+  // Mma::load_t on the swizzled tile: contraction index along the tile's rows k0 .. k0 + 15, columns c0 .. c0 + 31
+  static __device__ __forceinline__ M::Frag load_t(const T* tile, int k0, int c0, int lane) {
+    const int grp = lane >> 4;
+    const typename Mma16Types::short4_ lo = tr4(tile, k0 + 8 * (grp >> 1), c0 + 16 * (grp & 1), lane);
+    const typename Mma16Types::short4_ hi = tr4(tile, k0 + 8 * (grp >> 1) + 4, c0 + 16 * (grp & 1), lane);
+    const typename Mma16Types::short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(M::Frag, v);
+  }
+  // Mma::load on the swizzled tile: eight consecutive elements of row r from column c (c % 8 == 0)
+  static __device__ __forceinline__ M::Frag load(const T* tile, int r, int c) { return *reinterpret_cast<const M::Frag*>(tile + at(r, c)); }
+};
+
 template <int DK> struct BChunkL {
   static constexpr int SV = 32;
-  static constexpr int LDV = SV + 8;       // dO, V slabs [64][SV], read by rows
-  static constexpr int LDT = 64 + 32;      // D^T, dR^T slabs [SV][64], transposing reads only
-  static constexpr int LDKT = DK + 32;     // S^T, dS'^T slabs [SV][DK] and the K, Q tiles [64][DK], transposing reads
+  typedef SwzTile<64, SV> TokT;            // dO, V slabs [64][SV]
+  typedef SwzTile<SV, 64> TrT;             // D^T, dR^T slabs [SV][64]
+  typedef SwzTile<SV, DK> StT;             // S^T, dS'^T slabs [SV][DK]
+  static constexpr int LDKT = DK + 32;     // the epilogue's K, Q tiles [64][DK], transposing reads
   static constexpr int LDC = 64 + 8;       // dPe, dPe^T, dXa, dXe^T [64][64], read by rows
   static constexpr int LDK = DK + 8;       // staging tile for dq, dk [64][DK]
-  static constexpr int kTok = 64 * LDV, kT = SV * LDT, kSt = SV * LDKT, kC = 64 * LDC, kRow = 64 * LDKT;
-  static constexpr size_t loop_bytes = sizeof(T) * (2 * kTok + 2 * kT + 2 * kSt);
+  static constexpr int kC = 64 * LDC, kRow = 64 * LDKT;
+  // one slab of the loop: dO | V | D^T | dR^T | S^T | dS'^T, unpadded; two of them, filled by LDS-direct loads in turn
+  static constexpr int oV = TokT::BYTES, oDT = 2 * TokT::BYTES, odRT = oDT + TrT::BYTES, oSn = odRT + TrT::BYTES, odSn = oSn + StT::BYTES;
+  static constexpr int slab_bytes = odSn + StT::BYTES;
+  static constexpr size_t loop_bytes = 2 * slab_bytes;
   static constexpr size_t epi_bytes = sizeof(T) * (2 * kRow + 4 * kC);
   static_assert(64 * LDK <= 2 * kC, "the staging tile overlays dPe and dPe^T");
   static constexpr int nfloat = 64 * 8;
   static constexpr size_t bytes = sizeof(float) * nfloat + (epi_bytes > loop_bytes ? epi_bytes : loop_bytes);
+  static_assert(bytes <= 80 * 1024, "two workgroups per CU");
 };
 
 template <int DK, int GATE>
 __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   typedef BChunkL<DK> L;
-  constexpr int SV = L::SV, LDV = L::LDV, LDT = L::LDT, LDKT = L::LDKT, LDC = L::LDC, LDK = L::LDK;
+  constexpr int SV = L::SV, LDKT = L::LDKT, LDC = L::LDC, LDK = L::LDK;
+  typedef typename L::TokT TokT;
+  typedef typename L::TrT TrT;
+  typedef typename L::StT StT;
   constexpr int NKT = DK / 64;  // key-column tiles per wave
   extern __shared__ __align__(16) char smem[];
   float* sG = reinterpret_cast<float*>(smem);
@@ -880,13 +943,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   float* sNq = sMisc + 64;    // normalisation factors of the q and k rows (1 when the inputs come normalised)
   float* sNk = sNq + 64;
   T* tiles = reinterpret_cast<T*>(smem + sizeof(float) * L::nfloat);
-  // loop phase
-  T* sdO = tiles;
-  T* sV = sdO + L::kTok;
-  T* sDT = sV + L::kTok;
-  T* sdRT = sDT + L::kT;
-  T* sSn = sdRT + L::kT;
-  T* sdSn = sSn + L::kSt;
+  char* sSlab = reinterpret_cast<char*>(tiles);  // [2][slab_bytes]
   // epilogue
   T* sPe = tiles;             // [i][j]
   T* sPeT = sPe + L::kC;      // [j][i]
@@ -909,26 +966,7 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   const int wi = wave >> 1, wj = wave & 1;
   const int fr = lane & 31, kg8 = 8 * (lane >> 5);
 
-  TileRegs<T, 64, SV> rdO, rV;
-  TileRegs<T, SV, 64> rDT, rdRT;
-  TileRegs<T, SV, DK> rSn, rdSn;
-  TileRegs<T, 64, DK> rK, rQ;
-  // The loads of a slab in three parts (< 0: all): issued in one piece they held the wave for as long as the memory path
-  // took to admit them; a part before each half of the slab's products and one between them: 0.407 -> 0.390 ms.
-  auto fetch = [&](int v0, int part = -1) {
-    if (part < 0 || part == 0) {
-      rSn.load(at<const T>(p.ws, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
-      rdO.load(p.d_o + tbase * p.dv + v0, tsv, len, tid);
-    }
-    if (part < 0 || part == 1) {
-      rdSn.load(at<const T>(p.ws, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK, DK, SV, tid);
-      rV.load(p.v + tbase * p.dv + v0, tsv, len, tid);
-    }
-    if (part < 0 || part == 2) {
-      rDT.load(at<const T>(p.ws, p.off.D) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, SV, tid);
-      rdRT.load(at<const T>(p.ws, p.off.dD) + slot * p.dv * 64 + (int64_t)v0 * 64, 64, SV, tid);
-    }
-  };
+  TileRegs<T, 64, DK> rK, rQ;  // the epilogue's tiles, requested during the last slab
   floatx16 aP[1][1], aA[1][1], aQ[1][NKT], aK1[1][NKT], aK2[1][NKT];
   frag_zero(aP);
   frag_zero(aA);
@@ -936,7 +974,6 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
   frag_zero(aK1);
   frag_zero(aK2);
   float ss = 0.f, rdv = 0.f;
-  fetch(0);  // first, so that the small loads below do not hold it up
   if (tid < 64) {
     sG[tid] = (GATE == LNX_GATE_SCALAR) ? at<const float>(p.ws, p.off.G)[slot * 64 + tid] : 0.f;
     sBeta[tid] = (tid < len) ? p.beta[tbase + tid * ts] : 0.f;
@@ -945,56 +982,98 @@ __global__ __launch_bounds__(256, 2) void bwd_chunk_kernel(DirectParams p) {
     sNq[tid] = at<const float>(p.ws, p.off.Nq)[slot * 64 + tid];
     sNk[tid] = at<const float>(p.ws, p.off.Nk)[slot * 64 + tid];
   }
+  // ---- the slab loads: 32 one-KB instructions per slab, eight per wave, straight into LDS buffer `b` ----
+  // Token rows past the chunk's end fetch the chunk's last row instead of zeros: whatever they hold only reaches rows of
+  // dq, dk, dbeta, dg that are not stored (q, k and beta of those rows are zero).
+  const unsigned slab0 = lds_byte_addr(sSlab);
+  const T* gSn = at<const T>(p.ws, p.off.SnT) + slot * p.dv * DK;
+  const T* gdSn = at<const T>(p.ws, p.off.dSn) + slot * p.dv * DK;
+  const T* gDT = at<const T>(p.ws, p.off.D) + slot * p.dv * 64;
+  const T* gdRT = at<const T>(p.ws, p.off.dD) + slot * p.dv * 64;
+  const T* gdO = p.d_o + tbase * p.dv;
+  const T* gV = p.v + tbase * p.dv;
+  auto issue = [&](int v0, int b) {
+    const unsigned dst = slab0 + b * L::slab_bytes;
+    int r, c;
+    // wave w: instructions w, w + 4, ... of each tile
+#pragma unroll
+    for (int j = wave; j < StT::NINSTR; j += 4) {
+      StT::src(j, lane, r, c);
+      dma16(gSn + (int64_t)(v0 + r) * DK + c, dst + L::oSn + 1024 * j);
+      dma16(gdSn + (int64_t)(v0 + r) * DK + c, dst + L::odSn + 1024 * j);
+    }
+#pragma unroll
+    for (int j = wave; j < TokT::NINSTR; j += 4) {
+      TokT::src(j, lane, r, c);
+      r = min(r, len - 1);
+      dma16(gdO + (int64_t)r * tsv + v0 + c, dst + 1024 * j);
+      dma16(gV + (int64_t)r * tsv + v0 + c, dst + L::oV + 1024 * j);
+    }
+#pragma unroll
+    for (int j = wave; j < TrT::NINSTR; j += 4) {
+      TrT::src(j, lane, r, c);
+      dma16(gDT + (int64_t)(v0 + r) * 64 + c, dst + L::oDT + 1024 * j);
+      dma16(gdRT + (int64_t)(v0 + r) * 64 + c, dst + L::odRT + 1024 * j);
+    }
+  };
+  constexpr int PER_WAVE = (2 * StT::NINSTR + 2 * TokT::NINSTR + 2 * TrT::NINSTR) / 4;  // loads per wave and slab
+  static_assert(StT::NINSTR % 4 == 0 && TokT::NINSTR % 4 == 0 && TrT::NINSTR % 4 == 0, "the same count for every wave");
+  __builtin_amdgcn_s_waitcnt(0);  // the small loads above are behind us: from here on this wave's vmcnt counts slab loads only
+  issue(0, 0);
+  if (SV < p.dv) issue(SV, 1);
+  int b = 0;
 #pragma unroll 1
-  for (int v0 = 0; v0 < p.dv; v0 += SV) {
-    lds_barrier();  // the previous slab's tiles are dead
-    rdO.store(sdO, LDV, tid);
-    rV.store(sV, LDV, tid);
-    rDT.store(sDT, LDT, tid);
-    rdRT.store(sdRT, LDT, tid);
-    rSn.store(sSn, LDKT, tid);
-    rdSn.store(sdSn, LDKT, tid);
+  for (int v0 = 0; v0 < p.dv; v0 += SV, b ^= 1) {
+    // this slab has landed: all but the next slab's loads of this wave, then every wave's
+    if (v0 + SV < p.dv) dma_wait<PER_WAVE>();
+    else dma_wait<0>();
     lds_barrier();
-    static_assert(SV == 32, "two 16-wide steps per slab: one part of the next slab's loads before and after each");
-    if (v0 + SV < p.dv) fetch(v0 + SV, 0);
-    else {  // last slab: the epilogue's K and Q tiles instead
+    const T* sdO = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes);
+    const T* sV = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes + L::oV);
+    const T* sDT = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes + L::oDT);
+    const T* sdRT = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes + L::odRT);
+    const T* sSn = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes + L::oSn);
+    const T* sdSn = reinterpret_cast<const T*>(sSlab + b * L::slab_bytes + L::odSn);
+    static_assert(SV == 32, "two 16-wide steps per slab");
+    if (v0 + SV >= p.dv) {  // last slab: the epilogue's K and Q tiles (a slab earlier gains nothing)
       rK.load(p.k + tbase * DK, tsk, len, tid);
       rQ.load(p.q + tbase * DK, tsk, len, tid);
     }
 #pragma unroll
     for (int k0 = 0; k0 < SV; k0 += 16) {
-      const M::Frag fdO = M::load(sdO + (32 * wi + fr) * LDV + k0 + kg8);
-      const M::Frag fdR = M::load_t(sdRT, LDT, k0, 32 * wi, lane);
-      const M::Frag fDi = M::load_t(sDT, LDT, k0, 32 * wi, lane);
-      const M::Frag fDj = M::load_t(sDT, LDT, k0, 32 * wj, lane);
+      const M::Frag fdO = TokT::load(sdO, 32 * wi + fr, k0 + kg8);
+      const M::Frag fdR = TrT::load_t(sdRT, k0, 32 * wi, lane);
+      const M::Frag fDi = TrT::load_t(sDT, k0, 32 * wi, lane);
+      const M::Frag fDj = TrT::load_t(sDT, k0, 32 * wj, lane);
       M::mma(aP[0][0], fdO, fDj);
       M::mma(aA[0][0], fdR, fDj);
 #pragma unroll
       for (int c = 0; c < NKT; ++c) {
-        const M::Frag fS = M::load_t(sSn, LDKT, k0, 32 * (NKT * wj + c), lane);
-        const M::Frag fdS = M::load_t(sdSn, LDKT, k0, 32 * (NKT * wj + c), lane);
+        const M::Frag fS = StT::load_t(sSn, k0, 32 * (NKT * wj + c), lane);
+        const M::Frag fdS = StT::load_t(sdSn, k0, 32 * (NKT * wj + c), lane);
         M::mma(aQ[0][c], fdO, fS);
         M::mma(aK1[0][c], fdR, fS);
         M::mma(aK2[0][c], fDi, fdS);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      if (v0 + SV < p.dv) fetch(v0 + SV, k0 == 0 ? 1 : 2);
-      __builtin_amdgcn_sched_barrier(0);
     }
     {  // <dR_t, v_t> over this slab: thread = (token tid / 4, eight value columns)
       const int t = tid >> 2, c0 = 8 * (tid & 3);
-      const M::Frag vv = M::load(sV + t * LDV + c0);
+      const M::Frag vv = TokT::load(sV, t, c0);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) rdv += (float)vv[e] * (float)sdRT[(c0 + e) * LDT + t];
+      for (int e = 0; e < 8; ++e) rdv += (float)vv[e] * (float)sdRT[TrT::at(c0 + e, t)];
     }
-    if (GATE == LNX_GATE_SCALAR) {  // <dS', S> over this slab: thread = (value row tid / 8, DK / 8 key columns)
-      const int r = tid >> 3, c0 = (tid & 7) * (DK / 8);
+    if (GATE == LNX_GATE_SCALAR) {  // <dS', S> over this slab: the two tiles share one layout, so granule by granule
 #pragma unroll
-      for (int u = 0; u < DK / 8; u += 8) {
-        const M::Frag a = M::load(sSn + r * LDKT + c0 + u), b = M::load(sdSn + r * LDKT + c0 + u);
+      for (int u = 0; u < StT::BYTES / 16 / 256; ++u) {
+        const M::Frag a = *reinterpret_cast<const M::Frag*>(sSn + 8 * (tid + 256 * u));
+        const M::Frag b2 = *reinterpret_cast<const M::Frag*>(sdSn + 8 * (tid + 256 * u));
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ss += (float)a[e] * (float)b[e];
+        for (int e = 0; e < 8; ++e) ss += (float)a[e] * (float)b2[e];
       }
+    }
+    if (v0 + 2 * SV < p.dv) {  // this buffer takes the slab after the next, once every wave has read it
+      lds_barrier();
+      issue(v0 + 2 * SV, b);
     }
   }
   rdv += __shfl_xor(rdv, 1, LNX_WAVE);
