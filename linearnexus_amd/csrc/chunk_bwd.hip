@@ -37,6 +37,7 @@ struct BwdParams {
   const float* gA;
   const float* gbias;
   float gthr;
+  bool gband;  // softplus(threshold) != threshold in fp32: the activation's two branches overlap in the gate's values
   void* dgraw;
   float* gpart;       // [2][prows + LNX_SUM_SLICES][H * dk]: per-chunk partial sums of d_bias and of dg * g
   int64_t gprows;     // partial rows: chunk slots per head
@@ -934,6 +935,10 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK;
   const T* vg = reinterpret_cast<const T*>(p.v) + tbase * p.dv;
   const int wi = wave >> 1, wj = wave & 1;
+  // The head's gate scale -e^{A_log}, fetched here: a load issued behind the epilogue's stores would have to wait for
+  // every one of them to be acknowledged (the memory counter retires in order).
+  float gna = 0.f;
+  if constexpr (GRAW) gna = -__expf(p.gA[row % p.geom.H]);
   // V slabs first, K slabs last: without a per-channel gate the K slabs then stay in LDS for the epilogue
   const int nvs = p.dv / 64, nslab = NKS + nvs;
   constexpr bool KEEP_K = L::KEEP_K;
@@ -1160,8 +1165,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
         store4(sOut + r * LDF + c, dg0[it] + kk * (up[it] - um));  // dG of this half, in place of the column-type part
       }
       lds_barrier();
+      // From here to the end of the half every index is derived from a thread id that has passed through an empty asm:
+      // addresses formed outside the loop over the halves are spilled across its first part, and a reload behind the
+      // stores of dk waits until every one of them has been acknowledged (the memory counter retires in order).
+      int tl = tid;
+      asm volatile("" : "+v"(tl));
       {  // dg = reverse cumulative sum of dG over the chunk, per channel: 16-token segments in parallel, then their offsets
-        const int c = tid & 63, seg = tid >> 6;
+        const int c = tl & 63, seg = tl >> 6;
         float acc = 0.f;  // running sums written back in place: no array of sixteen values held across the barrier
 #pragma unroll 4
         for (int i = 15; i >= 0; --i) {
@@ -1180,56 +1190,59 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? (GATE == LNX_GATE_VECTOR || 
       // token, as in the pass above, makes four times as many memory instructions).  With the gate activated inside
       // the op, g = -e^{A_log} softplus(x), x = raw + bias (kda.py:153-165), the gradient goes on to the raw projection,
       // d_raw = dg (-e^{A_log}) softplus'(x), and the rows add to the channel's sums of d_raw (-> d_bias) and of dg g
-      // (-> d_A_log).  One exponential serves softplus and its derivative: softplus(x) = max(x, 0) + log(1 + e),
-      // sigmoid(x) = (x >= 0 ? 1 : e) / (1 + e), e = e^-|x|.
-      typedef typename Mma<T>::Quad Quad;  // four elements of T
-      Quad rq[4];
-      if constexpr (GRAW) {
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-          const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
-          rq[it] = *reinterpret_cast<const Quad*>(reinterpret_cast<const T*>(p.graw) + (tbase + (int64_t)min(r, len - 1) * ts) * DK + ch0 + c);
-        }
-      }
+      // (-> d_A_log).  Neither x nor a logarithm is needed for that: the activated gate is the difference of two rows of
+      // the cumulative gate in LDS, g_t = G_t - G_{t-1}, and with s = softplus(x) = g / -e^{A_log} the derivative is
+      // sigmoid(x) = 1 - e^{-s}; beyond the threshold s = x and the derivative is 1.  That needs s to tell the branch:
+      // true when softplus(threshold) rounds to the threshold (from about 15 on; the reference's default is 20).  A lower
+      // threshold leaves a band of s that both branches reach; then (gband) x is read again and decides.
       lds_barrier();
       if constexpr (!GRAW) {
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          const int idx = tid + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
+          const int idx = tl + 256 * it, r = idx >> 4, c = (idx & 15) * 4;
           if (r < len) store4(p.dg + (tbase + (int64_t)r * ts) * DK + ch0 + c, load4(sOut + r * LDF + c));
         }
       } else {
-        const int c = (tid & 15) * 4;
-        const float na = -__expf(p.gA[row % p.geom.H]);
-        floatx4 bias = {0.f, 0.f, 0.f, 0.f}, sb = bias, sa = bias;
-        if (p.gbias) bias = load4(p.gbias + (row % p.geom.H) * DK + ch0 + c);
+        const int c = (tl & 15) * 4;
+        const float na = gna, inv_na = 1.f / na;
+        floatx4 sb = {0.f, 0.f, 0.f, 0.f}, sa = sb;
+        typedef typename Mma<T>::Quad Quad;  // four elements of T
+        const int r0 = tl >> 4;
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          const int r = (tid >> 4) + 16 * it;
+          const int r = r0 + 16 * it;
           const floatx4 dgv = load4(sOut + r * LDF + c);
+          floatx4 gv = load4(sGc + r * LDF + c);
+          if (r > 0) gv = gv - load4(sGc + (r - 1) * LDF + c);
+          floatx4 xv = {0.f, 0.f, 0.f, 0.f};  // x = raw + bias, fetched where it is used: the unusual case may wait
+          if (p.gband) {
+            if (p.gbias) xv = load4(p.gbias + (row % p.geom.H) * DK + ch0 + c);
+            const Quad rq = *reinterpret_cast<const Quad*>(reinterpret_cast<const T*>(p.graw) + (tbase + (int64_t)min(r, len - 1) * ts) * DK + ch0 + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xv[e] += to_f32(rq[e]);
+          }
           floatx4 dr;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float x = to_f32(rq[it][e]) + bias[e];
-            const bool lin = x > p.gthr;
-            const float ex = __expf(-fabsf(x)), rc = __builtin_amdgcn_rcpf(1.f + ex);
-            const float sp = lin ? x : fmaxf(x, 0.f) + __logf(1.f + ex), ds = lin ? 1.f : (x >= 0.f ? rc : ex * rc);
+            const float sp = gv[e] * inv_na;
+            const bool lin = p.gband ? xv[e] > p.gthr : sp > p.gthr;
+            const float ds = lin ? 1.f : 1.f - __expf(-sp);
             dr[e] = r < len ? dgv[e] * na * ds : 0.f;
             sb[e] += dr[e];
-            sa[e] += r < len ? dgv[e] * na * sp : 0.f;
+            sa[e] += r < len ? dgv[e] * gv[e] : 0.f;
           }
           if (r < len) store4(reinterpret_cast<T*>(p.dgraw) + (tbase + (int64_t)r * ts) * DK + ch0 + c, dr);
         }
         float* sPart = reinterpret_cast<float*>(sKr);  // [2][16 row groups][64]: the K tile is dead, the segment totals read
-        store4(sPart + (tid >> 4) * 64 + c, sb);
-        store4(sPart + 1024 + (tid >> 4) * 64 + c, sa);
+        store4(sPart + r0 * 64 + c, sb);
+        store4(sPart + 1024 + r0 * 64 + c, sa);
         lds_barrier();
-        if (tid < 128) {  // the sixteen row groups in a fixed order
-          const float* src = sPart + (tid >> 6) * 1024 + (tid & 63);
+        if (tl < 128) {  // the sixteen row groups in a fixed order
+          const float* src = sPart + (tl >> 6) * 1024 + (tl & 63);
           float t = 0.f;
 #pragma unroll
           for (int q = 0; q < 16; ++q) t += src[64 * q];
-          gate_part(tid >> 6)[ch0 + (tid & 63)] = t;
+          gate_part(tl >> 6)[ch0 + (tl & 63)] = t;
         }
       }
     }
@@ -1418,6 +1431,7 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
   p.dv = a->dv; p.gate = a->gate; p.scale = a->scale; p.slab = a->test_scan_slab;
   const bool raw_gate = a->gate == LNX_GATE_VECTOR && a->gate_raw != nullptr;
   p.graw = raw_gate ? a->gate_raw : nullptr; p.gA = a->gate_A_log; p.gbias = a->gate_bias; p.gthr = a->gate_threshold;
+  p.gband = a->gate_threshold + log1pf(expf(-a->gate_threshold)) != a->gate_threshold;
   p.dgraw = a->d_gate_raw;
   p.gprows = (int64_t)(packed ? 1 : a->B) * lnx_chunk_slots(a);
   p.gpart = raw_gate ? reinterpret_cast<float*>(reinterpret_cast<char*>(a->workspace) + w.gpart) : nullptr;
