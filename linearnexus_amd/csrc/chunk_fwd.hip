@@ -470,21 +470,24 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
   TileRegs<T, 64, 64> rK, rQ;
   TileRegs<typename std::conditional<GRAW, T, float>::type, 64, 64> rG;
   const float gna = GRAW ? -__expf(p.gA[row % p.geom.H]) : 0.f;
+  typedef TileRegs<T, 64, 64> GT;
+  float gbias[GRAW ? GT::N : 1];  // the bias of this thread's channel group (256 % VPR == 0: the same group in every pass)
   auto fetch_half = [&](int h) {
     rK.load(kg + 64 * h, tsk, len, tid);
     rQ.load(qg + 64 * h, tsk, len, tid);
-    if constexpr (GRAW) rG.load(reinterpret_cast<const T*>(p.graw) + tbase * DK + 64 * h, tsk, len, tid);
-    else rG.load(p.g + tbase * DK + 64 * h, tsk, len, tid);
+    if constexpr (GRAW) {
+      rG.load(reinterpret_cast<const T*>(p.graw) + tbase * DK + 64 * h, tsk, len, tid);
+#pragma unroll
+      for (int e = 0; e < GT::N; ++e) gbias[e] = p.gbias ? p.gbias[(row % p.geom.H) * DK + 64 * h + (tid % GT::VPR) * GT::N + e] : 0.f;
+    } else {
+      rG.load(p.g + tbase * DK + 64 * h, tsk, len, tid);
+    }
   };
   // the raw gate tile -> activated fp32 gate in LDS; rows past the chunk's end stay zero (they read as raw zeros,
   // whose activation is not zero)
   auto store_gate = [&](int h) {
     if constexpr (GRAW) {
-      typedef TileRegs<T, 64, 64> GT;
-      const int c = (tid % GT::VPR) * GT::N;  // a thread keeps its channel group in every pass (256 % VPR == 0)
-      float bias[GT::N];
-#pragma unroll
-      for (int e = 0; e < GT::N; ++e) bias[e] = p.gbias ? p.gbias[(row % p.geom.H) * DK + 64 * h + c + e] : 0.f;
+      const int c = (tid % GT::VPR) * GT::N;
 #pragma unroll
       for (int it = 0; it < GT::IT; ++it) {
         const int r = (tid + 256 * it) / GT::VPR;
@@ -492,7 +495,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
         for (int e0 = 0; e0 < GT::N; e0 += 4) {
           floatx4 g4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) g4[e] = r < len ? gna * lnx_softplus_thr(to_f32(rG.x[it][e0 + e]) + bias[e0 + e], p.gthr) : 0.f;
+          for (int e = 0; e < 4; ++e) g4[e] = r < len ? gna * lnx_softplus_thr(to_f32(rG.x[it][e0 + e]) + gbias[e0 + e], p.gthr) : 0.f;
           store4(sG + r * LDF + c + e0, g4);
         }
       }
@@ -612,6 +615,13 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
     }
     }
   }
+  // From here on every index is derived from a thread id that has passed through an empty asm: what the phases below
+  // need would otherwise be formed at the kernel's start, spilled across phase A, and each reload would wait until all
+  // earlier stores have been acknowledged (the memory counter retires in order).
+  int tid_late = threadIdx.x;
+  asm volatile("" : "+v"(tid_late));
+  {
+  const int tid = tid_late, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, kq = lane >> 4;
   // ---- phase B: assemble X and <q, k>_E in sA / sT, write X and P, A = beta X, inverse ----
   if constexpr (LEVELS) {
     const int ti = 2 + (wave >> 1), tj = wave & 1, t16 = (wave < 2) ? 1 : 3;
@@ -736,6 +746,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 2 : 1)) void kda_prepare_ker
       unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.W) + slot * 64 * DK + 64 * s_, DK, sOut, LDC, 64, tid);
     else
       unstage_tile<T, 64, 64>(ws_ptr<T>(p, p.off.U) + slot * 64 * p.dv + 64 * (s_ - NH), p.dv, sOut, LDC, 64, tid);
+  }
   }
 }
 
