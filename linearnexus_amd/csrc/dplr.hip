@@ -25,12 +25,7 @@ __device__ __forceinline__ floatx4 rowgroup_sum(floatx4 x) {  // over the eight 
   for (int c = 0; c < 4; ++c)
     x[c] += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x[c]), 0x128, 0xF, 0xF, true));  // row_ror:8 = lane ^ 8
 #pragma unroll
-  for (int m = 16; m <= 32; m <<= 1) {
-    x[0] += __shfl_xor(x[0], m, LNX_WAVE);
-    x[1] += __shfl_xor(x[1], m, LNX_WAVE);
-    x[2] += __shfl_xor(x[2], m, LNX_WAVE);
-    x[3] += __shfl_xor(x[3], m, LNX_WAVE);
-  }
+  for (int c = 0; c < 4; ++c) x[c] = xor32_sum(xor16_sum(x[c]));
   return x;
 }
 
@@ -184,24 +179,37 @@ __global__ __launch_bounds__(64) void dplr_recurrent_kernel(DplrParams p) {
           *a = static_cast<const T*>(p.a) + tok0 * DK, *b = static_cast<const T*>(p.b) + tok0 * DK;
   const T* v = static_cast<const T*>(p.v) + tok0 * p.dv + ccol;
   const float* gk = p.gk + tok0 * DK;
-  // Token t + 1 is fetched (raw) while token t is applied; the barriers order LDS only (see TokenRegs).
-  TokenRegs<T, DK> cur, nxt;
-  Raw4<T> vc, vn;
-  if (p.T > 0) {
-    cur.fetch(q, k, a, b, gk, lane);
-    vc.load(v);
-  }
-  for (int t = 0; t < p.T; ++t) {
-    const int64_t r = (int64_t)min(t + 1, p.T - 1) * DK;
-    nxt.fetch(q + r, k + r, a + r, b + r, gk + r, lane);
-    vn.load(v + (int64_t)min(t + 1, p.T - 1) * p.dv);
+  // A token's compute time is a fraction of a memory round trip, so its vectors are requested four tokens before their
+  // use: four register sets in rotation, each refilled as soon as its token has been written to LDS.  The barriers order
+  // LDS only (see TokenRegs).
+  TokenRegs<T, DK> s0, s1, s2, s3;
+  Raw4<T> w0, w1, w2, w3;
+  auto fetch = [&](TokenRegs<T, DK>& s, Raw4<T>& w, int t) {
+    const int64_t tc = min(t, p.T - 1);
+    s.fetch(q + tc * DK, k + tc * DK, a + tc * DK, b + tc * DK, gk + tc * DK, lane);
+    w.load(v + tc * p.dv);
+  };
+  auto step = [&](TokenRegs<T, DK>& s, Raw4<T>& w, int t) {
+    if (t >= p.T) return;
     lds_barrier();  // the previous token's reads of sm are done
-    const floatx2 dots = cur.commit(sm, lane, p.scale);
+    const floatx2 dots = s.commit(sm, lane, p.scale);
+    const floatx4 v4 = w.f32();
     lds_barrier();
-    const floatx4 o4 = apply_token<DK>(S, sm, row0, vc.f32(), dots);
+    fetch(s, w, t + 4);
+    const floatx4 o4 = apply_token<DK>(S, sm, row0, v4, dots);
     if ((lane >> 3) == 0 && active) store_o4(p.o, (tok0 + t) * p.dv + col0, o4, p.o_dtype);
-    cur = nxt;
-    vc = vn;
+  };
+  if (p.T > 0) {
+    fetch(s0, w0, 0);
+    fetch(s1, w1, 1);
+    fetch(s2, w2, 2);
+    fetch(s3, w3, 3);
+  }
+  for (int t = 0; t < p.T; t += 4) {
+    step(s0, w0, t);
+    step(s1, w1, t + 1);
+    step(s2, w2, t + 2);
+    step(s3, w3, t + 3);
   }
   if (active) {
 #pragma unroll

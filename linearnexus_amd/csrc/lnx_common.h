@@ -82,12 +82,23 @@ __device__ __forceinline__ float quad_sum(float x) {
   return x;
 }
 
+// x + (x of lane ^ 16) and x + (x of lane ^ 32), in every lane, on the VALU: v_permlane16_swap exchanges the odd rows
+// (16 lanes) of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first
+// with the lower half of the second; fed the same value twice they return it with the even rows / lower half
+// repeated and with the odd rows / upper half repeated.  (A shuffle would go through the LDS crossbar.)
+__device__ __forceinline__ float xor16_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor32_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
   // inside a row of 16 lanes with DPP (no LDS crossbar): quads, the two quads of a half row, the two half rows
   x = quad_sum(x);
   x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x141, 0xF, 0xF, true));  // row_half_mirror: lane i <-> 7 - i
   x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x128, 0xF, 0xF, true));  // row_ror:8 = lane ^ 8
-  x += __shfl_xor(x, 16, LNX_WAVE);
-  x += __shfl_xor(x, 32, LNX_WAVE);
-  return x;
+  return xor32_sum(xor16_sum(x));
 }
