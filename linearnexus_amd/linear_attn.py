@@ -93,6 +93,8 @@ def _as_layout(x: Optional[Tensor], token_first: bool) -> Optional[Tensor]:
     """``x`` (logical [B, H, T, ...]) with dense memory in the chosen layout; no copy when it already has it."""
     if x is None:
         return None
+    if x.data_ptr() % 16:  # a dense view that starts inside a 16-byte vector of its storage: the kernels need a copy
+        x = x.clone(memory_format=torch.preserve_format)
     if token_first:
         return x if _is_token_first(x) else x.transpose(1, 2).contiguous().transpose(1, 2)
     return x.contiguous()

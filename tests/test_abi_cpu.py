@@ -20,6 +20,16 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(lnx_[a-z0-9_]+)\s*\(", text)))
 
 
+_dummies = []
+
+
+def _aligned_dummy():
+    """A 16-byte aligned host address for calls that are refused before anything is dereferenced."""
+    buf = (ctypes.c_char * 64)()
+    _dummies.append(buf)
+    return ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+
+
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_symbols()
@@ -60,8 +70,7 @@ def test_one_kernel_set_per_shape_and_no_environment_dispatch():
     a.gate = _lib.GATE_VECTOR
     assert int(lib.lnx_chunk_workspace_bytes(a)) > n_bf16 and lib.lnx_chunk_fuses_l2norm(a) == 0
     a.gate, a.test_scan_slab = _lib.GATE_SCALAR, 48
-    one = ctypes.c_float(0)
-    a.q = a.k = a.v = a.beta = a.o = a.final_state = a.g = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    a.q = a.k = a.v = a.beta = a.o = a.final_state = a.g = _aligned_dummy()
     assert lib.lnx_chunk_fwd(a, None) == -2 and b"test_scan_slab" in lib.lnx_last_error()
     csrc = os.path.join(ROOT, "linearnexus_amd", "csrc")
     for f in os.listdir(csrc):
@@ -82,8 +91,8 @@ def test_argument_validation_without_gpu():
         assert fn(a, None) == 0
     # value_cols (v holds only the leading value columns) is a forward-only feature, in whole 64-column slabs
     a.B, a.dv, a.value_cols = 1, 128, 64
-    one = ctypes.c_float(0)
-    p = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    p = _aligned_dummy()
+    base = p.value
     a.q = a.k = a.v = a.beta = a.o = a.final_state = p
     assert lib.lnx_chunk_fwd(a, None) == -2 and b"value_cols" in lib.lnx_last_error()      # forward_only not set
     a.forward_only, a.value_cols = 1, 32
@@ -92,6 +101,9 @@ def test_argument_validation_without_gpu():
     assert lib.lnx_chunk_fwd(a, None) == -2 and b"value_cols" in lib.lnx_last_error()      # more than dv
     a.value_cols, a.o = 64, None
     assert lib.lnx_chunk_fwd(a, None) == -4 and b"workspace" in lib.lnx_last_error()       # accepted up to the workspace
+    a.k = ctypes.c_void_p(base + 2)  # rows are moved as 16-byte vectors
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"16-byte aligned" in lib.lnx_last_error()
+    a.k = p
     assert lib.lnx_l2norm_fwd(None, None, 4, 8, 0, None) == -1
     d = _lib.DplrArgs()
     assert lib.lnx_dplr_step(d, None) == -2 and lib.lnx_dplr_recurrent_fwd(d, None) == -2
@@ -175,8 +187,7 @@ def test_malformed_cu_seqlens_is_refused_on_the_host():
 def test_static_scratch_entry_point_refuses_without_gpu():
     """lnx_chunk_fwd_static checks the shape against the library's scratch size before it touches the GPU."""
     lib = _lib.load()
-    one = ctypes.c_float(0)
-    p = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    p = _aligned_dummy()
     a = _lib.ScanArgs()
     a.B, a.H, a.T, a.dk, a.dv, a.chunk = 8, 16, 4096, 128, 128, 64
     a.dtype = a.o_dtype = _lib.LNX_BF16

@@ -366,3 +366,46 @@ def test_bf16_inputs_with_fp32_outputs_take_the_same_kernels(gate, slab, monkeyp
         assert torch.equal(a, b)
     o_ref, S_ref = oracle_fwd(xb, gate)
     assert max_rel(res[1][0].cpu().numpy(), o_ref) < 2e-2 and max_rel(res[1][1].cpu().numpy(), S_ref) < 2e-2
+
+
+def test_views_that_start_inside_a_16_byte_vector_are_copied_and_the_abi_refuses_them():
+    """The kernels move rows as 16-byte vectors.  The Python ops copy a dense view whose first element does not sit on
+    a 16-byte boundary of its storage (same values and gradients as from aligned tensors); the C-ABI refuses such a
+    pointer instead of launching."""
+    import linearnexus_amd as la
+    from linearnexus_amd import _lib
+    B, H, T, d = 1, 2, 130, 64
+    x = make_inputs(93, B, H, T, d, d, gate="scalar")
+    n = B * H * T * d
+
+    def leaves(offset):
+        out = []
+        for name in ("q", "k", "v"):
+            flat = torch.zeros(n + 8, dtype=torch.bfloat16, device=DEV)
+            flat[offset:offset + n] = torch.from_numpy(x[name]).to(DEV).to(torch.bfloat16).flatten()
+            out.append(flat[offset:offset + n].view(B, H, T, d).detach().requires_grad_(True))
+        return out
+
+    g, beta = torch.from_numpy(x["g"]).to(DEV), torch.from_numpy(x["beta"]).to(DEV)
+    res = []
+    for offset in (0, 1):  # 0 and 2 bytes into the storage
+        q, k, v = leaves(offset)
+        assert q.data_ptr() % 16 == 2 * offset
+        o, S = la.gated_delta_rule_chunkwise(q, k, v, g, beta, use_qk_l2norm=False)
+        grads = torch.autograd.grad([o, S], [q, k, v], [torch.ones_like(o), torch.ones_like(S)])
+        res.append([o, S, *grads])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    lib = _lib.load()
+    q, k, v = leaves(1)
+    a = _lib.ScanArgs()
+    a.B, a.H, a.T, a.dk, a.dv, a.chunk = B, H, T, d, d, 64
+    a.dtype = a.o_dtype = _lib.LNX_BF16
+    a.gate, a.scale, a.forward_only = _lib.GATE_SCALAR, d ** -0.5, 1
+    o = torch.empty(B, H, T, d, dtype=torch.bfloat16, device=DEV)
+    sT = torch.empty(B, H, d, d, dtype=torch.float32, device=DEV)
+    a.q, a.k, a.v, a.beta, a.g = q.data_ptr(), k.data_ptr(), v.data_ptr(), beta.data_ptr(), g.data_ptr()
+    a.o, a.final_state = o.data_ptr(), sT.data_ptr()
+    ws = torch.empty(int(lib.lnx_chunk_workspace_bytes(a)), dtype=torch.uint8, device=DEV)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    assert lib.lnx_chunk_fwd(a, None) == -2 and b"16-byte aligned" in lib.lnx_last_error()

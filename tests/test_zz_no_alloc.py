@@ -17,6 +17,13 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
+def _aligned_dummy():
+    """A 16-byte aligned host address for a call that is refused before anything is dereferenced."""
+    buf = (ctypes.c_char * 64)()
+    _aligned_dummy.keep = buf
+    return ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+
+
 def _args(x, B, H, T, dk, dv, cu=None):
     a = _lib.ScanArgs()
     a.B, a.H, a.T, a.dk, a.dv, a.chunk = B, H, T, dk, dv, 64
@@ -79,8 +86,7 @@ def test_static_scratch_forward_packed_batch():
 
 def test_static_scratch_forward_refuses_what_does_not_fit():
     lib = _lib.load()
-    one = ctypes.c_float(0)
-    p = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p)
+    p = _aligned_dummy()
     a = _lib.ScanArgs()
     a.B, a.H, a.T, a.dk, a.dv, a.chunk = 8, 16, 4096, 128, 128, 64
     a.dtype = a.o_dtype = _lib.LNX_BF16
