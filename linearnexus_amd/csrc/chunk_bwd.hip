@@ -585,8 +585,10 @@ __global__ __launch_bounds__(512) void bwd_scan_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
-// bwd_dqk: one workgroup per (chunk, 64-channel half of dk).  Loop over 64-column slabs of dv
-// with the next slab prefetched into registers; every product is one 32x32 tile per wave.
+// bwd_dqk: one workgroup per (chunk, 64-channel part of dk).  Loop over 32-column slabs of dv, every product one 32x32
+// tile per wave.  A slab's compute time is a fraction of a memory round trip, so with 2-byte inputs the slabs arrive
+// through loads that bypass the registers (mma_tiles.h) into NBUF unpadded LDS buffers, NBUF - 1 slabs ahead of the
+// one being multiplied; 4-byte inputs prefetch the next slab into registers.
 // ---------------------------------------------------------------------------------------
 template <typename T, int DK, int GATE> struct DqkCfg {
   static constexpr int PAD = Mma<T>::PAD;
@@ -595,7 +597,11 @@ template <typename T, int DK, int GATE> struct DqkCfg {
   // loop phase: dO, D, dD slabs [64][SV] and S_n, dS_n slabs [SV][64], five tiles of kLoop elements
   static constexpr int SV = 32, LDSV = SV + PAD;
   static constexpr int kLoop = (64 * LDSV > SV * LDC) ? 64 * LDSV : SV * LDC;
-  static constexpr size_t loop_bytes = sizeof(T) * 5 * kLoop;
+  // 2-byte inputs: NBUF buffers of dO | D | dD ([64][SV], read by rows) | S_n | dS_n ([SV][64], transposing reads)
+  static constexpr bool DMA = sizeof(T) == 2;
+  static constexpr int NBUF = GATE == LNX_GATE_VECTOR ? 3 : 2;  // what two / three workgroups per CU leave room for
+  static constexpr int slab_bytes = 5 * 64 * SV * 2;
+  static constexpr size_t loop_bytes = DMA ? (size_t)NBUF * slab_bytes : sizeof(T) * 5 * kLoop;
   // scalar epilogue: dPe, K rows, Q rows and one staging tile (dW, then dk), four [64][64] tiles
   static constexpr size_t scalar_bytes = sizeof(T) * 4 * kTile;
   // vector epilogue: alpha, out (fp32 [64][LDF]) and K, Q rows, plus dP in fp32
@@ -604,6 +610,7 @@ template <typename T, int DK, int GATE> struct DqkCfg {
   static constexpr size_t big = epi_bytes > loop_bytes ? epi_bytes : loop_bytes;
   static constexpr int kSmall = 64 * 4 + (GATE == LNX_GATE_VECTOR ? 64 * LNX_LDA : 0);  // floats
   static constexpr size_t bytes = sizeof(float) * kSmall + big;
+  static_assert(!DMA || bytes * (GATE == LNX_GATE_VECTOR ? 2 : 3) <= 160 * 1024, "workgroups per CU");
 };
 
 template <typename T, int DK, int GATE>
@@ -637,9 +644,100 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
   const T* kg = reinterpret_cast<const T*>(p.k) + tbase * DK + ch0;
   const int wi = wave >> 1, wj = wave & 1;
 
-  // dv is consumed in slabs of SV columns; narrow slabs keep the prefetch registers few enough
-  // for three waves per SIMD
+  // dv is consumed in slabs of SV columns
   constexpr int SV = L::SV, LDS_ = L::LDSV;
+  // per-channel gate: K, Q rows and the cumulative gate of this half for the epilogue, fetched during the last slab
+  TileRegs<T, 64, (GATE == LNX_GATE_VECTOR ? 64 : 8)> rk, rq;
+  TileRegs<float, 64, (GATE == LNX_GATE_VECTOR ? 64 : 4)> rGe;
+  auto fetch_epilogue = [&]() {
+    rk.load(kg, tsk, len, tid);
+    rq.load(qg, tsk, len, tid);
+    rGe.load(wsp<float>(p, p.off.G) + slot * 64 * DK + ch0, DK, 64, tid);
+  };
+  floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
+  frag_zero(aP);
+  frag_zero(aQ);
+  frag_zero(aW);
+  frag_zero(aK);
+  float ss = 0.f;
+  if constexpr (L::DMA) {
+    typedef Mma<bf16_t> M;
+    typedef SwzTile<64, SV> TokT;  // dO, D, dD slabs
+    typedef SwzTile<SV, 64> TrT;   // S_n, dS_n slabs of this part's channels
+    static_assert(TokT::NINSTR == 4 && TrT::NINSTR == 4, "one 1 KB load per wave and tile");
+    constexpr int PER_WAVE = 5, NBUF = L::NBUF;
+    char* sSlab = reinterpret_cast<char*>(sdO);
+    const unsigned slab0 = lds_byte_addr(sSlab);
+    const bf16_t* gdO = reinterpret_cast<const bf16_t*>(p.d_o) + tbase * p.dv;
+    const bf16_t* gD = wsp<bf16_t>(p, p.off.D) + slot * 64 * p.dv;
+    const bf16_t* gdD = wsp<bf16_t>(p, p.off.dD) + slot * 64 * p.dv;
+    const bf16_t* gSn = wsp<bf16_t>(p, p.off.SnT) + slot * p.dv * DK + ch0;
+    const bf16_t* gdSn = wsp<bf16_t>(p, p.off.dSn) + slot * p.dv * DK + ch0;
+    // Token rows of dO past the chunk's end fetch the chunk's last row instead of zeros: they only reach rows of dq and
+    // products with rows of q that are zero.
+    auto issue = [&](int v0, int b) {
+      const unsigned dst = slab0 + b * L::slab_bytes + 1024 * wave;
+      int r, c;
+      TokT::src(wave, lane, r, c);
+      dma16(gdO + (int64_t)min(r, len - 1) * tsv + v0 + c, dst);
+      dma16(gD + (int64_t)r * p.dv + v0 + c, dst + 4096);
+      dma16(gdD + (int64_t)r * p.dv + v0 + c, dst + 2 * 4096);
+      TrT::src(wave, lane, r, c);
+      dma16(gSn + (int64_t)(v0 + r) * DK + c, dst + 3 * 4096);
+      dma16(gdSn + (int64_t)(v0 + r) * DK + c, dst + 4 * 4096);
+    };
+    const int nslab = p.dv / SV;
+#pragma unroll
+    for (int b = 0; b < NBUF; ++b)
+      if (b < nslab) issue(b * SV, b);  // first, so that the small load below does not hold them up
+    if (tid < 64) {
+      sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
+      sSS[tid] = 0.f;
+      sMisc[tid] = 0.f;
+    }
+    const int fr = lane & 31, kg8 = 8 * (lane >> 5);
+    int b = 0;
+#pragma unroll 1
+    for (int s_ = 0; s_ < nslab; ++s_, b = (b + 1 == NBUF) ? 0 : b + 1) {
+      // this slab has landed: all but the loads of the slabs behind it that have been requested
+      const int behind = min(NBUF - 1, nslab - 1 - s_);
+      if (behind >= 2) dma_wait<2 * PER_WAVE>();
+      else if (behind == 1) dma_wait<PER_WAVE>();
+      else dma_wait<0>();
+      lds_barrier();
+      if (GATE == LNX_GATE_VECTOR && s_ + 1 == nslab) fetch_epilogue();
+      const bf16_t* tdO = reinterpret_cast<const bf16_t*>(sSlab + b * L::slab_bytes);
+      const bf16_t* tD = tdO + 2048;
+      const bf16_t* tdD = tD + 2048;
+      const bf16_t* tSn = tdD + 2048;
+      const bf16_t* tdSn = tSn + 2048;
+#pragma unroll
+      for (int k0 = 0; k0 < SV; k0 += 16) {
+        const M::Frag fdO = TokT::load(tdO, 32 * wi + fr, k0 + kg8);
+        const M::Frag fDi = TokT::load(tD, 32 * wi + fr, k0 + kg8);
+        const M::Frag fDj = TokT::load(tD, 32 * wj + fr, k0 + kg8);
+        const M::Frag fdD = TokT::load(tdD, 32 * wi + fr, k0 + kg8);
+        const M::Frag fS = TrT::load_t(tSn, k0, 32 * wj, lane);
+        const M::Frag fdS = TrT::load_t(tdSn, k0, 32 * wj, lane);
+        M::mma(aP[0][0], fdO, fDj);
+        M::mma(aQ[0][0], fdO, fS);
+        M::mma(aW[0][0], fdD, fS);
+        M::mma(aK[0][0], fDi, fdS);
+      }
+      if (GATE != LNX_GATE_NONE) {  // <dS_n, S_n> per channel: thread = (channel tid / 4, quarter of the slab's rows)
+        constexpr int QV = SV / 4;
+        const int r = tid >> 2, q4 = (tid & 3) * QV;
+        float t = 0.f;
+#pragma unroll
+        for (int e = 0; e < QV; ++e) t += to_f32(tSn[TrT::at(q4 + e, r)]) * to_f32(tdSn[TrT::at(q4 + e, r)]);
+        ss += t;
+      }
+      if (s_ + NBUF < nslab) {  // this buffer takes the slab NBUF ahead, once every wave has read it
+        lds_barrier();
+        issue((s_ + NBUF) * SV, b);
+      }
+    }
+  } else {
   TileRegs<T, 64, SV> rdO, rD, rdD;
   TileRegs<T, SV, 64> rSn, rdSn;  // S_n and dS_n slabs stay [v][c]: contracted along their rows
   auto fetch = [&](int v0) {
@@ -649,15 +747,6 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     rSn.load(wsp<T>(p, p.off.SnT) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
     rdSn.load(wsp<T>(p, p.off.dSn) + slot * p.dv * DK + (int64_t)v0 * DK + ch0, DK, SV, tid);
   };
-  // per-channel gate: K, Q rows and the cumulative gate of this half for the epilogue, fetched during the last slab
-  TileRegs<T, 64, (GATE == LNX_GATE_VECTOR ? 64 : 8)> rk, rq;
-  TileRegs<float, 64, (GATE == LNX_GATE_VECTOR ? 64 : 4)> rGe;
-  floatx16 aP[1][1], aQ[1][1], aW[1][1], aK[1][1];
-  frag_zero(aP);
-  frag_zero(aQ);
-  frag_zero(aW);
-  frag_zero(aK);
-  float ss = 0.f;
   fetch(0);  // first, so that the small load below does not hold it up
   if (tid < 64) {
     sG[tid] = (GATE == LNX_GATE_SCALAR) ? wsp<float>(p, p.off.G)[slot * 64 + tid] : 0.f;
@@ -673,11 +762,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
     rdSn.store(sdSn, LDC, tid);
     lds_barrier();
     if (v0 + SV < p.dv) fetch(v0 + SV);
-    else if (GATE == LNX_GATE_VECTOR) {  // last slab: the epilogue's K, Q and gate tiles instead
-      rk.load(kg, tsk, len, tid);
-      rq.load(qg, tsk, len, tid);
-      rGe.load(wsp<float>(p, p.off.G) + slot * 64 * DK + ch0, DK, 64, tid);
-    }
+    else if (GATE == LNX_GATE_VECTOR) fetch_epilogue();  // last slab: the epilogue's K, Q and gate tiles instead
     mma_nt<T, 1, 1>(aP, sdO + 32 * wi * LDS_, LDS_, sD + 32 * wj * LDS_, LDS_, SV, lane);
     mma_x<T, 1, 1, false, true>(aQ, sdO + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
     mma_x<T, 1, 1, false, true>(aW, sdD + 32 * wi * LDS_, LDS_, sSn + 32 * wj, LDC, SV, lane);
@@ -690,6 +775,7 @@ __global__ __launch_bounds__(256, (GATE == LNX_GATE_VECTOR ? (sizeof(T) == 2 ? 2
       for (int e = 0; e < QV; ++e) t += to_f32(sSn[(q4 + e) * LDC + r]) * to_f32(sdSn[(q4 + e) * LDC + r]);
       ss += t;
     }
+  }
   }
   if (GATE == LNX_GATE_VECTOR) {
     ss += __shfl_xor(ss, 1, LNX_WAVE);

@@ -34,12 +34,6 @@ namespace {
 
 using T = bf16_t;
 typedef Mma<T> M;
-struct Mma16Types {
-  typedef short short4_ __attribute__((ext_vector_type(4)));
-  typedef short short8_ __attribute__((ext_vector_type(8)));
-  typedef __attribute__((address_space(3))) short4_ lds_short4;
-};
-
 template <typename X> __device__ __forceinline__ X* at(char* ws, uint64_t off) { return reinterpret_cast<X*>(ws + off); }
 
 // dst[col][row0 + ...] = fragment (transposed store, four consecutive rows per 8-byte vector)
@@ -858,58 +852,11 @@ int launch_scan_bwd(const DirectParams& p, int nstate, hipStream_t st) {
 // is there, 6.2 us for the loop, 2.1 us staging K, Q and the four small tiles, 1.8 us for the epilogue's products and
 // 3.4 us until dq, dk have left -- memory latency at every step; the kernel moves 4.9 TB/s.
 // ---------------------------------------------------------------------------------------
-// ---- loads that go straight to LDS (global_load_lds_dwordx4): one wave instruction fetches 16 bytes per lane from
-// per-lane global addresses and writes them to 1 KB of consecutive LDS, lane l at `dst` + 16 l; no registers hold the
-// data, so a whole slab can be in flight behind the one being multiplied.  The LDS layout of a tile is therefore
-// unpadded; which 16-byte granule a lane fetches is free, so the granules of a row are permuted by an XOR of the row
-// index instead (SwzTile) -- rows that an access pattern reads together land in different banks.  The compiler does
-// not know that these instructions write LDS or count towards vmcnt: the callers wait with dma_wait<N>() (all but the N
-// youngest of this wave's loads have landed) and a workgroup barrier before reading.
-typedef __attribute__((address_space(3))) char lds_char_t;
-__device__ __forceinline__ unsigned lds_byte_addr(const void* p) { return (unsigned)(uintptr_t)(lds_char_t*)p; }
-__device__ __forceinline__ void dma16(const void* src, unsigned dst) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(dst)) : "memory", "m0");
-}
-template <int N> __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-
-// A [ROWS][COLS] 2-byte tile in LDS without padding, COLS * 2 bytes per row, granule g (16 bytes) of row r at granule
-// position g ^ x(r):  256-byte rows x = 4 (r % 4), 128-byte rows x = 4 (r / 2 % 2), 64-byte rows x = r / 4 % 4.  With these
-// the four rows times 64 bytes that half a wave touches in a transposing read, and the sixteen rows times 16 bytes that
-// a 16-lane group touches in a row read of the 64-byte tiles, each cover all 256 bytes of bank space once.
-template <int ROWS, int COLS> struct SwzTile {
-  static constexpr int G = COLS / 8, BYTES = ROWS * COLS * 2, NINSTR = BYTES / 1024;
-  static_assert(G == 16 || G == 8 || G == 4, "rows of 256, 128 or 64 bytes");
-  static __device__ __forceinline__ int x(int r) { return G == 16 ? (r & 3) << 2 : G == 8 ? ((r >> 1) & 1) << 2 : (r >> 2) & 3; }
-  // element offset of (row r, column c)
-  static __device__ __forceinline__ int at(int r, int c) { return r * COLS + ((((c >> 3) ^ x(r)) << 3) | (c & 7)); }
-  // instruction j of the tile's DMA: the row and the column of the granule this lane fetches
-  static __device__ __forceinline__ void src(int j, int lane, int& r, int& c) {
-    const int p = 64 * j + lane;
-    r = p / G;
-    c = ((p % G) ^ x(r)) << 3;
-  }
-  // the four consecutive rows r0 .. r0 + 3 (r0 % 4 == 0) of column c0 + (this lane's column): one transposing read
-  static __device__ __forceinline__ typename Mma16Types::short4_ tr4(const T* tile, int r0, int c0, int lane) {
-    const int s = lane & 15;
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((typename Mma16Types::lds_short4*)(tile + at(r0 + (s >> 2), c0 + 4 * (s & 3))));
-  }
-  // Mma::load_t on the swizzled tile: contraction index along the tile's rows k0 .. k0 + 15, columns c0 .. c0 + 31
-  static __device__ __forceinline__ M::Frag load_t(const T* tile, int k0, int c0, int lane) {
-    const int grp = lane >> 4;
-    const typename Mma16Types::short4_ lo = tr4(tile, k0 + 8 * (grp >> 1), c0 + 16 * (grp & 1), lane);
-    const typename Mma16Types::short4_ hi = tr4(tile, k0 + 8 * (grp >> 1) + 4, c0 + 16 * (grp & 1), lane);
-    const typename Mma16Types::short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(M::Frag, v);
-  }
-  // Mma::load on the swizzled tile: eight consecutive elements of row r from column c (c % 8 == 0)
-  static __device__ __forceinline__ M::Frag load(const T* tile, int r, int c) { return *reinterpret_cast<const M::Frag*>(tile + at(r, c)); }
-};
-
 template <int DK> struct BChunkL {
   static constexpr int SV = 32;
-  typedef SwzTile<64, SV> TokT;            // dO, V slabs [64][SV]
-  typedef SwzTile<SV, 64> TrT;             // D^T, dR^T slabs [SV][64]
-  typedef SwzTile<SV, DK> StT;             // S^T, dS'^T slabs [SV][DK]
+  typedef SwzTile<64, SV> TokT;            // dO, V slabs [64][SV], read by rows
+  typedef SwzTile<SV, 64, false> TrT;      // D^T, dR^T slabs [SV][64], transposing reads only
+  typedef SwzTile<SV, DK, false> StT;      // S^T, dS'^T slabs [SV][DK], transposing reads only
   static constexpr int LDKT = DK + 32;     // the epilogue's K, Q tiles [64][DK], transposing reads
   static constexpr int LDC = 64 + 8;       // dPe, dPe^T, dXa, dXe^T [64][64], read by rows
   static constexpr int LDK = DK + 8;       // staging tile for dq, dk [64][DK]

@@ -170,6 +170,69 @@ __device__ __forceinline__ void mma_x(floatx16 (&acc)[MT][NT], const T* A, int l
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Loads that go straight to LDS (global_load_lds_dwordx4): one wave instruction fetches 16 bytes per lane from per-lane
+// global addresses and writes them to 1 KB of consecutive LDS, lane l at `dst` + 16 l; no registers hold the data, so
+// whole slabs can be in flight behind the one being multiplied.  The LDS layout of a tile is therefore unpadded; which
+// 16-byte granule a lane fetches is free, so the granules of a row are permuted by an XOR of the row index instead
+// (SwzTile) -- rows that an access pattern reads together land in different banks.  The compiler does not know that
+// these instructions write LDS or count towards vmcnt: the callers wait with dma_wait<N>() (all but the N youngest of
+// this wave's memory instructions have completed; the counter retires in order) and a workgroup barrier before reading.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) char lds_char_t;
+__device__ __forceinline__ unsigned lds_byte_addr(const void* p) { return (unsigned)(uintptr_t)(lds_char_t*)p; }
+__device__ __forceinline__ void dma16(const void* src, unsigned dst) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(dst)) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// A [ROWS][COLS] bf16 tile in LDS without padding, COLS * 2 bytes per row, granule g (16 bytes) of row r at granule
+// position g ^ x(r).  x is chosen so that both ways of reading the tile touch every bank once per access:
+//   a row read (16 lanes = 16 consecutive rows, one granule each) needs 16 rows on 16 different 16-byte slots of the
+//   256 bytes of bank space, a transposing read (half a wave = 4 consecutive rows r0 % 4 == 0 times 4 aligned granules)
+//   needs the 4 rows on different 64-byte quarters:
+//   256-byte rows: x = 4 (r % 4) + r / 4 % 4;  128-byte rows: x = 4 (r / 2 % 2) + r / 4 % 4;  64-byte rows: x = r / 4 % 4.
+// Tiles of 256- or 128-byte rows that are only read through transposing reads (ROW_READS = false) drop the second
+// term: fewer address instructions.
+template <int ROWS, int COLS, bool ROW_READS = true> struct SwzTile {
+  typedef bf16_t T;
+  typedef Mma<bf16_t> M;
+  typedef short short4_ __attribute__((ext_vector_type(4)));
+  typedef short short8_ __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) short4_ lds_short4;
+  static constexpr int G = COLS / 8, BYTES = ROWS * COLS * 2, NINSTR = BYTES / 1024;
+  static_assert(G == 16 || G == 8 || G == 4, "rows of 256, 128 or 64 bytes");
+  static __device__ __forceinline__ int x(int r) {
+    const int lo = ROW_READS || G == 4 ? (r >> 2) & 3 : 0;
+    return G == 16 ? ((r & 3) << 2) | lo : G == 8 ? (((r >> 1) & 1) << 2) | lo : lo;
+  }
+  // element offset of (row r, column c)
+  static __device__ __forceinline__ int at(int r, int c) { return r * COLS + ((((c >> 3) ^ x(r)) << 3) | (c & 7)); }
+  // instruction j of the tile's load: the row and the column of the granule this lane fetches
+  static __device__ __forceinline__ void src(int j, int lane, int& r, int& c) {
+    const int p = 64 * j + lane;
+    r = p / G;
+    c = ((p % G) ^ x(r)) << 3;
+  }
+  // the four consecutive rows r0 .. r0 + 3 (r0 % 4 == 0) of column c0 + (this lane's column): one transposing read
+  static __device__ __forceinline__ short4_ tr4(const T* tile, int r0, int c0, int lane) {
+    const int s = lane & 15;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(tile + at(r0 + (s >> 2), c0 + 4 * (s & 3))));
+  }
+  // Mma::load_t on the swizzled tile: contraction index along the tile's rows k0 .. k0 + 15, columns c0 .. c0 + 31
+  static __device__ __forceinline__ typename M::Frag load_t(const T* tile, int k0, int c0, int lane) {
+    const int grp = lane >> 4;
+    const short4_ lo = tr4(tile, k0 + 8 * (grp >> 1), c0 + 16 * (grp & 1), lane);
+    const short4_ hi = tr4(tile, k0 + 8 * (grp >> 1) + 4, c0 + 16 * (grp & 1), lane);
+    const short8_ v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(typename M::Frag, v);
+  }
+  // Mma::load on the swizzled tile: eight consecutive elements of row r from column c (c % 8 == 0)
+  static __device__ __forceinline__ typename M::Frag load(const T* tile, int r, int c) {
+    return *reinterpret_cast<const typename M::Frag*>(tile + at(r, c));
+  }
+};
+
 __device__ __forceinline__ int frag_row(int e, int lane) { return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3); }
 __device__ __forceinline__ int frag_col(int lane) { return lane & 31; }
 
