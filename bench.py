@@ -305,7 +305,48 @@ def bench_chunk(args, torch, la, _lib, name):
     if tr:  # the same kernel against the HBM roof, from its measured traffic
         out["roofline_hbm_measured"] = {"kernel": dom, "achieved": tr / (avg[dom] * 1e-3) / 1e9, "peak": PEAK_HBM,
                                         "unit": "GB/s", "frac": tr / (avg[dom] * 1e-3) / 1e9 / PEAK_HBM}
+    # The whole step against the HBM roof: every input read once and every output written once (no intermediates),
+    # beside the traffic the kernels were measured to move (None when a kernel has no current entry).
+    es, n = (4 if fp32 else 2), B * H * T
+    eo = 4 if variant == "kda" else es  # kda_chunkwise returns fp32 (kda.py:655), so o and dO are fp32
+    gate_el = {"delta": 0, "gated": 1, "kda": d}[variant]
+    nstate = (nseq or B) * H * d * dv * 4
+    alg = n * (es * (2 * d + dv) + eo * dv + 4 * (1 + gate_el)) + nstate * (2 if s0 is not None else 1)
+    if backward:
+        alg += n * (es * (2 * d + dv) + eo * dv + es * (2 * d + dv) + 4 * 2 * (1 + gate_el)) + (nstate if s0 is not None else 0)
+    per = [measured_traffic(name, k_)[0] for k_ in avg]
+    moved = sum(per) if all(per) else None
+    out["step_hbm"] = {"algorithmic_bytes": alg, "algorithmic_GBps": alg / dtm / 1e9, "measured_bytes": moved,
+                       "measured_GBps": None if moved is None else moved / dtm / 1e9,
+                       "frac_of_peak_measured": None if moved is None else moved / dtm / 1e9 / PEAK_HBM, "peak": PEAK_HBM}
     return out, (B, H, T, d)
+
+
+def bench_hbm_streams(torch, steps):
+    """What plain streaming passes over 2 GiB sustain on this GPU: a read (sum), a write (fill) and a copy, as library
+    kernels.  The byte-bound kernels are judged against these as well as against the 8 TB/s of the data sheet: reads and
+    writes share the bus, and writes sustain markedly less than reads."""
+    n = (2 << 30) // 4
+    x = torch.ones(n, dtype=torch.float32, device="cuda:0")
+    y = torch.empty_like(x)
+    ops = {"read (sum)": (lambda: x.sum(), 4 * n), "write (fill_)": (lambda: y.fill_(1.0), 4 * n),
+           "copy (copy_)": (lambda: y.copy_(x), 8 * n)}
+    clock_warmup(torch, ops["copy (copy_)"][0], CLOCK_WARMUP_S)
+    res = {}
+    for name, (fn, nbytes) in ops.items():
+        for _ in range(5):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        res[name] = {"ms": round(ms, 4), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM, 3)}
+    return {"metric": "streaming passes over 2 GiB: GB/s", "value": res["read (sum)"]["GBps"], "unit": "GB/s", "n_gpus": 1,
+            "steps": steps, "warmup": 5, "ms_per_step": res["read (sum)"]["ms"], "higher_is_better": True, "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic", "config": {"workload": "hbm_streams", "bytes": 4 * n}, "streams": res}
 
 
 def bench_decode(args, torch, la, _lib, steps=None):
@@ -621,7 +662,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "dplr_train", "rmsnorm_gated", "kda_gate", "prefill_long"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=list(CHUNK_CONFIGS) + ["decode", "decode_graph", "conv", "dplr_decode", "dplr_train", "rmsnorm_gated", "kda_gate", "prefill_long", "hbm_streams"])
     ap.add_argument("--clock-warmup-seconds", type=float, default=2.0,
                     help="untimed run of the workload before the W warm-up steps, so that the timed steps see the GPU's "
                          "clocks at their loaded level and not on the way up from idle (0: none; counter runs use that)")
@@ -647,6 +688,9 @@ def main():
         print("bench.py needs an MI355X (no GPU visible)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "hbm_streams":
+        print(json.dumps(bench_hbm_streams(torch, args.steps)))
+        return
     if args.workload == "kda_gate":
         print(json.dumps(bench_kda_gate(torch, la, _lib, args.steps, args.warmup)))
         return
