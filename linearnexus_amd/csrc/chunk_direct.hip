@@ -21,10 +21,11 @@
 //   bwd_chunk  (one workgroup per chunk, all in parallel)                         dq, dk, dbeta, dg from q, k, v, dO, the
 //              two saved states and D, dR as the scans left them (dv leaves the reverse scan)
 //
-// Both scans split their 512 threads into four compute waves (matrix work on the tiles in LDS, the fp32 state in MFMA
-// accumulators for the whole sequence) and four mover waves (global loads two chunks ahead into registers, tile
-// writes into LDS as soon as a tile's last reader is past, LDS -> global copies of results as whole rows); K, Pm and
-// the per-token scalars are double-buffered in LDS so that three LDS-only barriers per chunk suffice.
+// Both scans split their waves into one compute wave per 32 value columns of the slab (two for the 64-column slabs:
+// matrix work on the tiles in LDS, the fp32 state in MFMA accumulators for the whole sequence) and four mover waves
+// (global loads two chunks ahead into registers, the next chunk's tiles into LDS, LDS -> global copies of results as
+// whole rows); all five input tiles and the per-token scalars are double-buffered in LDS, so two LDS-only barriers per
+// chunk suffice.  bwd_chunk brings its slabs in with loads that go straight to LDS (mma_tiles.h).
 
 #include <type_traits>
 

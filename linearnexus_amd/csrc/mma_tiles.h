@@ -351,7 +351,6 @@ template <typename T> struct TriRegs {
     o1 = r * ld + 8 * c;
   }
   __device__ __forceinline__ void load(const T* src, int tid) {
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, LNX_TRI_VECS * 16, 0x00020000);
     x[0] = __builtin_bit_cast(typename Vec16<T>::V, __builtin_amdgcn_raw_buffer_load_b128(rsrc, 16 * tid, 0, 0));
     // threads without a second vector read past the end: the range check returns zeros, nothing sits behind a branch
