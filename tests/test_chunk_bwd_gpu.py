@@ -76,6 +76,17 @@ def test_chunk_backward_matches_adjoint_oracle(gate, bf16, shape):
 
 
 @pytest.mark.parametrize("gate", GATES)
+@pytest.mark.parametrize("dk,dv", [(128, 192), (64, 320), (128, 64)])
+def test_chunk_backward_slab_buffer_rotation(gate, dk, dv):
+    """bf16 inputs: the chunk-local backward kernels take the value dimension in 32-column slabs that arrive through
+    loads straight to LDS into two or three buffers in rotation; 2, 6 and 10 slabs leave the rotation at every buffer."""
+    x = make_inputs(57, 1, 2, 150, dk, dv, gate=gate, with_state=True, with_grad=True)
+    x, dt = _prep(x, True)
+    ref = delta_rule_adjoint(x["q"], x["k"], x["v"], x["beta"], x["dO"], x.get("g"), x["dS"], None, x["S0"], False)
+    check(gpu_grads(x, gate, dt), ref, 2e-2)
+
+
+@pytest.mark.parametrize("gate", GATES)
 def test_backward_without_state_gradients(gate):
     """Zero initial state, no gradient flowing into the final state."""
     x = make_inputs(52, 1, 2, 192, 128, 128, gate=gate, with_grad=True)
