@@ -465,6 +465,9 @@ class _ChunkScan(torch.autograd.Function):
         ctx.save_for_backward(*saved)
         ctx.meta = meta
         ctx.raw_gate = None if A_log is None else (float(threshold), A_log.dtype, None if g_bias is None else g_bias.dtype)
+        # an output that takes no part in the loss arrives in backward() as None, not as a tensor of zeros that a fill
+        # kernel wrote and lnx_chunk_bwd would read: a null d_final_state is the kernels' "no gradient"
+        ctx.set_materialize_grads(False)
         return o, sT
 
     @staticmethod
