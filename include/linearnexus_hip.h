@@ -145,7 +145,7 @@ int lnx_recurrent_fwd(const lnx_scan_args* a, void* hip_stream);
  * Shapes: dk in {64, 128, 256} (256 is the head_dim of the reference's Gated DeltaNet presets,
  * models.py:142-143), dv a multiple of 64.  q, k, v, o, a per-channel gate (g or gate_raw), the states, the workspace
  * and the gradients of all of these must be 16-byte aligned (the kernels move their rows as 16-byte vectors);
- * LNX_ERR_SHAPE otherwise.  beta, a scalar gate and their gradients only need their element's alignment.
+ * LNX_ERR_SHAPE otherwise (LNX_ERR_WORKSPACE for the workspace).  beta, a scalar gate and their gradients only need their element's alignment.
  */
 uint64_t lnx_chunk_workspace_bytes(const lnx_scan_args* a);
 int lnx_chunk_fwd(const lnx_scan_args* a, void* hip_stream);

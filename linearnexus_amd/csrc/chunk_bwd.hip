@@ -1503,6 +1503,7 @@ extern "C" int lnx_chunk_bwd(const lnx_scan_args* a, void* stream) {
     return LNX_OK;
   }
   const ChunkWs w = lnx_chunk_ws_layout(a);
+  if (reinterpret_cast<uintptr_t>(a->workspace) & 15) return lnx_set_error(LNX_ERR_WORKSPACE, "the workspace must be 16-byte aligned");
   if (!a->workspace || a->workspace_bytes < w.total)
     return lnx_set_error(LNX_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)w.total,
                          (unsigned long long)a->workspace_bytes);

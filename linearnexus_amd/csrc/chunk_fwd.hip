@@ -1459,9 +1459,10 @@ int lnx_chunk_check(const lnx_scan_args* a, bool backward) {
   if (backward && a->forward_only) return lnx_set_error(LNX_ERR_SHAPE, "forward_only is set: the workspace holds nothing for a backward pass");
   if (a->cu_seqlens && (a->B != 1 || a->nseq <= 0))
     return lnx_set_error(LNX_ERR_SHAPE, "packed batches need B == 1 and nseq > 0 (B=%d nseq=%d)", a->B, a->nseq);
-  // the kernels move rows of these tensors as 16-byte vectors (beta, the scalar gate and their gradients go by elements)
+  // the kernels move rows of these tensors as 16-byte vectors (beta, the scalar gate and their gradients go by elements;
+  // the workspace is checked where it is used: lnx_chunk_fwd_static ignores the field)
   const void* vec16[] = {a->q, a->k, a->v, a->o, a->initial_state, a->final_state, a->gate == LNX_GATE_VECTOR ? a->g : nullptr,
-                         a->gate_raw, a->workspace, a->d_o, a->d_final_state, a->d_q, a->d_k, a->d_v,
+                         a->gate_raw, a->d_o, a->d_final_state, a->d_q, a->d_k, a->d_v,
                          a->gate == LNX_GATE_VECTOR ? a->d_g : nullptr, a->d_gate_raw, a->d_initial_state};
   for (const void* ptr : vec16)
     if (reinterpret_cast<uintptr_t>(ptr) & 15)
@@ -1515,6 +1516,7 @@ int chunk_fwd_on(const lnx_scan_args* a, void* workspace, uint64_t workspace_byt
     return LNX_OK;
   }
   const ChunkWs w = lnx_chunk_ws_layout(a);
+  if (reinterpret_cast<uintptr_t>(workspace) & 15) return lnx_set_error(LNX_ERR_WORKSPACE, "the workspace must be 16-byte aligned");
   if (!workspace || workspace_bytes < w.total)
     return lnx_set_error(LNX_ERR_WORKSPACE, "workspace of %llu bytes needed, %llu given", (unsigned long long)w.total,
                          (unsigned long long)workspace_bytes);

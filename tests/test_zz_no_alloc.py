@@ -55,7 +55,7 @@ def _run_both(seed, B, H, T, d, cu_list=None):
         a = _args(x, B, H, T, d, d, cu)
         a.o, a.final_state = o.data_ptr(), sT.data_ptr()
         if static:
-            a.workspace, a.workspace_bytes = None, 0  # ignored
+            a.workspace, a.workspace_bytes = 3, 0  # ignored, whatever they hold
             _lib.check(lib.lnx_chunk_fwd_static(a, stream), "lnx_chunk_fwd_static")
         else:
             n = int(lib.lnx_chunk_workspace_bytes(a))
